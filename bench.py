@@ -1,0 +1,270 @@
+#!/usr/bin/env python3
+"""Benchmark of the conv-as-GEMM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg1|cfg3|cfg4|cfg5]
+
+A "step" is one pass of the hot path over one batch of synthetic input that is already resident in
+HBM.  The default workload is the VGG16-style 3x3 layer (N=64, 256 -> 256 channels, 56x56, fp32,
+NCHW): forward + filter gradient + bias gradient + input gradient through the implicit-GEMM
+kernels.  One JSON line is printed: whole-step GFLOP/s as ``value``, the forward kernel's measured
+fraction of the fp32 MFMA peak under ``roofline`` (HIP events around that kernel inside the timed
+region), and the CPU restatement of the reference's path (Cython-style im2col in C/OpenMP + NumPy
+``@``), timed on the host cores on a bounded sample, under ``cpu_baseline``.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+METRIC = "conv GFLOP/s & % fp32 MFMA peak (3x3 VGG layer); VGG16 train img/s, 1 GPU"
+FP32_MFMA_PEAK_TFLOPS = 157.3   # 256 CU x 2.4 GHz x 256 FLOP/clk/CU
+HBM_PEAK_GBS = 8000.0
+
+# HBM bytes per launch of the forward kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# (see profiles/); None until measured for the workload.
+MEASURED_TRAFFIC_BYTES = {"cfg2": None}
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-vgg16", action="store_true", help="skip the VGG16 training-step extra of the default run")
+    return ap.parse_args()
+
+
+# --------------------------------------------------------------------------- synthetic inputs (seed 0)
+
+def he_normal(rng, shape, fan_in):
+    import numpy as np
+    return (rng.standard_normal(shape) * np.sqrt(2.0 / fan_in)).astype(np.float32)
+
+
+def make_cfg2(n=64):
+    import numpy as np
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((n, 256, 56, 56), dtype=np.float32)
+    w = he_normal(rng, (256, 256, 3, 3), 2304)
+    b = np.zeros(256, np.float32)
+    dy = rng.standard_normal((n, 256, 56, 56), dtype=np.float32)
+    return x, w, b, dy
+
+
+class Timer:
+    """HIP events on torch's current stream, which is the stream every kernel here is launched on."""
+
+    def __init__(self, torch):
+        self.torch = torch
+        self.pairs = []
+
+    def __call__(self, fn, *a, **kw):
+        s, e = self.torch.cuda.Event(enable_timing=True), self.torch.cuda.Event(enable_timing=True)
+        s.record()
+        out = fn(*a, **kw)
+        e.record()
+        self.pairs.append((s, e))
+        return out
+
+    def mean_ms(self):
+        return sum(s.elapsed_time(e) for s, e in self.pairs) / max(1, len(self.pairs))
+
+
+def timed_steps(torch, step, steps, warmup):
+    for _ in range(warmup):
+        step(None)
+    torch.cuda.synchronize()
+    timers = {}
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step(timers)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps, timers
+
+
+# --------------------------------------------------------------------------- workloads
+
+def run_cfg2(torch, pd, args):
+    import numpy as np
+    x, w, b, dy = make_cfg2()
+    n = x.shape[0]
+    model = pd.Model(tensor_format="NCHW", batch_size=n)
+    model.mode = pd.TRAIN_MODE
+    conv = pd.Conv2D(nfilters=256, filter_shape=(3, 3), padding=1)
+    conv.set_model(model)
+    conv.initialize(prev_shape=(256, 56, 56))
+    conv.weights, conv.biases = torch.from_numpy(w).cuda(), torch.from_numpy(b).cuda()
+    xd, dyd = torch.from_numpy(x).cuda(), torch.from_numpy(dy).cuda()
+    from pydtnn_amd import ops
+
+    def step(timers):
+        if timers is None:
+            conv.forward(xd)
+            conv.backward(dyd)
+            return
+        for name in ("fwd", "dw", "db", "dx"):
+            timers.setdefault(name, Timer(torch))
+        kw = conv._cg_kwargs()
+        conv.cg_x = xd
+        timers["fwd"](conv.cg.conv_gemm_nchw, conv.weights, xd, biases=None, biases_vector=conv.biases, **kw)
+        dw = torch.empty_like(conv.weights)
+        timers["dw"](conv.cg.conv_gemm_nchw, dyd, xd, biases=dw, trans=True, **kw)
+        timers["db"](ops.bias_grad, dyd, 256, 56 * 56)
+        dx = torch.empty_like(xd)
+        timers["dx"](conv.cg.deconv_gemm_nchw, conv.weights, dyd, dx, **kw)
+
+    ms, timers = timed_steps(torch, step, args.steps, args.warmup)
+    gemm_flop = 2.0 * 256 * 2304 * n * 56 * 56
+    step_flop = 3 * gemm_flop
+    fwd_ms = timers["fwd"].mean_ms()
+    achieved = gemm_flop / (fwd_ms * 1e-3) / 1e12
+    kernels = {k: round(t.mean_ms(), 4) for k, t in timers.items()}
+    extra = {
+        "kernel_ms": kernels,
+        "fwd_tflops": round(achieved, 2),
+        "dw_tflops": round(gemm_flop / (kernels["dw"] * 1e-3) / 1e12, 2),
+        "dx_tflops": round(gemm_flop / (kernels["dx"] * 1e-3) / 1e12, 2),
+        "fwd_pct_fp32_mfma_peak": round(100 * achieved / FP32_MFMA_PEAK_TFLOPS, 2),
+        "step_gflop": round(step_flop / 1e9, 2),
+    }
+    # explicit-path streams: bytes(x) + bytes(cols) and bytes(cols) + bytes(dx)
+    cols_t, c2i_t = Timer(torch), Timer(torch)
+    geom = (3, 3, 1, 1, 1, 1, 1, 1)
+    for i in range(4):
+        cols = ops.im2col_nchw(xd, *geom) if i == 0 else cols_t(ops.im2col_nchw, xd, *geom)
+        back = ops.col2im_nchw(cols, n, 256, 56, 56, *geom) if i == 0 else c2i_t(ops.col2im_nchw, cols, n, 256, 56,
+                                                                                56, *geom)
+        del back
+        if i < 3:
+            del cols
+    torch.cuda.synchronize()
+    stream_bytes = x.nbytes + cols.numel() * 4
+    extra["im2col_gbs"] = round(stream_bytes / (cols_t.mean_ms() * 1e-3) / 1e9, 1)
+    extra["col2im_gbs"] = round(stream_bytes / (c2i_t.mean_ms() * 1e-3) / 1e9, 1)
+    extra["im2col_pct_hbm_peak"] = round(100 * extra["im2col_gbs"] / HBM_PEAK_GBS, 1)
+    extra["col2im_pct_hbm_peak"] = round(100 * extra["col2im_gbs"] / HBM_PEAK_GBS, 1)
+    del cols
+    roofline = {"bound": "mfma", "kernel": "gemm_kernel<128x128, PlainK, Im2colNchwMN, EpiNchw> (forward)",
+                "achieved": round(achieved, 3), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES["cfg2"]}
+    workload = ("cfg2: VGG16-style 3x3 conv layer fwd+dW+db+dX, fp32 NCHW, N=64, 256->256, 56x56, stride 1, pad 1, "
+                "implicit GEMM")
+    return ms, step_flop / (ms * 1e-3) / 1e9, workload, roofline, extra
+
+
+def cpu_baseline_cfg2(sample_images=16):
+    """The reference's CPU route (im2col -> NumPy @ -> bias add -> 1023 transpose; backward likewise) restated
+    by the oracle, timed on this host on `sample_images` of the 64 images."""
+    import numpy as np
+    from oracle import cpu_ref
+    x, w, b, dy = make_cfg2(sample_images)
+    p = cpu_ref.ConvParams(3, 3, 1, 1)
+    best = None
+    for it in range(3):
+        t0 = time.perf_counter()
+        y, x_cols = cpu_ref.conv2d_forward_nchw_i2c(x, w, b, p)
+        cpu_ref.conv2d_backward_nchw_i2c(dy, x_cols, w, x.shape, p)
+        dt = time.perf_counter() - t0
+        if it > 0:
+            best = dt if best is None else min(best, dt)
+    flop = 3 * 2.0 * 256 * 2304 * sample_images * 56 * 56
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    return {"value": round(flop / best / 1e9, 1), "unit": "GFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"{sample_images} of 64 images of cfg2, fwd+dW+db+dX, 1 warm-up then best of 2 "
+                      f"({best:.2f} s); C/OpenMP im2col+col2im, NumPy(OpenBLAS) matmul"}
+
+
+def build_vgg16(pd, n=64):
+    model = pd.Model(tensor_format="NCHW", batch_size=n)
+    model.add(pd.Input(shape=(224, 224, 3)))
+    for nlayers, nfilters in [[2, 64], [2, 128], [3, 256], [3, 512], [3, 512]]:
+        for _ in range(nlayers):
+            model.add(pd.Conv2D(nfilters=nfilters, filter_shape=(3, 3), padding=1, stride=1, activation="relu",
+                                weights_initializer="he_normal"))
+        model.add(pd.MaxPool2D(pool_shape=(2, 2), stride=2))
+    model.add(pd.Flatten())
+    # pydtnn/models/vgg16.py:34-38 without the two Dropout(0.5) layers (the configuration has none)
+    model.add(pd.FC(shape=(4096,), activation="relu", weights_initializer="he_normal"))
+    model.add(pd.FC(shape=(4096,), activation="relu", weights_initializer="he_normal"))
+    model.add(pd.FC(shape=(1000,), activation="softmax", weights_initializer="he_normal"))
+    return model
+
+
+def run_cfg5(torch, pd, args, steps=None, warmup=None):
+    import numpy as np
+    np.random.seed(0)
+    n = 64
+    model = build_vgg16(pd, n)
+    rng = np.random.default_rng(0)
+    x = torch.from_numpy(rng.random((n, 3, 224, 224), dtype=np.float32)).cuda()
+    labels = rng.integers(0, 1000, n)
+    y_targ = torch.zeros((n, 1000), device="cuda")
+    y_targ[torch.arange(n), torch.from_numpy(labels).cuda()] = 1.0
+    loss_fn, opt = pd.CategoricalCrossEntropy(), pd.SGD(learning_rate=0.01, momentum=0.9)
+    losses = []
+
+    def step(timers):
+        losses.append(model.train_batch(x, y_targ, loss_fn, opt))
+
+    ms, _ = timed_steps(torch, step, steps or args.steps, warmup if warmup is not None else args.warmup)
+    flop = 5929.5e9
+    extra = {"vgg16_train_img_per_s": round(n / (ms * 1e-3), 1), "vgg16_ms_per_step": round(ms, 2),
+             "vgg16_tflops": round(flop / (ms * 1e-3) / 1e12, 2),
+             "vgg16_pct_fp32_mfma_peak": round(100 * flop / (ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS, 2),
+             "vgg16_first_last_loss": [round(float(losses[0]), 4), round(float(losses[-1]), 4)],
+             "vgg16_params": int(model.nparams)}
+    return ms, extra
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on one GPU; --gpus {args.gpus} is not supported "
+              f"(no collectives or sharding are part of it).", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    import pydtnn_amd as pd
+    from pydtnn_amd import native
+    native.lib()
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the kernels have no CPU fallback.", file=sys.stderr)
+        sys.exit(2)
+    torch.cuda.set_device(0)
+
+    if args.workload == "cfg2":
+        ms, value, workload, roofline, extra = run_cfg2(torch, pd, args)
+        unit = "GFLOP/s"
+        if not args.no_vgg16:
+            _, vgg = run_cfg5(torch, pd, args, steps=3, warmup=1)
+            extra.update(vgg)
+    elif args.workload == "cfg5":
+        ms, extra = run_cfg5(torch, pd, args)
+        value, unit = 5929.5e9 / (ms * 1e-3) / 1e9, "GFLOP/s"
+        workload = "cfg5: full VGG16 training step, fp32 NCHW, batch 64, 3x224x224, SGD momentum"
+        roofline = {"bound": "mfma", "kernel": "whole step", "achieved": round(value / 1e3, 3),
+                    "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(value / 1e3 / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": None}
+    else:
+        from bench_configs import run_other
+        ms, value, unit, workload, roofline, extra = run_other(torch, pd, args, Timer, timed_steps)
+
+    cpu = None
+    if not args.no_cpu_baseline and args.workload == "cfg2":
+        cpu = cpu_baseline_cfg2()
+
+    print(json.dumps({
+        "metric": METRIC, "value": round(value, 1), "unit": unit, "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": workload}, "roofline": roofline, "cpu_baseline": cpu, "extra": extra}))
+
+
+if __name__ == "__main__":
+    main()

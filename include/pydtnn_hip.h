@@ -1,0 +1,221 @@
+/*
+ * C ABI of libpydtnn_hip.so: the MI355X (gfx950) implementation of PyDTNN's conv-as-GEMM path.
+ *
+ * Two flavours are exported.
+ *
+ *  (1) Device-pointer entry points, prefixed pydtnn_hip_.  Every pointer is a device address
+ *      (for instance torch.Tensor.data_ptr()), `stream` is a hipStream_t passed as void*
+ *      (NULL = the default stream), work is enqueued asynchronously and the return value is a
+ *      PYDTNN_HIP_* status.  Tensors are dense, C-contiguous fp32.  Entry points that need
+ *      scratch memory take `workspace` / `workspace_bytes`; the matching *_workspace_bytes
+ *      query says how much.  Nothing here allocates or frees device memory.
+ *
+ *  (2) Host-pointer entry points with exactly the names and argument lists of the external
+ *      libconvGemm that PyDTNN binds with ctypes (pydtnn/backends/cpu/libs/conv_gemm.py:85-107):
+ *      alloc_pack_buffs, sconvGemmNCHW, sconvGemmNHWC, sconvGemmNCHW_back, sconvGemmNHWC_back.
+ *      They live in libconvGemm.so (same sources plus the shim), copy operands to the GPU, run
+ *      the flavour-(1) kernels and copy the result back, so the reference's own ConvGemm class
+ *      can load this build through LD_LIBRARY_PATH unchanged.
+ *
+ * Paths cited below are relative to the PyDTNN source tree.
+ */
+#ifndef PYDTNN_HIP_H
+#define PYDTNN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+#include <stdbool.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PYDTNN_HIP_OK 0
+#define PYDTNN_HIP_ERR_INVALID 1
+#define PYDTNN_HIP_ERR_WORKSPACE 2
+#define PYDTNN_HIP_ERR_LAUNCH 3
+#define PYDTNN_HIP_ERR_UNSUPPORTED 4
+
+/* Library identification: returns 10000*major + 100*minor + patch. */
+int pydtnn_hip_version(void);
+/* Human-readable text for a status code (static storage). */
+const char *pydtnn_hip_status_string(int status);
+
+/* ------------------------------------------------------------------------------------------
+ * Explicit im2col / col2im.  Replace the Cython modules
+ *   im2col_nchw_cython / col2im_nchw_cython   pydtnn/cython_modules/im2col_nchw_cython.pyx:28-52, :150-173
+ *   im2row_nhwc_cython / row2im_nhwc_cython   pydtnn/cython_modules/im2row_nhwc_cython.pyx:25-49, :123-146
+ * with identical index maps.  cols is (c*kh*kw, b*ho*wo); rows is (b*ho*wo, c*kh*kw); the output
+ * is fully written (padding positions get 0; col2im/row2im need no pre-zeroed dx).
+ * ---------------------------------------------------------------------------------------- */
+int pydtnn_hip_im2col_nchw(const float *x, float *cols, int b, int c, int h, int w, int kh, int kw,
+                           int vpadding, int hpadding, int vstride, int hstride, int vdilation, int hdilation,
+                           void *stream);
+int pydtnn_hip_col2im_nchw(const float *cols, float *dx, int b, int c, int h, int w, int kh, int kw,
+                           int vpadding, int hpadding, int vstride, int hstride, int vdilation, int hdilation,
+                           void *stream);
+int pydtnn_hip_im2row_nhwc(const float *x, float *rows, int b, int h, int w, int c, int kh, int kw,
+                           int vpadding, int hpadding, int vstride, int hstride, int vdilation, int hdilation,
+                           void *stream);
+int pydtnn_hip_row2im_nhwc(const float *rows, float *dx, int b, int h, int w, int c, int kh, int kw,
+                           int vpadding, int hpadding, int vstride, int hstride, int vdilation, int hdilation,
+                           void *stream);
+
+/* ------------------------------------------------------------------------------------------
+ * GEMM.  Replaces pydtnn.utils.matmul (pydtnn/utils/__init__.py:148-158: a @ b) for row-major
+ * fp32 operands, with the transposed views NumPy would pass to BLAS:
+ *     C(m x n) = op(A) * op(B),  op(A) = A (m x k, lda) or A^T (A stored k x m, lda) when transa != 0,
+ *                                op(B) = B (k x n, ldb) or B^T (B stored n x k, ldb) when transb != 0.
+ * Optional fused epilogue on C: + bias[n] (FC forward, pydtnn/backends/cpu/layers/fc_cpu.py:63), then ReLU.
+ * Small m*n with long k is split along k; then `workspace` must hold
+ * pydtnn_hip_sgemm_workspace_bytes(m, n, k) bytes (0 means none needed).
+ * ---------------------------------------------------------------------------------------- */
+size_t pydtnn_hip_sgemm_workspace_bytes(long m, long n, long k);
+int pydtnn_hip_sgemm(int transa, int transb, long m, long n, long k, const float *a, long lda, const float *b,
+                     long ldb, float *c, long ldc, const float *bias, int relu, void *workspace,
+                     size_t workspace_bytes, void *stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Implicit-im2col convolution GEMMs: the column matrix is never materialised.
+ * Same argument meaning and order as libconvGemm's sconvGemmNCHW / sconvGemmNHWC
+ * (call sites pydtnn/backends/cpu/libs/conv_gemm.py:191-205 and :234-248), minus the two CPU
+ * packing buffers, plus workspace and stream:
+ *   trans == 'N' : forward.  in1 = weights (NCHW: kn,c,kh,kw; NHWC: c,kh,kw,kn), out = y
+ *                  (NCHW: b,kn,ho,wo; NHWC: b,ho,wo,kn), then per output channel
+ *                  + bias_vector -> ((v - bn_running_mean) * bn_inv_std) * bn_gamma + bn_beta -> ReLU,
+ *                  each stage skipped when its pointer is NULL / relu is false.  The BN stage is
+ *                  applied when bn_running_mean is non-NULL and then needs all four vectors.
+ *   trans == 'Y' : filter gradient.  in1 = dy (layout of y), out = dw (layout of weights);
+ *                  epilogue arguments must be NULL / false.  Needs a workspace of
+ *                  pydtnn_hip_conv_workspace_bytes(PYDTNN_HIP_OP_DW, ...) bytes.
+ * ---------------------------------------------------------------------------------------- */
+#define PYDTNN_HIP_OP_FWD 0
+#define PYDTNN_HIP_OP_DW 1
+#define PYDTNN_HIP_OP_DX 2
+#define PYDTNN_HIP_OP_DX_I2C 3 /* explicit GEMM + col2im/row2im variant of dX */
+#define PYDTNN_HIP_OP_DB 4     /* bias gradient */
+
+size_t pydtnn_hip_conv_workspace_bytes(int op, int nhwc, int b, int c, int h, int w, int kn, int kh, int kw,
+                                       int vpadding, int hpadding, int vstride, int hstride, int vdilation,
+                                       int hdilation);
+
+int pydtnn_hip_sconvGemmNCHW(char trans, unsigned b, unsigned c, unsigned h, unsigned w, unsigned kn, unsigned kh,
+                             unsigned kw, unsigned vpadding, unsigned hpadding, unsigned vstride, unsigned hstride,
+                             unsigned vdilation, unsigned hdilation, const float *in1, const float *x, float *out,
+                             const float *bias_vector, const float *bn_running_mean, const float *bn_inv_std,
+                             const float *bn_gamma, const float *bn_beta, bool relu, void *workspace,
+                             size_t workspace_bytes, void *stream);
+int pydtnn_hip_sconvGemmNHWC(char trans, unsigned b, unsigned h, unsigned w, unsigned c, unsigned kn, unsigned kh,
+                             unsigned kw, unsigned vpadding, unsigned hpadding, unsigned vstride, unsigned hstride,
+                             unsigned vdilation, unsigned hdilation, const float *in1, const float *x, float *out,
+                             const float *bias_vector, const float *bn_running_mean, const float *bn_inv_std,
+                             const float *bn_gamma, const float *bn_beta, bool relu, void *workspace,
+                             size_t workspace_bytes, void *stream);
+
+/* Input gradient dx = col2im(W^T dy) without the (K x P) matrix: libconvGemm's sconvGemmNCHW_back /
+ * sconvGemmNHWC_back (pydtnn/backends/cpu/libs/conv_gemm.py:299-307, :321-328; note stride comes before
+ * padding in this argument list, as in the reference).  dx is fully overwritten (the reference
+ * requires the caller to zero it first; here that is not needed).  Workspace:
+ * pydtnn_hip_conv_workspace_bytes(PYDTNN_HIP_OP_DX, ...). */
+int pydtnn_hip_sconvGemmNCHW_back(unsigned b, unsigned c, unsigned h, unsigned w, unsigned kn, unsigned kh,
+                                  unsigned kw, unsigned vstride, unsigned hstride, unsigned vpadding,
+                                  unsigned hpadding, unsigned vdilation, unsigned hdilation, const float *weights,
+                                  const float *dy, float *dx, void *workspace, size_t workspace_bytes,
+                                  void *stream);
+int pydtnn_hip_sconvGemmNHWC_back(unsigned b, unsigned h, unsigned w, unsigned c, unsigned kn, unsigned kh,
+                                  unsigned kw, unsigned vstride, unsigned hstride, unsigned vpadding,
+                                  unsigned hpadding, unsigned vdilation, unsigned hdilation, const float *weights,
+                                  const float *dy, float *dx, void *workspace, size_t workspace_bytes,
+                                  void *stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Explicit ("i2c") convolution GEMMs over a materialised column / row matrix: the GEMM steps of
+ *   Conv2DCPU._forward_nchw_i2c / _backward_nchw_i2c   pydtnn/backends/cpu/layers/conv_2d_cpu.py:264-291, :447-481
+ *   Conv2DCPU._forward_nhwc_i2c / _backward_nhwc_i2c   pydtnn/backends/cpu/layers/conv_2d_cpu.py:183-209, :363-397
+ * `mat` is x_cols (NCHW: c*kh*kw x b*ho*wo) or x_rows (NHWC: b*ho*wo x c*kh*kw).
+ *   forward : y = W * x_cols (+ bias), written straight in the tensor format (the reference's
+ *             separate bias pass and 1023 transpose are folded into the store).
+ *   dw      : dw = dy_cols * x_cols^T   (NHWC: x_rows^T * dy_rows).  Workspace: OP_DW bytes.
+ *   dx      : dx = col2im(W^T * dy_cols) (NHWC: row2im(dy_rows * W^T)); the (K x P) product goes
+ *             through the workspace: OP_DX_I2C bytes.
+ * ---------------------------------------------------------------------------------------- */
+int pydtnn_hip_conv_i2c_forward(int nhwc, int b, int c, int h, int w, int kn, int kh, int kw, int vpadding,
+                                int hpadding, int vstride, int hstride, int vdilation, int hdilation,
+                                const float *weights, const float *mat, float *y, const float *bias_vector,
+                                void *stream);
+int pydtnn_hip_conv_i2c_dw(int nhwc, int b, int c, int h, int w, int kn, int kh, int kw, int vpadding, int hpadding,
+                           int vstride, int hstride, int vdilation, int hdilation, const float *dy, const float *mat,
+                           float *dw, void *workspace, size_t workspace_bytes, void *stream);
+int pydtnn_hip_conv_i2c_dx(int nhwc, int b, int c, int h, int w, int kn, int kh, int kw, int vpadding, int hpadding,
+                           int vstride, int hstride, int vdilation, int hdilation, const float *weights,
+                           const float *dy, float *dx, void *workspace, size_t workspace_bytes, void *stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Stand-alone per-channel epilogue (for layers that are not fused into a convolution):
+ *   y = relu?( bn?( x (+ residual) + bias ) )    with channel = (index / inner) % channels.
+ * inner = ho*wo for NCHW tensors, 1 for NHWC tensors and (rows, C) matrices.  Covers
+ *   add_nchw_cython / add_nhwc_cython            pydtnn/cython_modules/add_nchw_cython.pyx:51-58, add_nhwc_cython.pyx:51-58
+ *   bn_inference_cython / bn_inference_nchw      pydtnn/cython_modules/bn_inference_cython.pyx:61-72, :127-140
+ *   bn_relu_inference_cython                     pydtnn/cython_modules/bn_relu_inference_cython.pyx:59-70
+ *   eltw_sum_cython (residual)                   pydtnn/cython_modules/eltw_sum_cython.pyx:25-36
+ * Any of residual, bias, the four BN vectors may be NULL; x and y may alias.
+ * ---------------------------------------------------------------------------------------- */
+int pydtnn_hip_chan_eltwise(const float *x, const float *residual, float *y, long total, int inner, int channels,
+                            const float *bias, const float *bn_running_mean, const float *bn_inv_std,
+                            const float *bn_gamma, const float *bn_beta, int relu, void *stream);
+
+/* relu_cython (pydtnn/cython_modules/relu_cython.pyx:25-59): y = x > 0 ? x : 0, mask = x > 0 (int8; may be NULL).
+ * Backward dx = dy * mask (pydtnn/backends/cpu/activations/relu_cpu.py:38-40). */
+int pydtnn_hip_relu_fwd(const float *x, float *y, int8_t *mask, long total, void *stream);
+int pydtnn_hip_relu_bwd(const float *dy, const int8_t *mask, float *dx, long total, void *stream);
+
+/* db = sum of dy over batch and pixels (pydtnn/backends/cpu/layers/conv_2d_cpu.py:377, :463; fc_cpu.py:70).
+ * dy is (outer, channels, inner): inner = ho*wo for NCHW, 1 for NHWC / FC.
+ * Workspace: pydtnn_hip_conv_workspace_bytes(PYDTNN_HIP_OP_DB, ...) or 256*channels bytes. */
+int pydtnn_hip_bias_grad(const float *dy, float *db, long outer, int channels, int inner, void *workspace,
+                         size_t workspace_bytes, void *stream);
+
+/* MaxPool2D, NCHW (pydtnn/cython_modules/max_pool_2d_nchw_cython.pyx:25-52, :140-166); idx_max is int32 (b,c,ho,wo). */
+int pydtnn_hip_max_pool_2d_fwd_nchw(const float *x, float *y, int32_t *idx_max, int b, int c, int h, int w, int kh,
+                                    int kw, int vpadding, int hpadding, int vstride, int hstride, int vdilation,
+                                    int hdilation, void *stream);
+int pydtnn_hip_max_pool_2d_bwd_nchw(const float *dy, const int32_t *idx_max, float *dx, int b, int c, int h, int w,
+                                    int kh, int kw, int vpadding, int hpadding, int vstride, int hstride,
+                                    int vdilation, int hdilation, void *stream);
+
+/* SGD with momentum, in place (pydtnn/backends/cpu/optimizers/sgd_cpu.py:28-41). */
+int pydtnn_hip_sgd_momentum(float *w, const float *dw, float *velocity, long total, float lr, float momentum,
+                            float decay, int nesterov, void *stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Host-pointer compatibility flavour (exported by libconvGemm.so only).  Signatures are those
+ * PyDTNN's ctypes shim calls (pydtnn/backends/cpu/libs/conv_gemm.py:91-92, :191-205, :234-248,
+ * :299-307, :321-328).  ac_pack / bc_pack are accepted and ignored; alloc_pack_buffs hands out two
+ * small malloc() blocks because the reference free()s them with libc (:109-115, :332-349).
+ * Errors cannot be returned through this ABI (the reference has no error channel): a failure is
+ * reported on stderr and aborts the process rather than returning wrong numbers.
+ * ---------------------------------------------------------------------------------------- */
+int alloc_pack_buffs(float **ac_pack, float **bc_pack);
+void sconvGemmNCHW(char trans, unsigned b, unsigned c, unsigned h, unsigned w, unsigned kn, unsigned kh, unsigned kw,
+                   unsigned vpadding, unsigned hpadding, unsigned vstride, unsigned hstride, unsigned vdilation,
+                   unsigned hdilation, const float *in1, const float *x, float *out, const float *bias_vector,
+                   const float *bn_running_mean, const float *bn_inv_std, const float *bn_gamma,
+                   const float *bn_beta, bool relu, float *ac_pack, float *bc_pack);
+void sconvGemmNHWC(char trans, unsigned b, unsigned h, unsigned w, unsigned c, unsigned kn, unsigned kh, unsigned kw,
+                   unsigned vpadding, unsigned hpadding, unsigned vstride, unsigned hstride, unsigned vdilation,
+                   unsigned hdilation, const float *in1, const float *x, float *out, const float *bias_vector,
+                   const float *bn_running_mean, const float *bn_inv_std, const float *bn_gamma,
+                   const float *bn_beta, bool relu, float *ac_pack, float *bc_pack);
+void sconvGemmNCHW_back(unsigned b, unsigned c, unsigned h, unsigned w, unsigned kn, unsigned kh, unsigned kw,
+                        unsigned vstride, unsigned hstride, unsigned vpadding, unsigned hpadding, unsigned vdilation,
+                        unsigned hdilation, const float *weights, const float *dy, float *dx, float *ac_pack,
+                        float *bc_pack);
+void sconvGemmNHWC_back(unsigned b, unsigned h, unsigned w, unsigned c, unsigned kn, unsigned kh, unsigned kw,
+                        unsigned vstride, unsigned hstride, unsigned vpadding, unsigned hpadding, unsigned vdilation,
+                        unsigned hdilation, const float *weights, const float *dy, float *dx, float *ac_pack,
+                        float *bc_pack);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PYDTNN_HIP_H */

@@ -1,0 +1,138 @@
+"""``ConvGemm``: the reference's shim over libconvGemm, re-hosted on the MI355X library.
+
+Same class name, method names, keyword arguments, shape asserts and return values as
+pydtnn/backends/cpu/libs/conv_gemm.py:39-330, but operands are GPU tensors (``torch.Tensor`` on
+``cuda``) and the call goes to the device-pointer C ABI.  The convolution is an implicit GEMM:
+the im2col matrix never exists in memory.
+"""
+import torch
+
+from . import native
+from .native import check, f32, lib, stream_ptr
+
+is_conv_gemm_available = True  # pydtnn/backends/cpu/libs/conv_gemm.py:32-36: probe result of load_library
+
+
+class ConvGemm:
+    """Exposes the implicit-GEMM convolution entry points following the PyDTNN conventions."""
+
+    def __init__(self, dtype=torch.float32, debug=False, parent_layer=None):
+        # pydtnn/backends/cpu/libs/conv_gemm.py:79-86 accepts a type or its name
+        names = {"float32": torch.float32, "float64": torch.float64}
+        if isinstance(dtype, str):
+            if dtype not in names:
+                raise AttributeError("dtype '{}' not recognized".format(dtype))
+            dtype = names[dtype]
+        elif not isinstance(dtype, torch.dtype):
+            try:
+                import numpy as np
+                dtype = {np.dtype("float32"): torch.float32, np.dtype("float64"): torch.float64}[np.dtype(dtype)]
+            except (KeyError, TypeError):
+                raise AttributeError("dtype '{}' not recognized".format(dtype)) from None
+        self.dtype = dtype
+        if self.dtype != torch.float32:
+            # pydtnn/backends/cpu/libs/conv_gemm.py:101-107
+            raise ValueError("Type {} not supported by this version of libconvGemm!".format(str(self.dtype)))
+        native.lib()  # fail here, loudly, if the HIP library is not built
+        self.debug = debug
+        self.parent_layer = parent_layer
+
+    # ------------------------------------------------------------------ forward / dW
+    def conv_gemm_nchw(self, weights, x, biases=None, vpadding=0, hpadding=0, vstride=1, hstride=1,
+                       vdilation=1, hdilation=1, biases_vector=None, trans=False, bn_running_mean=None,
+                       bn_inv_std=None, bn_gamma=None, bn_beta=None, relu=False):
+        """``weights * im2col(x)`` (+ fused bias / BN / ReLU), or with ``trans`` the filter gradient
+        ``dy_cols * im2col(x)^T`` written into ``biases`` (pydtnn/backends/cpu/libs/conv_gemm.py:117-207)."""
+        b, c, h, w = x.shape
+        if not trans:
+            kn, ck, kh, kw = weights.shape
+            if biases is None:
+                ho = (h + 2 * vpadding - vdilation * (kh - 1) - 1) // vstride + 1
+                wo = (w + 2 * hpadding - hdilation * (kw - 1) - 1) // hstride + 1
+                biases = torch.empty((b, kn, ho, wo), dtype=weights.dtype, device=weights.device)
+            else:
+                bb, knb, ho, wo = biases.shape
+                assert kn == knb, "Number of filters must be the same!"
+                assert b == bb, "Batch size must be the same!"
+        else:
+            assert biases is not None, "If using the transposed convGemm, the biases matrix must be supplied"
+            kn, ck, kh, kw = biases.shape
+            bw, knw, ho, wo = weights.shape
+            assert kn == knw, "Number of filters must be the same!"
+            assert b == bw, "Batch size must be the same!"
+        assert ck == c, "Number of channels in weights and x should be the same!"
+        assert weights.dtype == x.dtype == biases.dtype, "All the matrices must have the same type of data!"
+        assert weights.dtype == self.dtype, \
+            "The input matrices must have the same type of data as the one specified when " \
+            "this class was instantiated!"
+        geom = (b, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
+        ws, ws_bytes = native.conv_workspace(native.OP_DW, 0, geom) if trans else (None, 0)
+        check(lib().pydtnn_hip_sconvGemmNCHW(
+            b'Y' if trans else b'N', b, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation,
+            hdilation, f32(weights), f32(x), f32(biases), f32(biases_vector), f32(bn_running_mean), f32(bn_inv_std),
+            f32(bn_gamma), f32(bn_beta), bool(relu), ws, ws_bytes, stream_ptr()), "sconvGemmNCHW")
+        return biases
+
+    def conv_gemm_nhwc(self, weights, x, biases=None, vpadding=0, hpadding=0, vstride=1, hstride=1,
+                       vdilation=1, hdilation=1, biases_vector=None, trans=False, bn_running_mean=None,
+                       bn_inv_std=None, bn_gamma=None, bn_beta=None, relu=False):
+        """NHWC twin (pydtnn/backends/cpu/libs/conv_gemm.py:209-250): weights (c, kh, kw, kn)."""
+        b, h, w, c = x.shape
+        if not trans:
+            ck, kh, kw, kn = weights.shape
+            if biases is None:
+                ho = (h + 2 * vpadding - vdilation * (kh - 1) - 1) // vstride + 1
+                wo = (w + 2 * hpadding - hdilation * (kw - 1) - 1) // hstride + 1
+                biases = torch.empty((b, ho, wo, kn), dtype=weights.dtype, device=weights.device)
+            else:
+                bb, ho, wo, knb = biases.shape
+                assert kn == knb, "Number of filters must be the same!"
+                assert b == bb, "Batch size must be the same!"
+        else:
+            assert biases is not None, "If using the transposed convGemm, the output matrix must be supplied"
+            ck, kh, kw, kn = biases.shape
+            bw, ho, wo, knw = weights.shape
+            assert kn == knw, "Number of filters must be the same!"
+            assert b == bw, "Batch size must be the same!"
+        assert ck == c, "Number of channels in weights and x should be the same!"
+        assert weights.dtype == x.dtype == biases.dtype, "All the matrices must have the same type of data!"
+        geom = (b, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
+        ws, ws_bytes = native.conv_workspace(native.OP_DW, 1, geom) if trans else (None, 0)
+        check(lib().pydtnn_hip_sconvGemmNHWC(
+            b'Y' if trans else b'N', b, h, w, c, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation,
+            hdilation, f32(weights), f32(x), f32(biases), f32(biases_vector), f32(bn_running_mean), f32(bn_inv_std),
+            f32(bn_gamma), f32(bn_beta), bool(relu), ws, ws_bytes, stream_ptr()), "sconvGemmNHWC")
+        return biases
+
+    # ------------------------------------------------------------------ dX
+    def deconv_gemm_nchw(self, weights, dy, dx, vpadding=0, hpadding=0, vstride=1, hstride=1,
+                         vdilation=1, hdilation=1):
+        """dx = col2im(weights_2D^T * dy_2D) (pydtnn/backends/cpu/libs/conv_gemm.py:252-309)."""
+        kn, ck, kh, kw = weights.shape
+        b2, kn2, ho, wo = dy.shape
+        b, c, h, w = dx.shape
+        assert kn == kn2, "Number of filters outputs in weights and dy should be the same!"
+        assert b == b2, "Different batch size!"
+        assert ck == c, "Number of channels in weights and x should be the same!"
+        geom = (b, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
+        ws, ws_bytes = native.conv_workspace(native.OP_DX, 0, geom)
+        check(lib().pydtnn_hip_sconvGemmNCHW_back(
+            b, c, h, w, kn, kh, kw, vstride, hstride, vpadding, hpadding, vdilation, hdilation,
+            f32(weights), f32(dy), f32(dx), ws, ws_bytes, stream_ptr()), "sconvGemmNCHW_back")
+        return dx
+
+    def deconv_gemm_nhwc(self, weights, dy, dx, vpadding=0, hpadding=0, vstride=1, hstride=1,
+                         vdilation=1, hdilation=1):
+        """NHWC twin (pydtnn/backends/cpu/libs/conv_gemm.py:311-330)."""
+        ck, kh, kw, kn = weights.shape
+        b2, ho, wo, kn2 = dy.shape
+        b, h, w, c = dx.shape
+        assert kn == kn2, "Number of filters outputs in weights and dy should be the same!"
+        assert b == b2, "Different batch size!"
+        assert ck == c, "Number of channels in weights and x should be the same!"
+        geom = (b, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
+        ws, ws_bytes = native.conv_workspace(native.OP_DX, 1, geom)
+        check(lib().pydtnn_hip_sconvGemmNHWC_back(
+            b, h, w, c, kn, kh, kw, vstride, hstride, vpadding, hpadding, vdilation, hdilation,
+            f32(weights), f32(dy), f32(dx), ws, ws_bytes, stream_ptr()), "sconvGemmNHWC_back")
+        return dx

@@ -1,0 +1,90 @@
+// Shared declarations for the gfx950 conv-as-GEMM kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+
+// Status codes returned by every device-pointer entry point.
+#define PYDTNN_HIP_OK 0
+#define PYDTNN_HIP_ERR_INVALID 1      // bad argument (null pointer, zero extent, unknown flag)
+#define PYDTNN_HIP_ERR_WORKSPACE 2    // workspace missing or too small
+#define PYDTNN_HIP_ERR_LAUNCH 3       // HIP reported a launch/runtime error
+#define PYDTNN_HIP_ERR_UNSUPPORTED 4  // extents beyond what the index arithmetic covers
+
+// Division of a small unsigned by a run-time constant as one mul-hi.
+// Exact for every n with n * div < 2^32 (checked on the host before a launch).
+struct FastDiv {
+    uint32_t mul;
+    uint32_t div;
+};
+
+static inline FastDiv make_fastdiv(uint32_t d)
+{
+    FastDiv f;
+    f.div = d;
+    f.mul = d <= 1 ? 0u : (uint32_t)(((1ull << 32) + d - 1) / d);
+    return f;
+}
+
+__device__ __forceinline__ uint32_t fd_div(uint32_t n, const FastDiv f)
+{
+    return f.div == 1 ? n : __umulhi(n, f.mul);
+}
+
+// Geometry of one convolution. Names follow PyDTNN's Conv2D (vpadding = vertical padding, ...).
+// Output extent: ho = (h + 2*vpadding - vdilation*(kh-1) - 1) / vstride + 1 (pydtnn/layers/conv_2d.py:75-76).
+struct ConvGeom {
+    int n, c, h, w;     // input batch, channels, height, width
+    int kn, kh, kw;     // filters, filter height, filter width
+    int vpadding, hpadding, vstride, hstride, vdilation, hdilation;
+    int ho, wo;         // output height, width
+    int k;              // c*kh*kw  (reduction length of the forward GEMM)
+    int khw;            // kh*kw
+    int howo;           // ho*wo
+    long p;             // n*ho*wo  (pixels = GEMM columns in NCHW, rows in NHWC)
+    FastDiv fd_khw, fd_kw, fd_wo, fd_c, fd_howo;
+};
+
+static inline int conv_out_dim(int in, int pad, int dil, int k, int stride)
+{
+    return (in + 2 * pad - dil * (k - 1) - 1) / stride + 1;
+}
+
+// Fills a ConvGeom; returns a PYDTNN_HIP_* status.
+int make_conv_geom(ConvGeom* g, int n, int c, int h, int w, int kn, int kh, int kw,
+                   int vpadding, int hpadding, int vstride, int hstride, int vdilation, int hdilation);
+
+// Per-channel epilogue applied to an accumulator before the single store:
+//   v += bias[ch];  v = ((v - mean[ch]) * inv_std[ch]) * gamma[ch] + beta[ch];  v = v > 0 ? v : 0
+// in that order (bias -> BN inference -> ReLU), each stage optional.
+struct ChanEpilogue {
+    const float* bias;
+    const float* mean;
+    const float* inv_std;
+    const float* gamma;
+    const float* beta;
+    int relu;
+};
+
+__device__ __forceinline__ float chan_epilogue_apply(const ChanEpilogue& e, int ch, float v)
+{
+    if (e.bias) v += e.bias[ch];
+    if (e.mean) {
+        float t = (v - e.mean[ch]) * e.inv_std[ch];
+        v = t * e.gamma[ch] + e.beta[ch];
+    }
+    if (e.relu) v = v > 0.0f ? v : 0.0f;
+    return v;
+}
+
+static inline ChanEpilogue no_epilogue()
+{
+    ChanEpilogue e = {nullptr, nullptr, nullptr, nullptr, nullptr, 0};
+    return e;
+}
+
+#define HIP_RETURN_IF_LAUNCH_FAILED()                         \
+    do {                                                      \
+        hipError_t e__ = hipGetLastError();                   \
+        if (e__ != hipSuccess) return PYDTNN_HIP_ERR_LAUNCH;  \
+    } while (0)

@@ -1,0 +1,629 @@
+// Device-pointer C ABI: argument checks, tile / split selection and kernel launches.
+#include "../../include/pydtnn_hip.h"
+#include "gemm_engine.h"
+
+// launchers defined in gather_kernels.hip / eltwise_kernels.hip
+int launch_im2col_nchw(const float*, float*, const ConvGeom&, hipStream_t);
+int launch_col2im_nchw(const float*, float*, const ConvGeom&, hipStream_t);
+int launch_im2row_nhwc(const float*, float*, const ConvGeom&, hipStream_t);
+int launch_row2im_nhwc(const float*, float*, const ConvGeom&, hipStream_t);
+int launch_chan_eltwise(const float*, const float*, float*, long, int, int, const ChanEpilogue&, hipStream_t);
+int launch_relu_fwd(const float*, float*, int8_t*, long, hipStream_t);
+int launch_relu_bwd(const float*, const int8_t*, float*, long, hipStream_t);
+size_t bias_grad_workspace_floats(long, int);
+int launch_bias_grad(const float*, float*, long, int, int, float*, hipStream_t);
+int launch_splitk_reduce(const float*, float*, long, int, long, int, int, int, const ChanEpilogue&, hipStream_t);
+int launch_flip_filter(const float*, float*, int, int, int, int, int, hipStream_t);
+int launch_max_pool_fwd_nchw(const float*, float*, int32_t*, const ConvGeom&, hipStream_t);
+int launch_max_pool_bwd_nchw(const float*, const int32_t*, float*, const ConvGeom&, hipStream_t);
+int launch_sgd_momentum(float*, const float*, float*, long, float, float, float, int, hipStream_t);
+
+namespace {
+
+using namespace gemm;
+
+typedef Tile<128, 128, 2, 2> T128x128;
+typedef Tile<64, 256, 1, 4> T64x256;
+typedef Tile<256, 64, 4, 1> T256x64;
+
+enum TileSel { SEL_128x128, SEL_64x256, SEL_256x64 };
+
+inline TileSel pick_tile(long m, long n)
+{
+    if (m <= 64) return SEL_64x256;
+    if (n <= 64) return SEL_256x64;
+    return SEL_128x128;
+}
+
+inline long tiles_of(TileSel sel, long m, long n)
+{
+    const long bm = sel == SEL_64x256 ? 64 : sel == SEL_256x64 ? 256 : 128;
+    const long bn = sel == SEL_64x256 ? 256 : sel == SEL_256x64 ? 64 : 128;
+    return ((m + bm - 1) / bm) * ((n + bn - 1) / bn);
+}
+
+#define WITH_TILE(sel, ...)                                                 \
+    switch (sel) {                                                          \
+        case SEL_64x256: { typedef T64x256 T; __VA_ARGS__; } break;         \
+        case SEL_256x64: { typedef T256x64 T; __VA_ARGS__; } break;         \
+        default: { typedef T128x128 T; __VA_ARGS__; } break;                \
+    }
+
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+inline long round_up(long v, long m) { return (v + m - 1) / m * m; }
+
+// Target number of workgroups for a launch that has to be split along the reduction axis:
+// four per CU on a 256-CU part.
+constexpr long kTargetBlocks = 1024;
+constexpr long kMinChunk = 256;
+constexpr size_t kMaxPartialBytes = (size_t)768 << 20;
+
+struct SplitPlan {
+    SplitInfo si;
+    int splits;
+};
+
+// Reduction over `images` segments of `seg` elements (pixels of one image).
+SplitPlan plan_pixel_split(long tiles, int images, int seg, long out_elems)
+{
+    const long total = (long)images * seg;
+    long want = tiles >= kTargetBlocks ? 1 : (kTargetBlocks + tiles - 1) / tiles;
+    const long max_by_ws = (long)(kMaxPartialBytes / ((size_t)out_elems * 4));
+    if (want > max_by_ws) want = max_by_ws < 1 ? 1 : max_by_ws;
+    long chunk = round_up((total + want - 1) / want, BK);
+    if (chunk < kMinChunk) chunk = kMinChunk;
+    SplitPlan p;
+    if (chunk >= seg) {
+        long ips = chunk / seg;
+        if (ips > images) ips = images;
+        // FastDiv by seg must stay exact for every reduction index of a group
+        const long ips_cap = (((1l << 32) - 1) / seg - 256) / seg;
+        if (ips > ips_cap) ips = ips_cap < 1 ? 1 : ips_cap;
+        p.si = make_split(seg, images, (int)ips, 1, (int)(ips * seg));
+        p.splits = (int)((images + ips - 1) / ips);
+    } else {
+        int cpg = (int)((seg + chunk - 1) / chunk);
+        chunk = round_up((seg + cpg - 1) / cpg, BK);
+        cpg = (int)((seg + chunk - 1) / chunk);
+        p.si = make_split(seg, images, 1, cpg, (int)chunk);
+        p.splits = images * cpg;
+    }
+    return p;
+}
+
+// Plain GEMM: one segment of length k.
+SplitPlan plan_plain_split(long tiles, long k, long out_elems)
+{
+    SplitPlan p;
+    long want = tiles >= 256 ? 1 : (kTargetBlocks + tiles - 1) / tiles;
+    const long max_by_ws = (long)(kMaxPartialBytes / ((size_t)out_elems * 4));
+    if (want > max_by_ws) want = max_by_ws < 1 ? 1 : max_by_ws;
+    long chunk = round_up((k + want - 1) / want, BK);
+    if (chunk < kMinChunk) chunk = kMinChunk;
+    if (chunk > k) chunk = k;
+    const int splits = (int)((k + chunk - 1) / chunk);
+    p.si = make_split((int)k, 1, 1, splits, (int)chunk);
+    p.splits = splits;
+    return p;
+}
+
+inline ChanEpilogue make_chan(const float* bias, const float* mean, const float* inv_std, const float* gamma,
+                              const float* beta, int relu)
+{
+    ChanEpilogue e = {bias, mean, inv_std, gamma, beta, relu};
+    return e;
+}
+
+inline bool bn_args_consistent(const float* mean, const float* inv_std, const float* gamma, const float* beta)
+{
+    const int set = (mean != nullptr) + (inv_std != nullptr) + (gamma != nullptr) + (beta != nullptr);
+    return set == 0 || set == 4;
+}
+
+template <int BMN, bool SEG>
+inline PlainK<BMN, SEG> plain_k(const float* base, long ld, long image_stride, long extent, int seg_len)
+{
+    PlainK<BMN, SEG> l;
+    l.base = base; l.ld = ld; l.image_stride = image_stride; l.extent = (int)extent;
+    l.seg_len = seg_len; l.fd_seg = make_fastdiv((uint32_t)(seg_len > 0 ? seg_len : 1));
+    return l;
+}
+
+template <int BMN>
+inline PlainMN<BMN> plain_mn(const float* base, long ld, long image_stride, long extent)
+{
+    PlainMN<BMN> l;
+    l.base = base; l.ld = ld; l.image_stride = image_stride; l.extent = (int)extent;
+    return l;
+}
+
+inline EpiPlain epi_plain(float* out, long ldc, long split_stride, long m, long n, const ChanEpilogue& chan)
+{
+    EpiPlain e;
+    e.out = out; e.ldc = ldc; e.split_stride = split_stride; e.m_extent = (int)m; e.n_extent = (int)n; e.chan = chan;
+    return e;
+}
+
+inline EpiNchw epi_nchw(float* out, int channels, int howo, long p, const ChanEpilogue& chan)
+{
+    EpiNchw e;
+    e.out = out; e.m_extent = channels; e.howo = howo; e.p = p; e.chan = chan;
+    return e;
+}
+
+// ---------------------------------------------------------------- forward (implicit)
+int conv_fwd_nchw(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan,
+                  hipStream_t stream)
+{
+    const TileSel sel = pick_tile(g.kn, g.p);
+    int rc = PYDTNN_HIP_OK;
+    WITH_TILE(sel, {
+        auto al = plain_k<T::BM, false>(w, g.k, 0, g.kn, 0);
+        Im2colNchwMN<T::BN> bl;
+        bl.x = x; bl.g = g;
+        rc = launch<T>(al, bl, epi_nchw(y, g.kn, g.howo, g.p, chan), g.kn, g.p, no_split(g.k), 1, stream);
+    })
+    return rc;
+}
+
+int conv_fwd_nhwc(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan,
+                  hipStream_t stream)
+{
+    const TileSel sel = pick_tile(g.p, g.kn);
+    int rc = PYDTNN_HIP_OK;
+    WITH_TILE(sel, {
+        Im2rowNhwcK<T::BM> al;
+        al.x = x; al.g = g;
+        FilterNhwcMN<T::BN> bl;
+        bl.w = w; bl.g = g;
+        rc = launch<T>(al, bl, epi_plain(y, g.kn, 0, g.p, g.kn, chan), g.p, g.kn, no_split(g.k), 1, stream);
+    })
+    return rc;
+}
+
+// ---------------------------------------------------------------- filter gradient
+// mat == nullptr: implicit (x gathered on the fly); otherwise the materialised x_cols / x_rows.
+SplitPlan plan_dw(const ConvGeom& g, int nhwc)
+{
+    const long m = nhwc ? g.k : g.kn, n = nhwc ? g.kn : g.k;
+    const TileSel sel = pick_tile(m, n);
+    return plan_pixel_split(tiles_of(sel, m, n), g.n, g.howo, (long)g.kn * g.k);
+}
+
+int conv_dw_nchw(const ConvGeom& g, const float* dy, const float* x, const float* cols, float* dw, float* ws,
+                 size_t ws_bytes, hipStream_t stream)
+{
+    const SplitPlan sp = plan_dw(g, 0);
+    const long out_elems = (long)g.kn * g.k;
+    if (!ws || ws_bytes < (size_t)sp.splits * out_elems * 4) return PYDTNN_HIP_ERR_WORKSPACE;
+    const TileSel sel = pick_tile(g.kn, g.k);
+    int rc = PYDTNN_HIP_OK;
+    WITH_TILE(sel, {
+        // A(m = filter, k = (image, pixel)) = dy[image][filter][pixel]
+        auto al = plain_k<T::BM, true>(dy, g.howo, (long)g.kn * g.howo, g.kn, g.howo);
+        const EpiPlain ep = epi_plain(ws, g.k, out_elems, g.kn, g.k, no_epilogue());
+        if (cols) {
+            // B(k = (image, pixel), n = row of cols) = cols[n][image*howo + pixel]
+            auto bl = plain_k<T::BN, true>(cols, g.p, g.howo, g.k, g.howo);
+            rc = launch<T>(al, bl, ep, g.kn, g.k, sp.si, sp.splits, stream);
+        } else {
+            Im2colNchwK<T::BN> bl;
+            bl.x = x; bl.g = g;
+            rc = launch<T>(al, bl, ep, g.kn, g.k, sp.si, sp.splits, stream);
+        }
+    })
+    if (rc != PYDTNN_HIP_OK) return rc;
+    return launch_splitk_reduce(ws, dw, g.kn, g.k, out_elems, sp.splits, 0, 0, no_epilogue(), stream);
+}
+
+int conv_dw_nhwc(const ConvGeom& g, const float* dy, const float* x, const float* rows, float* dw, float* ws,
+                 size_t ws_bytes, hipStream_t stream)
+{
+    const SplitPlan sp = plan_dw(g, 1);
+    const long out_elems = (long)g.kn * g.k;
+    if (!ws || ws_bytes < (size_t)sp.splits * out_elems * 4) return PYDTNN_HIP_ERR_WORKSPACE;
+    const TileSel sel = pick_tile(g.k, g.kn);
+    int rc = PYDTNN_HIP_OK;
+    WITH_TILE(sel, {
+        // B(k = (image, pixel), n = filter) = dy[(image*howo + pixel)*kn + n]
+        auto bl = plain_mn<T::BN>(dy, g.kn, (long)g.howo * g.kn, g.kn);
+        const EpiPlain ep = epi_plain(ws, g.kn, out_elems, g.k, g.kn, no_epilogue());
+        if (rows) {
+            // A(m = column of rows, k) = rows[(image*howo + pixel)*K + m]
+            auto al = plain_mn<T::BM>(rows, g.k, (long)g.howo * g.k, g.k);
+            rc = launch<T>(al, bl, ep, g.k, g.kn, sp.si, sp.splits, stream);
+        } else {
+            Im2rowNhwcMN<T::BM> al;
+            al.x = x; al.g = g;
+            rc = launch<T>(al, bl, ep, g.k, g.kn, sp.si, sp.splits, stream);
+        }
+    })
+    if (rc != PYDTNN_HIP_OK) return rc;
+    // implicit rows come out in (i, j, c) order; materialised x_rows already has the (c, i, j) order
+    const int perm_c = rows ? 0 : g.c;
+    return launch_splitk_reduce(ws, dw, g.k, g.kn, out_elems, sp.splits, perm_c, g.khw, no_epilogue(), stream);
+}
+
+// ---------------------------------------------------------------- input gradient
+// Stride 1: dx = forward convolution of dy with the flipped, channel-swapped filter and padding
+// dilation*(k-1) - padding.  Otherwise: the reference's own route, W^T dy then col2im / row2im.
+inline bool dx_as_forward(const ConvGeom& g)
+{
+    return g.vstride == 1 && g.hstride == 1 && g.vdilation * (g.kh - 1) >= g.vpadding &&
+           g.hdilation * (g.kw - 1) >= g.hpadding;
+}
+
+int conv_dx_i2c(const ConvGeom& g, int nhwc, const float* w, const float* dy, float* dx, float* ws, size_t ws_bytes,
+                hipStream_t stream)
+{
+    const size_t need = (size_t)g.k * g.p * 4;
+    if (!ws || ws_bytes < need) return PYDTNN_HIP_ERR_WORKSPACE;
+    if ((long)g.k * g.p >= (1l << 33)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+    int rc = PYDTNN_HIP_OK;
+    if (!nhwc) {
+        // res(K x P) = W^T (A(m = k, kk = filter) = w[kk*K + m]) * dy_cols (dy seen as a 1x1 im2col)
+        ConvGeom g1;
+        rc = make_conv_geom(&g1, g.n, g.kn, g.ho, g.wo, 1, 1, 1, 0, 0, 1, 1, 1, 1);
+        if (rc != PYDTNN_HIP_OK) return rc;
+        const TileSel sel = pick_tile(g.k, g.p);
+        WITH_TILE(sel, {
+            auto al = plain_mn<T::BM>(w, g.k, 0, g.k);
+            Im2colNchwMN<T::BN> bl;
+            bl.x = dy; bl.g = g1;
+            rc = launch<T>(al, bl, epi_plain(ws, g.p, 0, g.k, g.p, no_epilogue()), g.k, g.p, no_split(g.kn), 1,
+                           stream);
+        })
+        if (rc != PYDTNN_HIP_OK) return rc;
+        return launch_col2im_nchw(ws, dx, g, stream);
+    }
+    // res(P x K) = dy_rows (P x kn) * W_rows^T : B(kk = filter, n = k) = w[n*kn + kk]
+    const TileSel sel = pick_tile(g.p, g.k);
+    WITH_TILE(sel, {
+        auto al = plain_k<T::BM, false>(dy, g.kn, 0, g.p, 0);
+        auto bl = plain_k<T::BN, false>(w, g.kn, 0, g.k, 0);
+        rc = launch<T>(al, bl, epi_plain(ws, g.k, 0, g.p, g.k, no_epilogue()), g.p, g.k, no_split(g.kn), 1, stream);
+    })
+    if (rc != PYDTNN_HIP_OK) return rc;
+    return launch_row2im_nhwc(ws, dx, g, stream);
+}
+
+int conv_dx(const ConvGeom& g, int nhwc, const float* w, const float* dy, float* dx, float* ws, size_t ws_bytes,
+            hipStream_t stream)
+{
+    if (!dx_as_forward(g)) return conv_dx_i2c(g, nhwc, w, dy, dx, ws, ws_bytes, stream);
+    const size_t need = (size_t)g.kn * g.k * 4;
+    if (!ws || ws_bytes < need) return PYDTNN_HIP_ERR_WORKSPACE;
+    int rc = launch_flip_filter(w, ws, nhwc, g.kn, g.c, g.kh, g.kw, stream);
+    if (rc != PYDTNN_HIP_OK) return rc;
+    ConvGeom gb;  // input = dy (kn channels, ho x wo), filters = c, output = (h, w)
+    rc = make_conv_geom(&gb, g.n, g.kn, g.ho, g.wo, g.c, g.kh, g.kw, g.vdilation * (g.kh - 1) - g.vpadding,
+                        g.hdilation * (g.kw - 1) - g.hpadding, 1, 1, g.vdilation, g.hdilation);
+    if (rc != PYDTNN_HIP_OK) return rc;
+    if (gb.ho != g.h || gb.wo != g.w) return PYDTNN_HIP_ERR_INVALID;
+    return nhwc ? conv_fwd_nhwc(gb, ws, dy, dx, no_epilogue(), stream)
+                : conv_fwd_nchw(gb, ws, dy, dx, no_epilogue(), stream);
+}
+
+int geom_from_args(ConvGeom* g, long b, long c, long h, long w, long kn, long kh, long kw, long vpadding,
+                   long hpadding, long vstride, long hstride, long vdilation, long hdilation)
+{
+    const long lim = 1l << 30;
+    if (b >= lim || c >= lim || h >= lim || w >= lim || kn >= lim || kh >= lim || kw >= lim || vpadding >= lim ||
+        hpadding >= lim || vstride >= lim || hstride >= lim || vdilation >= lim || hdilation >= lim)
+        return PYDTNN_HIP_ERR_INVALID;
+    return make_conv_geom(g, (int)b, (int)c, (int)h, (int)w, (int)kn, (int)kh, (int)kw, (int)vpadding, (int)hpadding,
+                          (int)vstride, (int)hstride, (int)vdilation, (int)hdilation);
+}
+
+int sconv_gemm(int nhwc, char trans, const ConvGeom& g, const float* in1, const float* x, float* out,
+               const float* bias, const float* mean, const float* inv_std, const float* gamma, const float* beta,
+               bool relu, void* ws, size_t ws_bytes, hipStream_t stream)
+{
+    if (!in1 || !x || !out) return PYDTNN_HIP_ERR_INVALID;
+    if (trans == 'N') {
+        if (!bn_args_consistent(mean, inv_std, gamma, beta)) return PYDTNN_HIP_ERR_INVALID;
+        const ChanEpilogue chan = make_chan(bias, mean, inv_std, gamma, beta, relu ? 1 : 0);
+        return nhwc ? conv_fwd_nhwc(g, in1, x, out, chan, stream) : conv_fwd_nchw(g, in1, x, out, chan, stream);
+    }
+    if (trans == 'Y') {
+        if (bias || mean || inv_std || gamma || beta || relu) return PYDTNN_HIP_ERR_INVALID;
+        return nhwc ? conv_dw_nhwc(g, in1, x, nullptr, out, (float*)ws, ws_bytes, stream)
+                    : conv_dw_nchw(g, in1, x, nullptr, out, (float*)ws, ws_bytes, stream);
+    }
+    return PYDTNN_HIP_ERR_INVALID;
+}
+
+}  // namespace
+
+extern "C" {
+
+int pydtnn_hip_version(void) { return 10000 * 0 + 100 * 1 + 0; }
+
+const char* pydtnn_hip_status_string(int status)
+{
+    switch (status) {
+        case PYDTNN_HIP_OK: return "ok";
+        case PYDTNN_HIP_ERR_INVALID: return "invalid argument";
+        case PYDTNN_HIP_ERR_WORKSPACE: return "workspace missing or too small";
+        case PYDTNN_HIP_ERR_LAUNCH: return "HIP launch/runtime error";
+        case PYDTNN_HIP_ERR_UNSUPPORTED: return "extents not supported by the index arithmetic";
+        default: return "unknown status";
+    }
+}
+
+#define GEOM_ARGS b, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation
+
+int pydtnn_hip_im2col_nchw(const float* x, float* cols, int b, int c, int h, int w, int kh, int kw, int vpadding,
+                           int hpadding, int vstride, int hstride, int vdilation, int hdilation, void* stream)
+{
+    if (!x || !cols) return PYDTNN_HIP_ERR_INVALID;
+    ConvGeom g;
+    const int kn = 1;
+    const int rc = geom_from_args(&g, GEOM_ARGS);
+    return rc != PYDTNN_HIP_OK ? rc : launch_im2col_nchw(x, cols, g, as_stream(stream));
+}
+
+int pydtnn_hip_col2im_nchw(const float* cols, float* dx, int b, int c, int h, int w, int kh, int kw, int vpadding,
+                           int hpadding, int vstride, int hstride, int vdilation, int hdilation, void* stream)
+{
+    if (!dx || !cols) return PYDTNN_HIP_ERR_INVALID;
+    ConvGeom g;
+    const int kn = 1;
+    const int rc = geom_from_args(&g, GEOM_ARGS);
+    return rc != PYDTNN_HIP_OK ? rc : launch_col2im_nchw(cols, dx, g, as_stream(stream));
+}
+
+int pydtnn_hip_im2row_nhwc(const float* x, float* rows, int b, int h, int w, int c, int kh, int kw, int vpadding,
+                           int hpadding, int vstride, int hstride, int vdilation, int hdilation, void* stream)
+{
+    if (!x || !rows) return PYDTNN_HIP_ERR_INVALID;
+    ConvGeom g;
+    const int kn = 1;
+    const int rc = geom_from_args(&g, GEOM_ARGS);
+    return rc != PYDTNN_HIP_OK ? rc : launch_im2row_nhwc(x, rows, g, as_stream(stream));
+}
+
+int pydtnn_hip_row2im_nhwc(const float* rows, float* dx, int b, int h, int w, int c, int kh, int kw, int vpadding,
+                           int hpadding, int vstride, int hstride, int vdilation, int hdilation, void* stream)
+{
+    if (!dx || !rows) return PYDTNN_HIP_ERR_INVALID;
+    ConvGeom g;
+    const int kn = 1;
+    const int rc = geom_from_args(&g, GEOM_ARGS);
+    return rc != PYDTNN_HIP_OK ? rc : launch_row2im_nhwc(rows, dx, g, as_stream(stream));
+}
+
+// ---------------------------------------------------------------- GEMM
+size_t pydtnn_hip_sgemm_workspace_bytes(long m, long n, long k)
+{
+    if (m <= 0 || n <= 0 || k <= 0) return 0;
+    const TileSel sel = pick_tile(m, n);
+    const SplitPlan sp = plan_plain_split(tiles_of(sel, m, n), k, m * n);
+    return sp.splits > 1 ? (size_t)sp.splits * m * n * 4 : 0;
+}
+
+int pydtnn_hip_sgemm(int transa, int transb, long m, long n, long k, const float* a, long lda, const float* b,
+                     long ldb, float* c, long ldc, const float* bias, int relu, void* workspace,
+                     size_t workspace_bytes, void* stream)
+{
+    if (!a || !b || !c || m <= 0 || n <= 0 || k <= 0) return PYDTNN_HIP_ERR_INVALID;
+    const long lim = 1l << 31;
+    if (m >= lim || n >= lim || k >= lim) return PYDTNN_HIP_ERR_UNSUPPORTED;
+    if (lda < (transa ? m : k) || ldb < (transb ? k : n) || ldc < n) return PYDTNN_HIP_ERR_INVALID;
+    const TileSel sel = pick_tile(m, n);
+    const SplitPlan sp = plan_plain_split(tiles_of(sel, m, n), k, m * n);
+    const ChanEpilogue chan = make_chan(bias, nullptr, nullptr, nullptr, nullptr, relu);
+    float* dst = c;
+    long dst_ld = ldc;
+    ChanEpilogue gemm_chan = chan;
+    if (sp.splits > 1) {
+        if (!workspace || workspace_bytes < (size_t)sp.splits * m * n * 4) return PYDTNN_HIP_ERR_WORKSPACE;
+        dst = (float*)workspace;
+        dst_ld = n;
+        gemm_chan = no_epilogue();
+    }
+    const hipStream_t st = as_stream(stream);
+    int rc = PYDTNN_HIP_OK;
+    WITH_TILE(sel, {
+        const EpiPlain ep = epi_plain(dst, dst_ld, m * n, m, n, gemm_chan);
+        if (!transa && !transb)
+            rc = launch<T>(plain_k<T::BM, false>(a, lda, 0, m, 0), plain_mn<T::BN>(b, ldb, 0, n), ep, m, n, sp.si,
+                           sp.splits, st);
+        else if (!transa && transb)
+            rc = launch<T>(plain_k<T::BM, false>(a, lda, 0, m, 0), plain_k<T::BN, false>(b, ldb, 0, n, 0), ep, m, n,
+                           sp.si, sp.splits, st);
+        else if (transa && !transb)
+            rc = launch<T>(plain_mn<T::BM>(a, lda, 0, m), plain_mn<T::BN>(b, ldb, 0, n), ep, m, n, sp.si, sp.splits,
+                           st);
+        else
+            rc = launch<T>(plain_mn<T::BM>(a, lda, 0, m), plain_k<T::BN, false>(b, ldb, 0, n, 0), ep, m, n, sp.si,
+                           sp.splits, st);
+    })
+    if (rc != PYDTNN_HIP_OK || sp.splits == 1) return rc;
+    if (ldc != n) return PYDTNN_HIP_ERR_UNSUPPORTED;  // the split reduction writes a dense C
+    return launch_splitk_reduce((const float*)workspace, c, m, (int)n, m * n, sp.splits, 0, 0, chan, st);
+}
+
+// ---------------------------------------------------------------- convolution
+size_t pydtnn_hip_conv_workspace_bytes(int op, int nhwc, int b, int c, int h, int w, int kn, int kh, int kw,
+                                       int vpadding, int hpadding, int vstride, int hstride, int vdilation,
+                                       int hdilation)
+{
+    ConvGeom g;
+    if (geom_from_args(&g, GEOM_ARGS) != PYDTNN_HIP_OK) return 0;
+    switch (op) {
+        case PYDTNN_HIP_OP_DW: return (size_t)plan_dw(g, nhwc).splits * g.kn * g.k * 4;
+        case PYDTNN_HIP_OP_DX:
+            return dx_as_forward(g) ? (size_t)g.kn * g.k * 4 : (size_t)g.k * g.p * 4;
+        case PYDTNN_HIP_OP_DX_I2C: return (size_t)g.k * g.p * 4;
+        case PYDTNN_HIP_OP_DB: return bias_grad_workspace_floats(g.n, g.kn) * 4;
+        default: return 0;
+    }
+}
+
+int pydtnn_hip_sconvGemmNCHW(char trans, unsigned b, unsigned c, unsigned h, unsigned w, unsigned kn, unsigned kh,
+                             unsigned kw, unsigned vpadding, unsigned hpadding, unsigned vstride, unsigned hstride,
+                             unsigned vdilation, unsigned hdilation, const float* in1, const float* x, float* out,
+                             const float* bias_vector, const float* bn_running_mean, const float* bn_inv_std,
+                             const float* bn_gamma, const float* bn_beta, bool relu, void* workspace,
+                             size_t workspace_bytes, void* stream)
+{
+    ConvGeom g;
+    const int rc = geom_from_args(&g, GEOM_ARGS);
+    if (rc != PYDTNN_HIP_OK) return rc;
+    return sconv_gemm(0, trans, g, in1, x, out, bias_vector, bn_running_mean, bn_inv_std, bn_gamma, bn_beta, relu,
+                      workspace, workspace_bytes, as_stream(stream));
+}
+
+int pydtnn_hip_sconvGemmNHWC(char trans, unsigned b, unsigned h, unsigned w, unsigned c, unsigned kn, unsigned kh,
+                             unsigned kw, unsigned vpadding, unsigned hpadding, unsigned vstride, unsigned hstride,
+                             unsigned vdilation, unsigned hdilation, const float* in1, const float* x, float* out,
+                             const float* bias_vector, const float* bn_running_mean, const float* bn_inv_std,
+                             const float* bn_gamma, const float* bn_beta, bool relu, void* workspace,
+                             size_t workspace_bytes, void* stream)
+{
+    ConvGeom g;
+    const int rc = geom_from_args(&g, GEOM_ARGS);
+    if (rc != PYDTNN_HIP_OK) return rc;
+    return sconv_gemm(1, trans, g, in1, x, out, bias_vector, bn_running_mean, bn_inv_std, bn_gamma, bn_beta, relu,
+                      workspace, workspace_bytes, as_stream(stream));
+}
+
+int pydtnn_hip_sconvGemmNCHW_back(unsigned b, unsigned c, unsigned h, unsigned w, unsigned kn, unsigned kh,
+                                  unsigned kw, unsigned vstride, unsigned hstride, unsigned vpadding,
+                                  unsigned hpadding, unsigned vdilation, unsigned hdilation, const float* weights,
+                                  const float* dy, float* dx, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (!weights || !dy || !dx) return PYDTNN_HIP_ERR_INVALID;
+    ConvGeom g;
+    const int rc = geom_from_args(&g, GEOM_ARGS);
+    if (rc != PYDTNN_HIP_OK) return rc;
+    return conv_dx(g, 0, weights, dy, dx, (float*)workspace, workspace_bytes, as_stream(stream));
+}
+
+int pydtnn_hip_sconvGemmNHWC_back(unsigned b, unsigned h, unsigned w, unsigned c, unsigned kn, unsigned kh,
+                                  unsigned kw, unsigned vstride, unsigned hstride, unsigned vpadding,
+                                  unsigned hpadding, unsigned vdilation, unsigned hdilation, const float* weights,
+                                  const float* dy, float* dx, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (!weights || !dy || !dx) return PYDTNN_HIP_ERR_INVALID;
+    ConvGeom g;
+    const int rc = geom_from_args(&g, GEOM_ARGS);
+    if (rc != PYDTNN_HIP_OK) return rc;
+    return conv_dx(g, 1, weights, dy, dx, (float*)workspace, workspace_bytes, as_stream(stream));
+}
+
+// ---------------------------------------------------------------- explicit (i2c) GEMM steps
+int pydtnn_hip_conv_i2c_forward(int nhwc, int b, int c, int h, int w, int kn, int kh, int kw, int vpadding,
+                                int hpadding, int vstride, int hstride, int vdilation, int hdilation,
+                                const float* weights, const float* mat, float* y, const float* bias_vector,
+                                void* stream)
+{
+    if (!weights || !mat || !y) return PYDTNN_HIP_ERR_INVALID;
+    ConvGeom g;
+    int rc = geom_from_args(&g, GEOM_ARGS);
+    if (rc != PYDTNN_HIP_OK) return rc;
+    const ChanEpilogue chan = make_chan(bias_vector, nullptr, nullptr, nullptr, nullptr, 0);
+    const hipStream_t st = as_stream(stream);
+    if (!nhwc) {
+        const TileSel sel = pick_tile(g.kn, g.p);
+        WITH_TILE(sel, {
+            rc = launch<T>(plain_k<T::BM, false>(weights, g.k, 0, g.kn, 0), plain_mn<T::BN>(mat, g.p, 0, g.p),
+                           epi_nchw(y, g.kn, g.howo, g.p, chan), g.kn, g.p, no_split(g.k), 1, st);
+        })
+    } else {
+        const TileSel sel = pick_tile(g.p, g.kn);
+        WITH_TILE(sel, {
+            rc = launch<T>(plain_k<T::BM, false>(mat, g.k, 0, g.p, 0), plain_mn<T::BN>(weights, g.kn, 0, g.kn),
+                           epi_plain(y, g.kn, 0, g.p, g.kn, chan), g.p, g.kn, no_split(g.k), 1, st);
+        })
+    }
+    return rc;
+}
+
+int pydtnn_hip_conv_i2c_dw(int nhwc, int b, int c, int h, int w, int kn, int kh, int kw, int vpadding, int hpadding,
+                           int vstride, int hstride, int vdilation, int hdilation, const float* dy, const float* mat,
+                           float* dw, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (!dy || !mat || !dw) return PYDTNN_HIP_ERR_INVALID;
+    ConvGeom g;
+    const int rc = geom_from_args(&g, GEOM_ARGS);
+    if (rc != PYDTNN_HIP_OK) return rc;
+    return nhwc ? conv_dw_nhwc(g, dy, nullptr, mat, dw, (float*)workspace, workspace_bytes, as_stream(stream))
+                : conv_dw_nchw(g, dy, nullptr, mat, dw, (float*)workspace, workspace_bytes, as_stream(stream));
+}
+
+int pydtnn_hip_conv_i2c_dx(int nhwc, int b, int c, int h, int w, int kn, int kh, int kw, int vpadding, int hpadding,
+                           int vstride, int hstride, int vdilation, int hdilation, const float* weights,
+                           const float* dy, float* dx, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (!weights || !dy || !dx) return PYDTNN_HIP_ERR_INVALID;
+    ConvGeom g;
+    const int rc = geom_from_args(&g, GEOM_ARGS);
+    if (rc != PYDTNN_HIP_OK) return rc;
+    return conv_dx_i2c(g, nhwc, weights, dy, dx, (float*)workspace, workspace_bytes, as_stream(stream));
+}
+
+// ---------------------------------------------------------------- elementwise and friends
+int pydtnn_hip_chan_eltwise(const float* x, const float* residual, float* y, long total, int inner, int channels,
+                            const float* bias, const float* bn_running_mean, const float* bn_inv_std,
+                            const float* bn_gamma, const float* bn_beta, int relu, void* stream)
+{
+    if (!x || !y) return PYDTNN_HIP_ERR_INVALID;
+    if (!bn_args_consistent(bn_running_mean, bn_inv_std, bn_gamma, bn_beta)) return PYDTNN_HIP_ERR_INVALID;
+    return launch_chan_eltwise(x, residual, y, total, inner, channels,
+                               make_chan(bias, bn_running_mean, bn_inv_std, bn_gamma, bn_beta, relu),
+                               as_stream(stream));
+}
+
+int pydtnn_hip_relu_fwd(const float* x, float* y, int8_t* mask, long total, void* stream)
+{
+    if (!x || !y) return PYDTNN_HIP_ERR_INVALID;
+    return launch_relu_fwd(x, y, mask, total, as_stream(stream));
+}
+
+int pydtnn_hip_relu_bwd(const float* dy, const int8_t* mask, float* dx, long total, void* stream)
+{
+    if (!dy || !mask || !dx) return PYDTNN_HIP_ERR_INVALID;
+    return launch_relu_bwd(dy, mask, dx, total, as_stream(stream));
+}
+
+int pydtnn_hip_bias_grad(const float* dy, float* db, long outer, int channels, int inner, void* workspace,
+                         size_t workspace_bytes, void* stream)
+{
+    if (!dy || !db) return PYDTNN_HIP_ERR_INVALID;
+    if (!workspace || workspace_bytes < bias_grad_workspace_floats(outer, channels) * 4)
+        return PYDTNN_HIP_ERR_WORKSPACE;
+    return launch_bias_grad(dy, db, outer, channels, inner, (float*)workspace, as_stream(stream));
+}
+
+int pydtnn_hip_max_pool_2d_fwd_nchw(const float* x, float* y, int32_t* idx_max, int b, int c, int h, int w, int kh,
+                                    int kw, int vpadding, int hpadding, int vstride, int hstride, int vdilation,
+                                    int hdilation, void* stream)
+{
+    if (!x || !y || !idx_max) return PYDTNN_HIP_ERR_INVALID;
+    ConvGeom g;
+    const int kn = 1;
+    const int rc = geom_from_args(&g, GEOM_ARGS);
+    return rc != PYDTNN_HIP_OK ? rc : launch_max_pool_fwd_nchw(x, y, idx_max, g, as_stream(stream));
+}
+
+int pydtnn_hip_max_pool_2d_bwd_nchw(const float* dy, const int32_t* idx_max, float* dx, int b, int c, int h, int w,
+                                    int kh, int kw, int vpadding, int hpadding, int vstride, int hstride,
+                                    int vdilation, int hdilation, void* stream)
+{
+    if (!dy || !dx || !idx_max) return PYDTNN_HIP_ERR_INVALID;
+    ConvGeom g;
+    const int kn = 1;
+    const int rc = geom_from_args(&g, GEOM_ARGS);
+    return rc != PYDTNN_HIP_OK ? rc : launch_max_pool_bwd_nchw(dy, idx_max, dx, g, as_stream(stream));
+}
+
+int pydtnn_hip_sgd_momentum(float* w, const float* dw, float* velocity, long total, float lr, float momentum,
+                            float decay, int nesterov, void* stream)
+{
+    if (!w || !dw || !velocity) return PYDTNN_HIP_ERR_INVALID;
+    return launch_sgd_momentum(w, dw, velocity, total, lr, momentum, decay, nesterov, as_stream(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,402 @@
+// HBM-bound helper kernels around the GEMMs: stand-alone bias / BatchNorm-inference / ReLU /
+// residual epilogue, ReLU with mask, bias gradient, split-K reduction, filter re-layouts,
+// MaxPool2D (NCHW) and the SGD-momentum update.  Each is a single streaming pass with lanes on
+// the contiguous axis; algorithmic bytes are stated at each launcher.
+#include "common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+inline unsigned blocks_for(long total, int per_block = kThreads)
+{
+    return (unsigned)((total + per_block - 1) / per_block);
+}
+
+// ---------------------------------------------------------------- channel-wise epilogue
+// y[idx] = epilogue(ch, x[idx] (+ residual[idx])), ch = (idx / inner) % channels.
+// inner = ho*wo for NCHW tensors, 1 for NHWC tensors and 2-D (rows, C) matrices.
+// Order: residual add first (pydtnn/cython_modules/eltw_sum_cython.pyx:25-36 is a separate,
+// earlier layer in the reference), then bias -> BN -> ReLU as in chan_epilogue_apply.
+__global__ void __launch_bounds__(kThreads) chan_eltwise_kernel(const float* __restrict__ x,
+                                                               const float* __restrict__ residual,
+                                                               float* __restrict__ y, long total, int inner,
+                                                               int channels, ChanEpilogue epi)
+{
+    const long idx = (long)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= total) return;
+    const int ch = (int)((idx / inner) % channels);
+    float v = x[idx];
+    if (residual) v += residual[idx];
+    y[idx] = chan_epilogue_apply(epi, ch, v);
+}
+
+// Four consecutive elements per thread; valid when either all four share a channel
+// (inner % 4 == 0) or they are four consecutive channels (inner == 1, channels % 4 == 0).
+__global__ void __launch_bounds__(kThreads) chan_eltwise_vec4_kernel(const float4* __restrict__ x,
+                                                                    const float4* __restrict__ residual,
+                                                                    float4* __restrict__ y, long total4, int inner,
+                                                                    int channels, ChanEpilogue epi)
+{
+    const long i4 = (long)blockIdx.x * kThreads + threadIdx.x;
+    if (i4 >= total4) return;
+    const long idx = i4 * 4;
+    const int ch0 = (int)((idx / inner) % channels);
+    const int step = inner == 1 ? 1 : 0;
+    float4 v = x[i4];
+    if (residual) {
+        const float4 r = residual[i4];
+        v.x += r.x; v.y += r.y; v.z += r.z; v.w += r.w;
+    }
+    v.x = chan_epilogue_apply(epi, ch0, v.x);
+    v.y = chan_epilogue_apply(epi, ch0 + step, v.y);
+    v.z = chan_epilogue_apply(epi, ch0 + 2 * step, v.z);
+    v.w = chan_epilogue_apply(epi, ch0 + 3 * step, v.w);
+    y[i4] = v;
+}
+
+// ---------------------------------------------------------------- ReLU with mask
+// pydtnn/cython_modules/relu_cython.pyx:52-59 (strict x > 0); pydtnn/backends/cpu/activations/relu_cpu.py:38-40.
+__global__ void __launch_bounds__(kThreads) relu_fwd_kernel(const float* __restrict__ x, float* __restrict__ y,
+                                                           int8_t* __restrict__ mask, long total)
+{
+    const long idx = (long)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= total) return;
+    const float v = x[idx];
+    const bool pos = v > 0.0f;
+    y[idx] = pos ? v : 0.0f;
+    if (mask) mask[idx] = pos ? 1 : 0;
+}
+
+__global__ void __launch_bounds__(kThreads) relu_bwd_kernel(const float* __restrict__ dy,
+                                                           const int8_t* __restrict__ mask,
+                                                           float* __restrict__ dx, long total)
+{
+    const long idx = (long)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= total) return;
+    dx[idx] = dy[idx] * (float)mask[idx];
+}
+
+// ---------------------------------------------------------------- bias gradient
+// db[c] = sum over batch and pixels of dy (pydtnn/backends/cpu/layers/conv_2d_cpu.py:463 NCHW, :377 NHWC;
+// fc_cpu.py:70).  Two deterministic stages: per-(channel, slice) partial sums, then a sum over slices.
+__device__ __forceinline__ float block_sum(float v)
+{
+    __shared__ float red[kThreads / 64];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    float s = 0.0f;
+    if (threadIdx.x == 0)
+        for (int i = 0; i < kThreads / 64; ++i) s += red[i];
+    return s;  // valid on thread 0
+}
+
+// NCHW: grid (C, S); slice s covers images [s*per, (s+1)*per).
+__global__ void __launch_bounds__(kThreads) bias_grad_nchw_stage1(const float* __restrict__ dy,
+                                                                 float* __restrict__ partial, int n, int c,
+                                                                 int hw, int per)
+{
+    const int ch = blockIdx.x, s = blockIdx.y;
+    const int n0 = s * per, n1 = min(n, n0 + per);
+    float acc = 0.0f;
+    for (int nn = n0; nn < n1; ++nn) {
+        const float* plane = dy + ((long)nn * c + ch) * hw;
+        for (int i = threadIdx.x; i < hw; i += kThreads) acc += plane[i];
+    }
+    const float tot = block_sum(acc);
+    if (threadIdx.x == 0) partial[(long)s * c + ch] = tot;
+}
+
+// (rows, C) matrix: grid (S, ceil(C/64)); block = 64 channels x 4 row lanes.
+__global__ void __launch_bounds__(kThreads) bias_grad_rows_stage1(const float* __restrict__ dy,
+                                                                 float* __restrict__ partial, long rows, int c,
+                                                                 long per)
+{
+    __shared__ float red[4][64];
+    const int cl = threadIdx.x & 63, rl = threadIdx.x >> 6;
+    const int ch = blockIdx.y * 64 + cl;
+    const long r0 = (long)blockIdx.x * per;
+    const long r1 = r0 + per < rows ? r0 + per : rows;
+    float acc = 0.0f;
+    if (ch < c)
+        for (long r = r0 + rl; r < r1; r += 4) acc += dy[r * c + ch];
+    red[rl][cl] = acc;
+    __syncthreads();
+    if (rl == 0 && ch < c) partial[(long)blockIdx.x * c + ch] = (red[0][cl] + red[1][cl]) + (red[2][cl] + red[3][cl]);
+}
+
+__global__ void __launch_bounds__(kThreads) bias_grad_stage2(const float* __restrict__ partial,
+                                                            float* __restrict__ db, int c, int slices)
+{
+    const int ch = blockIdx.x * kThreads + threadIdx.x;
+    if (ch >= c) return;
+    float acc = 0.0f;
+    for (int s = 0; s < slices; ++s) acc += partial[(long)s * c + ch];
+    db[ch] = acc;
+}
+
+// ---------------------------------------------------------------- split-K reduction
+// out[map(r, col)] = epilogue(col, sum_s partial[s*stride + r*ncols + col]).
+// perm_c > 0 re-orders rows from the kernels' internal (i, j, c) order to the reference's
+// (c, i, j) weight rows: r = ij*perm_c + c  ->  c*khw + ij.
+__global__ void __launch_bounds__(kThreads) splitk_reduce_kernel(const float* __restrict__ partial,
+                                                                float* __restrict__ out, long total, long stride,
+                                                                int slices, int ncols, int perm_c, int khw,
+                                                                ChanEpilogue epi)
+{
+    const long idx = (long)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= total) return;
+    float acc = 0.0f;
+    for (int s = 0; s < slices; ++s) acc += partial[(long)s * stride + idx];
+    const int col = (int)(idx % ncols);
+    long r = idx / ncols;
+    if (perm_c > 0) {
+        const long ij = r / perm_c;
+        const long cc = r - ij * perm_c;
+        r = cc * khw + ij;
+    }
+    out[r * ncols + col] = chan_epilogue_apply(epi, col, acc);
+}
+
+// ---------------------------------------------------------------- filter re-layouts for dX
+// Stride-1 dX is a forward convolution of dy with the spatially flipped, channel-swapped filter.
+// NCHW: wf[c][co][i][j] = w[co][c][kh-1-i][kw-1-j]
+__global__ void __launch_bounds__(kThreads) flip_filter_nchw_kernel(const float* __restrict__ w,
+                                                                   float* __restrict__ wf, int kn, int c, int kh,
+                                                                   int kw)
+{
+    const long idx = (long)blockIdx.x * kThreads + threadIdx.x;
+    const long total = (long)kn * c * kh * kw;
+    if (idx >= total) return;
+    const int j = (int)(idx % kw);
+    long t = idx / kw;
+    const int i = (int)(t % kh);
+    t /= kh;
+    const int co = (int)(t % kn);
+    const int cc = (int)(t / kn);
+    wf[idx] = w[(((long)co * c + cc) * kh + (kh - 1 - i)) * kw + (kw - 1 - j)];
+}
+
+// NHWC: wf[co][i][j][c] = w[c][kh-1-i][kw-1-j][co]
+__global__ void __launch_bounds__(kThreads) flip_filter_nhwc_kernel(const float* __restrict__ w,
+                                                                   float* __restrict__ wf, int kn, int c, int kh,
+                                                                   int kw)
+{
+    const long idx = (long)blockIdx.x * kThreads + threadIdx.x;
+    const long total = (long)kn * c * kh * kw;
+    if (idx >= total) return;
+    const int cc = (int)(idx % c);
+    long t = idx / c;
+    const int j = (int)(t % kw);
+    t /= kw;
+    const int i = (int)(t % kh);
+    const int co = (int)(t / kh);
+    wf[idx] = w[(((long)cc * kh + (kh - 1 - i)) * kw + (kw - 1 - j)) * kn + co];
+}
+
+// ---------------------------------------------------------------- MaxPool2D NCHW
+// Forward: pydtnn/cython_modules/max_pool_2d_nchw_cython.pyx:86-110 (first maximum wins, index ii*kw+jj).
+__global__ void __launch_bounds__(kThreads) max_pool_fwd_nchw_kernel(const float* __restrict__ x,
+                                                                    float* __restrict__ y,
+                                                                    int32_t* __restrict__ idx_max, ConvGeom g)
+{
+    const long idx = (long)blockIdx.x * kThreads + threadIdx.x;
+    const long total = (long)g.n * g.c * g.howo;
+    if (idx >= total) return;
+    const int ox = (int)(idx % g.wo);
+    long t = idx / g.wo;
+    const int oy = (int)(t % g.ho);
+    const long plane = t / g.ho;  // n*c + c
+    const float* src = x + plane * g.h * g.w;
+    float maxval = -3.402823466e+38f;
+    int best = 0;
+    for (int ii = 0; ii < g.kh; ++ii) {
+        const int x_x = g.vstride * oy + g.vdilation * ii - g.vpadding;
+        if ((unsigned)x_x >= (unsigned)g.h) continue;
+        for (int jj = 0; jj < g.kw; ++jj) {
+            const int x_y = g.hstride * ox + g.hdilation * jj - g.hpadding;
+            if ((unsigned)x_y >= (unsigned)g.w) continue;
+            const float val = src[x_x * g.w + x_y];
+            if (val > maxval) { maxval = val; best = ii * g.kw + jj; }
+        }
+    }
+    y[idx] = maxval;
+    idx_max[idx] = best;
+}
+
+// Backward in gather form: one thread per dx element sums dy of every window whose recorded
+// maximum decodes to this element.  The decode is the reference's own
+// (ii = idx / kh, jj = idx % kw, max_pool_2d_nchw_cython.pyx:204-205).  Windows are visited in
+// ascending (oy, ox), the order of the reference's scatter loop.
+__global__ void __launch_bounds__(kThreads) max_pool_bwd_nchw_kernel(const float* __restrict__ dy,
+                                                                    const int32_t* __restrict__ idx_max,
+                                                                    float* __restrict__ dx, ConvGeom g)
+{
+    const long idx = (long)blockIdx.x * kThreads + threadIdx.x;
+    const long total = (long)g.n * g.c * g.h * g.w;
+    if (idx >= total) return;
+    const int ww = (int)(idx % g.w);
+    long t = idx / g.w;
+    const int hh = (int)(t % g.h);
+    const long plane = t / g.h;
+    const float* gy = dy + plane * g.howo;
+    const int32_t* gi = idx_max + plane * g.howo;
+    float acc = 0.0f;
+    for (int ii = g.kh - 1; ii >= 0; --ii) {
+        const int ty = hh + g.vpadding - g.vdilation * ii;
+        if (ty < 0) continue;
+        const int oy = ty / g.vstride;
+        if (oy * g.vstride != ty || oy >= g.ho) continue;
+        for (int jj = g.kw - 1; jj >= 0; --jj) {
+            const int tx = ww + g.hpadding - g.hdilation * jj;
+            if (tx < 0) continue;
+            const int ox = tx / g.hstride;
+            if (ox * g.hstride != tx || ox >= g.wo) continue;
+            const int rec = gi[oy * g.wo + ox];
+            if (rec / g.kh == ii && rec % g.kw == jj) acc += gy[oy * g.wo + ox];
+        }
+    }
+    dx[idx] = acc;
+}
+
+// ---------------------------------------------------------------- SGD with momentum
+// pydtnn/backends/cpu/optimizers/sgd_cpu.py:28-41
+__global__ void __launch_bounds__(kThreads) sgd_momentum_kernel(float* __restrict__ w, const float* __restrict__ dw,
+                                                               float* __restrict__ velocity, long total, float lr,
+                                                               float momentum, float decay, int nesterov)
+{
+    const long idx = (long)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= total) return;
+    const float g = dw[idx];
+    const float v = momentum * velocity[idx] + g;
+    const float wv = w[idx];
+    const float upd = nesterov ? (decay * wv + g + momentum * v) : (decay * wv + v);
+    w[idx] = wv - lr * upd;
+    velocity[idx] = v;
+}
+
+}  // namespace
+
+// Algorithmic bytes: 2 * 4 * total (+ 4 * total when a residual is read).
+int launch_chan_eltwise(const float* x, const float* residual, float* y, long total, int inner, int channels,
+                        const ChanEpilogue& epi, hipStream_t stream)
+{
+    if (total <= 0 || inner <= 0 || channels <= 0) return PYDTNN_HIP_ERR_INVALID;
+    const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y) |
+                           reinterpret_cast<uintptr_t>(residual)) & 15) == 0;
+    const bool vec = aligned && total % 4 == 0 && (inner % 4 == 0 || (inner == 1 && channels % 4 == 0));
+    if (vec)
+        hipLaunchKernelGGL(chan_eltwise_vec4_kernel, dim3(blocks_for(total / 4)), dim3(kThreads), 0, stream,
+                           reinterpret_cast<const float4*>(x), reinterpret_cast<const float4*>(residual),
+                           reinterpret_cast<float4*>(y), total / 4, inner, channels, epi);
+    else
+        hipLaunchKernelGGL(chan_eltwise_kernel, dim3(blocks_for(total)), dim3(kThreads), 0, stream, x, residual, y,
+                           total, inner, channels, epi);
+    HIP_RETURN_IF_LAUNCH_FAILED();
+    return PYDTNN_HIP_OK;
+}
+
+// Algorithmic bytes: 4 * total read + 4 * total + total written.
+int launch_relu_fwd(const float* x, float* y, int8_t* mask, long total, hipStream_t stream)
+{
+    if (total <= 0) return PYDTNN_HIP_ERR_INVALID;
+    hipLaunchKernelGGL(relu_fwd_kernel, dim3(blocks_for(total)), dim3(kThreads), 0, stream, x, y, mask, total);
+    HIP_RETURN_IF_LAUNCH_FAILED();
+    return PYDTNN_HIP_OK;
+}
+
+int launch_relu_bwd(const float* dy, const int8_t* mask, float* dx, long total, hipStream_t stream)
+{
+    if (total <= 0) return PYDTNN_HIP_ERR_INVALID;
+    hipLaunchKernelGGL(relu_bwd_kernel, dim3(blocks_for(total)), dim3(kThreads), 0, stream, dy, mask, dx, total);
+    HIP_RETURN_IF_LAUNCH_FAILED();
+    return PYDTNN_HIP_OK;
+}
+
+size_t bias_grad_workspace_floats(long outer, int channels)
+{
+    (void)outer;
+    return (size_t)64 * channels;
+}
+
+// inner > 1: dy is (outer, channels, inner) [NCHW]; inner == 1: dy is (outer, channels) rows.
+// Algorithmic bytes: 4 * outer * channels * inner read.
+int launch_bias_grad(const float* dy, float* db, long outer, int channels, int inner, float* workspace,
+                     hipStream_t stream)
+{
+    if (outer <= 0 || channels <= 0 || inner <= 0 || !workspace) return PYDTNN_HIP_ERR_INVALID;
+    int slices;
+    if (inner > 1) {
+        const int n = (int)outer;
+        slices = n < 64 ? n : 64;
+        const int per = (n + slices - 1) / slices;
+        slices = (n + per - 1) / per;
+        hipLaunchKernelGGL(bias_grad_nchw_stage1, dim3(channels, slices), dim3(kThreads), 0, stream, dy, workspace, n,
+                           channels, inner, per);
+    } else {
+        slices = outer < 64 * 4 ? (int)((outer + 3) / 4) : 64;
+        const long per = (outer + slices - 1) / slices;
+        slices = (int)((outer + per - 1) / per);
+        hipLaunchKernelGGL(bias_grad_rows_stage1, dim3(slices, (channels + 63) / 64), dim3(kThreads), 0, stream, dy,
+                           workspace, outer, channels, per);
+    }
+    HIP_RETURN_IF_LAUNCH_FAILED();
+    hipLaunchKernelGGL(bias_grad_stage2, dim3(blocks_for(channels)), dim3(kThreads), 0, stream, workspace, db,
+                       channels, slices);
+    HIP_RETURN_IF_LAUNCH_FAILED();
+    return PYDTNN_HIP_OK;
+}
+
+int launch_splitk_reduce(const float* partial, float* out, long rows, int ncols, long stride, int slices, int perm_c,
+                         int khw, const ChanEpilogue& epi, hipStream_t stream)
+{
+    const long total = rows * ncols;
+    if (total <= 0 || slices <= 0) return PYDTNN_HIP_ERR_INVALID;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3(blocks_for(total)), dim3(kThreads), 0, stream, partial, out, total,
+                       stride, slices, ncols, perm_c, khw, epi);
+    HIP_RETURN_IF_LAUNCH_FAILED();
+    return PYDTNN_HIP_OK;
+}
+
+int launch_flip_filter(const float* w, float* wf, int nhwc, int kn, int c, int kh, int kw, hipStream_t stream)
+{
+    const long total = (long)kn * c * kh * kw;
+    if (nhwc)
+        hipLaunchKernelGGL(flip_filter_nhwc_kernel, dim3(blocks_for(total)), dim3(kThreads), 0, stream, w, wf, kn, c,
+                           kh, kw);
+    else
+        hipLaunchKernelGGL(flip_filter_nchw_kernel, dim3(blocks_for(total)), dim3(kThreads), 0, stream, w, wf, kn, c,
+                           kh, kw);
+    HIP_RETURN_IF_LAUNCH_FAILED();
+    return PYDTNN_HIP_OK;
+}
+
+int launch_max_pool_fwd_nchw(const float* x, float* y, int32_t* idx_max, const ConvGeom& g, hipStream_t stream)
+{
+    const long total = (long)g.n * g.c * g.howo;
+    hipLaunchKernelGGL(max_pool_fwd_nchw_kernel, dim3(blocks_for(total)), dim3(kThreads), 0, stream, x, y, idx_max, g);
+    HIP_RETURN_IF_LAUNCH_FAILED();
+    return PYDTNN_HIP_OK;
+}
+
+int launch_max_pool_bwd_nchw(const float* dy, const int32_t* idx_max, float* dx, const ConvGeom& g,
+                             hipStream_t stream)
+{
+    const long total = (long)g.n * g.c * g.h * g.w;
+    hipLaunchKernelGGL(max_pool_bwd_nchw_kernel, dim3(blocks_for(total)), dim3(kThreads), 0, stream, dy, idx_max, dx,
+                       g);
+    HIP_RETURN_IF_LAUNCH_FAILED();
+    return PYDTNN_HIP_OK;
+}
+
+int launch_sgd_momentum(float* w, const float* dw, float* velocity, long total, float lr, float momentum, float decay,
+                        int nesterov, hipStream_t stream)
+{
+    if (total <= 0) return PYDTNN_HIP_ERR_INVALID;
+    hipLaunchKernelGGL(sgd_momentum_kernel, dim3(blocks_for(total)), dim3(kThreads), 0, stream, w, dw, velocity, total,
+                       lr, momentum, decay, nesterov);
+    HIP_RETURN_IF_LAUNCH_FAILED();
+    return PYDTNN_HIP_OK;
+}

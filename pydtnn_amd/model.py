@@ -1,0 +1,219 @@
+"""Minimal ``Model``: what the conv-as-GEMM layers need from pydtnn/model.py and nothing else.
+
+Kept from the reference: keyword flags readable as attributes (``tensor_format``, ``dtype``,
+``batch_size``, ``enable_conv_gemm``, ``enable_fused_bn_relu`` / ``_conv_relu`` / ``_conv_bn`` /
+``_conv_bn_relu``; pydtnn/parser.py:64-79, :131), ``mode``, ``matmul``, a no-op ``tracer``,
+``add`` with ``need_dx = layer.id > 1`` (pydtnn/model.py:268-283), the layer-fusion rewrite
+(pydtnn/model.py:294-349) and the single-process forward / backward / update loop
+(pydtnn/model.py:450-492, :623-644).  Datasets, MPI, checkpoints, schedulers and the CLI are not
+part of this build.
+"""
+import torch
+
+from . import layers as L
+from . import ops
+from .layers import EVALUATE_MODE, TRAIN_MODE, UNSPECIFIED_MODE
+from .utils import PYDTNN_TENSOR_FORMAT_NCHW, PYDTNN_TENSOR_FORMAT_NHWC
+
+
+def _layer_id_generator():
+    current_layer_id = 0
+    while True:
+        yield current_layer_id
+        current_layer_id += 1
+
+
+class _NullTracer:
+    """Same call surface as pydtnn/tracers/tracer.py:72-90 with tracing disabled (rocprofv3 is the tracer here)."""
+
+    def emit_event(self, evt_type, evt_val):
+        pass
+
+    def emit_nevent(self, evt_types, evt_vals):
+        pass
+
+
+_DEFAULTS = dict(
+    batch_size=64,
+    tensor_format="AUTO",
+    enable_conv_gemm=True,   # the implicit-GEMM path is always available on this backend
+    enable_conv_winograd=False,
+    enable_best_of=False,
+    enable_memory_cache=False,
+    enable_fused_bn_relu=False,
+    enable_fused_conv_relu=False,
+    enable_fused_conv_bn=False,
+    enable_fused_conv_bn_relu=False,
+)
+
+
+class Model:
+
+    def __init__(self, dtype=torch.float32, **kwargs):
+        unknown = set(kwargs) - set(_DEFAULTS)
+        if unknown:
+            raise TypeError(f"unknown Model flags: {sorted(unknown)}")
+        self.kwargs = dict(_DEFAULTS)
+        self.kwargs.update(kwargs)
+        if isinstance(dtype, str):
+            dtype = {"float32": torch.float32, "float64": torch.float64}[dtype]
+        if dtype != torch.float32:
+            raise ValueError("only float32 models run on the MI355X kernels")
+        self.dtype = dtype
+        self.tracer = _NullTracer()
+        self.layers = []
+        self.layer_id = _layer_id_generator()
+        self.matmul = ops.matmul
+        self.nparams = 0
+        self.rank, self.nprocs, self.comm = 0, 1, None
+        self.mode = UNSPECIFIED_MODE
+        # pydtnn/model.py:207-215: AUTO resolves to NCHW on a GPU backend
+        fmt = self.kwargs["tensor_format"]
+        self.tensor_format = PYDTNN_TENSOR_FORMAT_NHWC if fmt == "NHWC" else PYDTNN_TENSOR_FORMAT_NCHW
+        self.batch_size = self.kwargs["batch_size"]
+        self._fused = False
+
+    def __getattr__(self, item):
+        try:
+            return self.__dict__["kwargs"][item]
+        except KeyError:
+            raise AttributeError(f"'Model' object has no attribute '{item}'") from None
+
+    # ------------------------------------------------------------------ construction
+    def add(self, layer):
+        layer.set_model(self)
+        need_dx = layer.id > 1
+        prev_shape = self.layers[-1].shape if layer.id > 0 else ()
+        layer.initialize(prev_shape, need_dx)
+        self.nparams += layer.nparams
+        self.layers.append(layer)
+        if layer.act:
+            self.add(layer.act())
+
+    def get_all_layers(self, from_layers=None):
+        if from_layers is None:
+            from_layers = self.layers
+        out = []
+        for layer in from_layers:
+            out.append(layer)
+            out += self.get_all_layers(layer.children)
+        return out
+
+    # ------------------------------------------------------------------ fusion (pydtnn/model.py:294-349)
+    def apply_layer_fusion(self, bn_relu=None, conv_relu=None, conv_bn=None, conv_bn_relu=None):
+        """Rewrites [Conv2D, BatchNormalization, Relu] runs into fused inference layers.  Flags default to
+        the model's ``enable_fused_*`` settings.  As in the reference a convolution is only fused when its
+        installed forward is one the fused class implements (the ``cg`` variants, never ``i2c``)."""
+        bn_relu = self.enable_fused_bn_relu if bn_relu is None else bn_relu
+        conv_relu = self.enable_fused_conv_relu if conv_relu is None else conv_relu
+        conv_bn = self.enable_fused_conv_bn if conv_bn is None else conv_bn
+        conv_bn_relu = self.enable_fused_conv_bn_relu if conv_bn_relu is None else conv_bn_relu
+
+        def fusable(conv, cls):
+            # pydtnn/model.py:313, :330: the convolution's installed forward must be one the fused class has
+            name = conv.forward.__name__
+            return name.endswith("_cg") and hasattr(cls, name)
+
+        def fuse(layers):
+            fused = []
+            for i, curr in enumerate(layers):
+                if curr.is_block_layer:
+                    for j, p in enumerate(curr.paths):
+                        curr.paths[j] = fuse(p)
+                elif conv_bn_relu and len(fused) > 1 and curr.canonical_name == "Relu" and \
+                        fused[-1].canonical_name == "BatchNormalization" and fused[-2].canonical_name == "Conv2D":
+                    cls = L.Conv2DBatchNormalizationRelu
+                    if fusable(fused[-2], cls):
+                        bn_layer = fused.pop()
+                        cv_layer = fused.pop()
+                        curr = cls(from_parent=cv_layer, from_parent2=bn_layer)
+                        curr.initialize(from_parent_dict=cv_layer.__dict__)
+                elif (conv_relu or conv_bn) and len(fused) > 0 and \
+                        (curr.canonical_name == "Relu" or curr.canonical_name == "BatchNormalization") and \
+                        fused[-1].canonical_name == "Conv2D" and \
+                        not (conv_bn_relu and i + 1 < len(layers) and layers[i + 1].canonical_name == "Relu"):
+                    # as in the reference, either flag enables both the conv+ReLU and the conv+BN rewrite
+                    cls = L.Conv2DRelu if curr.canonical_name == "Relu" else L.Conv2DBatchNormalization
+                    if fusable(fused[-1], cls):
+                        prev = fused.pop()
+                        curr = cls(from_parent=prev, from_parent2=curr)
+                        curr.initialize(from_parent_dict=prev.__dict__)
+                elif bn_relu and len(fused) > 0 and curr.canonical_name == "Relu" and \
+                        fused[-1].canonical_name == "BatchNormalization":
+                    prev = fused.pop()
+                    curr = L.BatchNormalizationRelu(from_parent=prev)
+                fused.append(curr)
+            return fused
+
+        if bn_relu or conv_relu or conv_bn or conv_bn_relu:
+            self.layers = fuse(self.layers)
+            self._fused = True
+
+    # ------------------------------------------------------------------ loops
+    def train_batch(self, x, y_targ, loss_func, optimizer, global_batch_size=None):
+        """One pass of pydtnn/model.py:450-492 (blocking path, one process): forward, loss, backward, update."""
+        if self._fused:
+            raise RuntimeError("Fused layers cannot be used in training mode!")
+        self.mode = TRAIN_MODE
+        if global_batch_size is None:
+            global_batch_size = x.shape[0]
+        for i in range(1, len(self.layers)):
+            x = self.layers[i].forward(x)
+        loss, dx = loss_func(x, y_targ, global_batch_size)
+        for i in range(len(self.layers) - 1, 0, -1):
+            dx = self.layers[i].backward(dx)
+        for i in range(len(self.layers) - 1, 0, -1):
+            self.layers[i].reduce_weights_sync()
+            self.layers[i].update_weights(optimizer)
+        return loss
+
+    def evaluate_batch(self, x):
+        """Forward pass of pydtnn/model.py:623-644."""
+        self.mode = EVALUATE_MODE
+        for i in range(1, len(self.layers)):
+            x = self.layers[i].forward(x)
+        return x
+
+    def evaluate_dataset_batch(self, x):
+        """pydtnn/model.py:653-667: the fusion pass runs once, on the first evaluation."""
+        if not self._fused:
+            self.apply_layer_fusion()
+        return self.evaluate_batch(x)
+
+
+# --------------------------------------------------------------------------- loss and optimizer
+class CategoricalCrossEntropy:
+    """pydtnn/backends/cpu/losses/categorical_cross_entropy_cpu.py:26-35 with torch ops on the GPU
+    (a (batch, classes) matrix: a few kilobytes).  Returns (loss tensor, dx)."""
+
+    def __init__(self, eps=1e-8):
+        self.eps = eps
+
+    def __call__(self, y_pred, y_targ, global_batch_size):
+        y_pred = torch.clamp(y_pred, min=self.eps, max=1 - self.eps)
+        b_range = torch.arange(y_pred.shape[0], device=y_pred.device)
+        amax = torch.argmax(y_targ, dim=1)
+        loss = -torch.sum(torch.log(y_pred[b_range, amax])) / y_pred.shape[0]
+        dx = y_targ.clone()
+        dx[b_range, amax] /= (-y_pred[b_range, amax] * global_batch_size)
+        return loss, dx
+
+
+class SGD:
+    """pydtnn/optimizers/sgd.py + pydtnn/backends/cpu/optimizers/sgd_cpu.py:26-41"""
+
+    def __init__(self, learning_rate=1e-2, momentum=0.9, nesterov=False, decay=0.0):
+        self.learning_rate = learning_rate
+        self.momentum = momentum
+        self.nesterov = nesterov
+        self.decay = decay
+
+    def update(self, layer):
+        for w_, dw_ in layer.grad_vars.items():
+            w, dw = getattr(layer, w_), getattr(layer, dw_)
+            velocity = getattr(layer, "velocity_%s" % w_, None)
+            if velocity is None:
+                velocity = torch.zeros_like(w)
+                setattr(layer, "velocity_%s" % w_, velocity)
+            ops.sgd_momentum(w, dw.reshape(w.shape).contiguous(), velocity, self.learning_rate, self.momentum,
+                             self.decay, self.nesterov)

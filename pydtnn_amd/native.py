@@ -1,0 +1,133 @@
+"""ctypes binding of libpydtnn_hip.so (C ABI declared in include/pydtnn_hip.h).
+
+PyTorch-ROCm is used only as the owner of device memory and of the HIP stream: every call
+passes ``tensor.data_ptr()`` and ``torch.cuda.current_stream().cuda_stream`` to the library.
+There is no fallback: if the shared library is missing, or no GPU is present, calls raise.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_DIR = os.path.join(_HERE, "lib")
+LIB_PATH = os.path.join(LIB_DIR, "libpydtnn_hip.so")
+COMPAT_LIB_PATH = os.path.join(LIB_DIR, "libconvGemm.so")
+
+OP_FWD, OP_DW, OP_DX, OP_DX_I2C, OP_DB = range(5)
+
+_c = ctypes
+_f32p, _i8p, _i32p, _vp = _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p
+_geom13_i = [_c.c_int] * 13
+_geom13_u = [_c.c_uint] * 13
+
+# name -> (restype, argtypes); kept in one table so a test can check every declared symbol loads
+SIGNATURES = {
+    "pydtnn_hip_version": (_c.c_int, []),
+    "pydtnn_hip_status_string": (_c.c_char_p, [_c.c_int]),
+    "pydtnn_hip_im2col_nchw": (_c.c_int, [_f32p, _f32p] + [_c.c_int] * 12 + [_vp]),
+    "pydtnn_hip_col2im_nchw": (_c.c_int, [_f32p, _f32p] + [_c.c_int] * 12 + [_vp]),
+    "pydtnn_hip_im2row_nhwc": (_c.c_int, [_f32p, _f32p] + [_c.c_int] * 12 + [_vp]),
+    "pydtnn_hip_row2im_nhwc": (_c.c_int, [_f32p, _f32p] + [_c.c_int] * 12 + [_vp]),
+    "pydtnn_hip_sgemm_workspace_bytes": (_c.c_size_t, [_c.c_long] * 3),
+    "pydtnn_hip_sgemm": (_c.c_int, [_c.c_int, _c.c_int, _c.c_long, _c.c_long, _c.c_long, _f32p, _c.c_long, _f32p,
+                                    _c.c_long, _f32p, _c.c_long, _f32p, _c.c_int, _vp, _c.c_size_t, _vp]),
+    "pydtnn_hip_conv_workspace_bytes": (_c.c_size_t, [_c.c_int, _c.c_int] + _geom13_i),
+    "pydtnn_hip_sconvGemmNCHW": (_c.c_int, [_c.c_char] + _geom13_u + [_f32p] * 8 + [_c.c_bool, _vp, _c.c_size_t, _vp]),
+    "pydtnn_hip_sconvGemmNHWC": (_c.c_int, [_c.c_char] + _geom13_u + [_f32p] * 8 + [_c.c_bool, _vp, _c.c_size_t, _vp]),
+    "pydtnn_hip_sconvGemmNCHW_back": (_c.c_int, _geom13_u + [_f32p] * 3 + [_vp, _c.c_size_t, _vp]),
+    "pydtnn_hip_sconvGemmNHWC_back": (_c.c_int, _geom13_u + [_f32p] * 3 + [_vp, _c.c_size_t, _vp]),
+    "pydtnn_hip_conv_i2c_forward": (_c.c_int, [_c.c_int] + _geom13_i + [_f32p] * 4 + [_vp]),
+    "pydtnn_hip_conv_i2c_dw": (_c.c_int, [_c.c_int] + _geom13_i + [_f32p] * 3 + [_vp, _c.c_size_t, _vp]),
+    "pydtnn_hip_conv_i2c_dx": (_c.c_int, [_c.c_int] + _geom13_i + [_f32p] * 3 + [_vp, _c.c_size_t, _vp]),
+    "pydtnn_hip_chan_eltwise": (_c.c_int, [_f32p, _f32p, _f32p, _c.c_long, _c.c_int, _c.c_int] + [_f32p] * 5 +
+                                [_c.c_int, _vp]),
+    "pydtnn_hip_relu_fwd": (_c.c_int, [_f32p, _f32p, _i8p, _c.c_long, _vp]),
+    "pydtnn_hip_relu_bwd": (_c.c_int, [_f32p, _i8p, _f32p, _c.c_long, _vp]),
+    "pydtnn_hip_bias_grad": (_c.c_int, [_f32p, _f32p, _c.c_long, _c.c_int, _c.c_int, _vp, _c.c_size_t, _vp]),
+    "pydtnn_hip_max_pool_2d_fwd_nchw": (_c.c_int, [_f32p, _f32p, _i32p] + [_c.c_int] * 12 + [_vp]),
+    "pydtnn_hip_max_pool_2d_bwd_nchw": (_c.c_int, [_f32p, _i32p, _f32p] + [_c.c_int] * 12 + [_vp]),
+    "pydtnn_hip_sgd_momentum": (_c.c_int, [_f32p, _f32p, _f32p, _c.c_long, _c.c_float, _c.c_float, _c.c_float,
+                                           _c.c_int, _vp]),
+}
+
+# Host-pointer flavour exported by libconvGemm.so with the reference's own names
+COMPAT_SYMBOLS = ["alloc_pack_buffs", "sconvGemmNCHW", "sconvGemmNHWC", "sconvGemmNCHW_back", "sconvGemmNHWC_back"]
+
+_LIB = None
+
+
+class HipError(RuntimeError):
+    pass
+
+
+def load_library(path=LIB_PATH):
+    """Load the shared library and attach prototypes.  Raises ImportError when it is not built."""
+    if not os.path.exists(path):
+        raise ImportError(f"{path} is missing: build it with `make -C pydtnn_amd/csrc` "
+                          f"(or __graft_entry__.build()); there is no CPU fallback.")
+    lib = ctypes.CDLL(path)
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = restype
+        fn.argtypes = argtypes
+    return lib
+
+
+def lib():
+    global _LIB
+    if _LIB is None:
+        _LIB = load_library()
+    return _LIB
+
+
+def check(status, what):
+    if status != 0:
+        raise HipError(f"{what}: {lib().pydtnn_hip_status_string(status).decode()} (status {status})")
+
+
+def stream_ptr():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def ptr(t):
+    """Device address of a dense fp32/int tensor, or NULL for None."""
+    if t is None:
+        return None
+    if not t.is_cuda:
+        raise ValueError("expected a tensor on the GPU")
+    if not t.is_contiguous():
+        raise ValueError("expected a C-contiguous tensor")
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def f32(t, name="tensor"):
+    if t is not None and t.dtype != torch.float32:
+        # pydtnn/backends/cpu/libs/conv_gemm.py:101-107: only float32 is supported by this ABI
+        raise ValueError(f"Type {t.dtype} of {name} not supported by this version of the library!")
+    return ptr(t)
+
+
+# --------------------------------------------------------------------------- workspace
+# One grow-only scratch buffer per device.  All work is enqueued on the caller's current stream,
+# so consecutive calls use it strictly one after the other.
+_WORKSPACE = {}
+
+
+def workspace(nbytes):
+    """Returns (void* or None, size) for a scratch buffer of at least ``nbytes`` bytes."""
+    if nbytes == 0:
+        return None, 0
+    dev = torch.cuda.current_device()
+    buf = _WORKSPACE.get(dev)
+    if buf is None or buf.numel() < nbytes:
+        if buf is not None:
+            del _WORKSPACE[dev]
+            del buf
+        buf = torch.empty(int(nbytes * 1.25) + 256, dtype=torch.uint8, device=f"cuda:{dev}")
+        _WORKSPACE[dev] = buf
+    return ctypes.c_void_p(buf.data_ptr()), buf.numel()
+
+
+def conv_workspace(op, nhwc, geom13):
+    return workspace(lib().pydtnn_hip_conv_workspace_bytes(op, int(nhwc), *geom13))

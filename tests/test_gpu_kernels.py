@@ -1,0 +1,392 @@
+"""GPU parity tests of the kernels, through the C ABI, against the CPU oracle on the same seeded inputs.
+
+Bar: bit-exact for the index-only kernels (im2col, col2im, im2row, row2im, ReLU mask, maxpool);
+max |a-b| / max |b| <= 1e-4 for fp32 arithmetic (GEMMs and fused epilogues).
+"""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import FP32_REL_TOL, announce, assert_close, dev, host, rel_err
+from shapes import D, alexnet_layers, small_grid, x_2x4, x_2x4_c2, x_4x4, x_4x8, x_8x8, w_1x1, w_1x2, w_2x2, w_3x3, \
+    w_c2_1234_4567
+
+pytestmark = pytest.mark.gpu
+
+mid_grid = [
+    D(3, 5, 20, 17, 70, 3, 3, 1, 1, 1, 1, 1, 1),
+    D(2, 16, 30, 30, 130, 3, 3, 1, 1, 1, 1, 1, 1),
+    D(4, 3, 35, 35, 96, 11, 11, 0, 0, 4, 4, 1, 1),
+    D(2, 33, 14, 14, 257, 1, 1, 0, 0, 1, 1, 1, 1),
+    D(5, 8, 19, 23, 20, 5, 3, 2, 1, 2, 1, 1, 1),
+    D(2, 12, 16, 16, 24, 3, 3, 2, 2, 1, 1, 2, 2),
+    D(9, 64, 14, 14, 64, 3, 3, 1, 1, 1, 1, 1, 1),
+    D(3, 1, 28, 28, 32, 3, 3, 1, 1, 1, 1, 1, 1),
+]
+all_grid = small_grid + mid_grid
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from pydtnn_amd import ops as _ops, native
+    native.lib()  # raises if the HIP library was not built: no fallback
+    assert torch.cuda.is_available()
+    return _ops
+
+
+@pytest.fixture(scope="module")
+def cg():
+    from pydtnn_amd.conv_gemm import ConvGemm
+    return ConvGemm()
+
+
+def case(d, seed=0):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((d.b, d.c, d.h, d.w)).astype(np.float32)
+    w = (rng.standard_normal((d.kn, d.c, d.kh, d.kw)) * np.sqrt(2.0 / (d.c * d.kh * d.kw))).astype(np.float32)
+    b = rng.standard_normal(d.kn).astype(np.float32)
+    dy = rng.standard_normal((d.b, d.kn, d.ho, d.wo)).astype(np.float32)
+    return x, w, b, dy
+
+
+def nhwc(a):
+    return np.ascontiguousarray(a.transpose(0, 2, 3, 1))
+
+
+def w_nhwc(w):
+    return np.ascontiguousarray(w.transpose(1, 2, 3, 0))  # (kn,c,kh,kw) -> (c,kh,kw,kn)
+
+
+# ------------------------------------------------------------------ explicit gathers: bit-exact
+
+@pytest.mark.parametrize("d", all_grid, ids=repr)
+def test_im2col_col2im_nchw_bit_exact(ops, oracle, d):
+    announce("im2col/col2im nchw", d)
+    x, _, _, _ = case(d)
+    cols = ops.im2col_nchw(dev(x), *d.geom())
+    ref = oracle.im2col_nchw(x, *d.geom())
+    assert np.array_equal(host(cols), ref)
+    rng = np.random.default_rng(1)
+    cmat = rng.standard_normal(ref.shape).astype(np.float32)
+    dx = ops.col2im_nchw(dev(cmat), d.b, d.c, d.h, d.w, *d.geom())
+    # same addends in the same order as the reference's scatter loop: identical fp32 sums
+    assert np.array_equal(host(dx), oracle.col2im_nchw(cmat, d.b, d.c, d.h, d.w, *d.geom()))
+
+
+@pytest.mark.parametrize("d", all_grid, ids=repr)
+def test_im2row_row2im_nhwc_bit_exact(ops, oracle, d):
+    announce("im2row/row2im nhwc", d)
+    x, _, _, _ = case(d)
+    xr = nhwc(x)
+    rows = ops.im2row_nhwc(dev(xr), *d.geom())
+    ref = oracle.im2row_nhwc(xr, *d.geom())
+    assert np.array_equal(host(rows), ref)
+    rng = np.random.default_rng(1)
+    rmat = rng.standard_normal(ref.shape).astype(np.float32)
+    dx = ops.row2im_nhwc(dev(rmat), d.b, d.h, d.w, d.c, *d.geom())
+    assert np.array_equal(host(dx), oracle.row2im_nhwc(rmat, d.b, d.h, d.w, d.c, *d.geom()))
+
+
+def test_im2col_unaligned_column_count(ops, oracle):
+    d = D(1, 2, 7, 9, 1, 3, 3, 0, 0, 1, 1)  # P = 35: scalar-store path
+    announce("im2col unaligned", d)
+    x, _, _, _ = case(d)
+    assert np.array_equal(host(ops.im2col_nchw(dev(x), *d.geom())), oracle.im2col_nchw(x, *d.geom()))
+
+
+def test_unsupported_dtype_raises(ops):
+    with pytest.raises(TypeError):
+        ops.im2col_nchw(torch.zeros((1, 1, 4, 4), dtype=torch.float64, device="cuda"), 3, 3, 0, 0, 1, 1, 1, 1)
+
+
+# ------------------------------------------------------------------ GEMM
+
+@pytest.mark.parametrize("m,n,k", [(1, 1, 1), (7, 5, 3), (64, 64, 64), (65, 129, 17), (128, 128, 256), (130, 70, 300),
+                                   (300, 40, 33), (40, 300, 1000), (64, 1000, 4096), (257, 255, 129)])
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_sgemm_against_fp64(ops, m, n, k, ta, tb):
+    announce("sgemm", m, n, k, ta, tb)
+    rng = np.random.default_rng(m * 1000 + n + k)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    b = rng.standard_normal((k, n)).astype(np.float32)
+    ad = dev(a.T).t() if ta else dev(a)
+    bd = dev(b.T).t() if tb else dev(b)
+    c = ops.matmul(ad, bd)
+    ref = a.astype(np.float64) @ b.astype(np.float64)
+    assert_close(host(c), ref, what="sgemm vs fp64")
+    assert_close(host(c), a @ b, what="sgemm vs OpenBLAS fp32")
+
+
+def test_sgemm_bias_relu_epilogue_with_and_without_split(ops):
+    for (m, n, k) in [(64, 96, 8192), (200, 300, 64)]:
+        announce("sgemm epilogue", m, n, k)
+        rng = np.random.default_rng(3)
+        a = rng.standard_normal((m, k)).astype(np.float32)
+        b = rng.standard_normal((k, n)).astype(np.float32)
+        bias = rng.standard_normal(n).astype(np.float32)
+        c = ops.matmul(dev(a), dev(b), bias=dev(bias), relu=True)
+        ref = np.maximum(a.astype(np.float64) @ b + bias, 0)
+        assert_close(host(c), ref, what="sgemm+bias+relu")
+
+
+def test_sgemm_rejects_bad_layout(ops):
+    a = torch.zeros((8, 8), device="cuda")[:, ::2]
+    with pytest.raises(ValueError):
+        ops.matmul(a, torch.zeros((4, 4), device="cuda"))
+
+
+# ------------------------------------------------------------------ implicit conv forward
+
+def _fwd_ref(oracle, x, w, b, d):
+    y, _ = oracle.conv2d_forward_nchw_i2c(x, w, b, oracle.ConvParams(*d.geom()))
+    return y
+
+
+def _kw(d):
+    return dict(vpadding=d.vpadding, hpadding=d.hpadding, vstride=d.vstride, hstride=d.hstride,
+                vdilation=d.vdilation, hdilation=d.hdilation)
+
+
+@pytest.mark.parametrize("d", all_grid, ids=repr)
+def test_conv_gemm_forward_both_formats(cg, oracle, d):
+    announce("conv_gemm fwd", d)
+    x, w, b, _ = case(d)
+    ref = _fwd_ref(oracle, x, w, b, d)
+    y = cg.conv_gemm_nchw(dev(w), dev(x), biases_vector=dev(b), **_kw(d))
+    assert_close(host(y), ref, what="nchw")
+    y2 = cg.conv_gemm_nhwc(dev(w_nhwc(w)), dev(nhwc(x)), biases_vector=dev(b), **_kw(d))
+    ref_nhwc, _ = oracle.conv2d_forward_nhwc_i2c(nhwc(x), w_nhwc(w), b, oracle.ConvParams(*d.geom()))
+    assert_close(host(y2), ref_nhwc, what="nhwc")
+
+
+@pytest.mark.parametrize("x,w,stride", [
+    (x_2x4, w_1x1, 1), (x_2x4, w_1x2, 1), (x_2x4, w_2x2, 1), (x_4x4, w_2x2, 2), (x_4x8, w_2x2, (1, 2)),
+    (x_8x8, w_3x3, 3), (x_8x8, w_2x2, 1), (x_2x4_c2, w_c2_1234_4567, 1)])
+def test_reference_hand_arrays_exact(cg, oracle, x, w, stride):
+    """Inputs of pydtnn/tests/conv_gemm.py:81-209 and conv2d_conv_gemm.py:72-103: small integers, exact in fp32."""
+    sv, sh = (stride, stride) if isinstance(stride, int) else stride
+    d = D(1, x.shape[1], x.shape[2], x.shape[3], w.shape[0], w.shape[2], w.shape[3], 0, 0, sv, sh)
+    announce("hand arrays", d)
+    y = cg.conv_gemm_nchw(dev(w), dev(x), **_kw(d))
+    assert np.array_equal(host(y), _fwd_ref(oracle, x, w, None, d))
+    if x is x_2x4 and w is w_2x2:
+        assert np.array_equal(host(y).ravel(), [51, 102, 204])
+
+
+def test_default_D_ones(cg):
+    d = D()
+    announce("default D ones", d)
+    y = host(cg.conv_gemm_nchw(dev(np.ones((1, 1, d.kh, d.kw), np.float32)),
+                               dev(np.ones((1, 1, d.h, d.w), np.float32)), **_kw(d)))
+    assert y.shape == (1, 1, 115, 93)
+    assert np.all(y[0, 0, 1:-1, 1:-1] == 160) and y[0, 0, 0, 0] == 135
+
+
+@pytest.mark.parametrize("i", range(10), ids=lambda i: f"alexnet{i}")
+def test_alexnet_layers_forward_and_deconv(cg, oracle, i):
+    """The ten layers of pydtnn/tests/common.py:77-90 (batch cut to 8 so the CPU oracle stays fast)."""
+    L = alexnet_layers[i]
+    d = D(8, L.c, L.h, L.w, L.kn, L.kh, L.kw, L.vpadding, L.hpadding, L.vstride, L.hstride)
+    announce("alexnet", i, d)
+    x, w, b, dy = case(d)
+    y = cg.conv_gemm_nchw(dev(w), dev(x), **_kw(d))
+    assert_close(host(y), _fwd_ref(oracle, x, w, None, d), what="fwd")
+    # pydtnn/tests/conv_gemm.py:489-524: deconv_gemm vs W^T dy + col2im
+    dx = torch.empty((d.b, d.c, d.h, d.w), device="cuda")
+    cg.deconv_gemm_nchw(dev(w), dev(dy), dx, **_kw(d))
+    res = w.reshape(d.kn, -1).T @ dy.transpose(1, 0, 2, 3).reshape(d.kn, -1)
+    assert_close(host(dx), oracle.col2im_nchw(res, d.b, d.c, d.h, d.w, *d.geom()), what="deconv")
+
+
+@pytest.mark.parametrize("fmt", ["NCHW", "NHWC"])
+@pytest.mark.parametrize("use_bias,use_bn,use_relu", [(1, 0, 1), (0, 1, 0), (1, 1, 1), (0, 0, 1)])
+def test_fused_epilogue(cg, oracle, fmt, use_bias, use_bn, use_relu):
+    d = mid_grid[1]
+    announce("fused epilogue", fmt, use_bias, use_bn, use_relu)
+    x, w, b, _ = case(d)
+    rng = np.random.default_rng(5)
+    mean = rng.normal(0, 0.1, d.kn).astype(np.float32)
+    var = rng.uniform(0.5, 1.5, d.kn).astype(np.float32)
+    gamma = rng.uniform(0.5, 1.5, d.kn).astype(np.float32)
+    beta = rng.normal(0, 0.1, d.kn).astype(np.float32)
+    inv_std = (1.0 / np.sqrt(var + np.float32(1e-5))).astype(np.float32)
+    bn = (mean, inv_std, gamma, beta)
+    kw = dict(_kw(d), biases_vector=dev(b) if use_bias else None, relu=bool(use_relu))
+    if use_bn:
+        kw.update(bn_running_mean=dev(mean), bn_inv_std=dev(inv_std), bn_gamma=dev(gamma), bn_beta=dev(beta))
+    p = oracle.ConvParams(*d.geom())
+    if fmt == "NCHW":
+        y = cg.conv_gemm_nchw(dev(w), dev(x), **kw)
+        ref, _ = oracle.conv2d_forward_nchw_i2c(x, w, b if use_bias else None, p)
+    else:
+        y = cg.conv_gemm_nhwc(dev(w_nhwc(w)), dev(nhwc(x)), **kw)
+        ref, _ = oracle.conv2d_forward_nhwc_i2c(nhwc(x), w_nhwc(w), b if use_bias else None, p)
+    ref = oracle.fused_epilogue(ref, fmt, bn=bn if use_bn else None, relu_flag=bool(use_relu))
+    assert_close(host(y), ref, what="fused")
+    if use_relu:
+        assert host(y).min() >= 0
+
+
+def test_bn_arguments_must_come_together(cg):
+    d = small_grid[1]
+    x, w, b, _ = case(d)
+    from pydtnn_amd.native import HipError
+    with pytest.raises(HipError):
+        cg.conv_gemm_nchw(dev(w), dev(x), bn_running_mean=dev(b), **_kw(d))
+
+
+# ------------------------------------------------------------------ implicit backward
+
+@pytest.mark.parametrize("d", all_grid, ids=repr)
+def test_conv_gemm_backward_both_formats(cg, oracle, d):
+    announce("conv_gemm bwd", d)
+    x, w, _, dy = case(d)
+    p = oracle.ConvParams(*d.geom())
+    _, x_cols = oracle.conv2d_forward_nchw_i2c(x, w, None, p)
+    dw_ref, _, dx_ref = oracle.conv2d_backward_nchw_i2c(dy, x_cols, w, x.shape, p)
+    dw = torch.empty(w.shape, device="cuda")
+    cg.conv_gemm_nchw(dev(dy), dev(x), biases=dw, trans=True, **_kw(d))
+    assert_close(host(dw), dw_ref, what="dw nchw")
+    dx = torch.empty(x.shape, device="cuda")
+    cg.deconv_gemm_nchw(dev(w), dev(dy), dx, **_kw(d))
+    assert_close(host(dx), dx_ref, what="dx nchw")
+    # NHWC, mapped back with the transposes of pydtnn/tests/check_tensor_format_models.py:124-129
+    dw2 = torch.empty(w_nhwc(w).shape, device="cuda")
+    cg.conv_gemm_nhwc(dev(nhwc(dy)), dev(nhwc(x)), biases=dw2, trans=True, **_kw(d))
+    assert_close(host(dw2).transpose(3, 0, 1, 2), dw_ref, what="dw nhwc")
+    dx2 = torch.empty(nhwc(x).shape, device="cuda")
+    cg.deconv_gemm_nhwc(dev(w_nhwc(w)), dev(nhwc(dy)), dx2, **_kw(d))
+    assert_close(host(dx2).transpose(0, 3, 1, 2), dx_ref, what="dx nhwc")
+
+
+def test_dw_split_over_several_images_and_chunks(cg, oracle):
+    """Small spatial extent (several images per reduction group) and large one (several chunks per image)."""
+    for d in [D(40, 6, 7, 7, 10, 3, 3, 1, 1, 1, 1), D(2, 3, 90, 90, 5, 3, 3, 1, 1, 1, 1)]:
+        announce("dw split", d)
+        x, w, _, dy = case(d)
+        p = oracle.ConvParams(*d.geom())
+        _, x_cols = oracle.conv2d_forward_nchw_i2c(x, w, None, p)
+        dw_ref, _, _ = oracle.conv2d_backward_nchw_i2c(dy, x_cols, w, x.shape, p, need_dx=False)
+        dw = torch.empty(w.shape, device="cuda")
+        cg.conv_gemm_nchw(dev(dy), dev(x), biases=dw, trans=True, **_kw(d))
+        assert_close(host(dw), dw_ref, what="dw nchw")
+        dw2 = torch.empty(w_nhwc(w).shape, device="cuda")
+        cg.conv_gemm_nhwc(dev(nhwc(dy)), dev(nhwc(x)), biases=dw2, trans=True, **_kw(d))
+        assert_close(host(dw2).transpose(3, 0, 1, 2), dw_ref, what="dw nhwc")
+
+
+# ------------------------------------------------------------------ elementwise kernels
+
+def test_chan_eltwise_matches_oracle(ops, oracle):
+    rng = np.random.default_rng(7)
+    for shape, fmt in [((3, 7, 5, 6), "NCHW"), ((3, 8, 4, 4), "NCHW"), ((3, 5, 6, 7), "NHWC"), ((2, 4, 4, 8), "NHWC")]:
+        announce("chan_eltwise", shape, fmt)
+        c = shape[1] if fmt == "NCHW" else shape[3]
+        x = rng.standard_normal(shape).astype(np.float32)
+        bn = [rng.standard_normal(c).astype(np.float32) for _ in range(4)]
+        if fmt == "NCHW":
+            y = ops.bn_inference_nchw(dev(x), *[dev(v) for v in bn], relu=True)
+            ref = np.maximum(oracle.bn_inference_nchw(x, *bn), 0)
+        else:
+            y = ops.bn_relu_inference(dev(x.reshape(-1, c)), *[dev(v) for v in bn]).reshape(shape)
+            ref = oracle.bn_inference(x.reshape(-1, c), *bn, relu=True).reshape(shape)
+        # one fused multiply-add instead of two roundings in the last step: a few ulp at most
+        assert_close(host(y), ref, tol=1e-6, what="bn+relu")
+    x2 = rng.standard_normal((6, 10)).astype(np.float32)
+    b6, b10 = rng.standard_normal(6).astype(np.float32), rng.standard_normal(10).astype(np.float32)
+    assert np.array_equal(host(ops.add_nchw(dev(x2), dev(b6))), oracle.add_nchw(x2.copy(), b6))
+    assert np.array_equal(host(ops.add_nhwc(dev(x2), dev(b10))), oracle.add_nhwc(x2.copy(), b10))
+    acc = dev(x2)
+    ops.eltw_sum(acc, dev(2 * x2))
+    assert np.array_equal(host(acc), oracle.eltw_sum(x2.copy(), 2 * x2))
+
+
+def test_relu_forward_backward(ops, oracle):
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((5, 1001)).astype(np.float32)
+    x[0, :4] = [0.0, -0.0, 1e-30, -1e-30]
+    y, mask = ops.relu(dev(x))
+    y_ref, m_ref = oracle.relu(x)
+    assert np.array_equal(host(y), y_ref) and np.array_equal(host(mask), m_ref)
+    dy = rng.standard_normal(x.shape).astype(np.float32)
+    assert np.array_equal(host(ops.relu_backward(dev(dy), mask)), dy * m_ref)
+
+
+def test_bias_grad(ops):
+    rng = np.random.default_rng(9)
+    for shape in [(3, 5, 7, 9), (64, 33, 14, 14), (1, 2, 3, 3)]:
+        announce("bias_grad", shape)
+        dy = rng.standard_normal(shape).astype(np.float32)
+        db = ops.bias_grad(dev(dy), shape[1], shape[2] * shape[3])
+        assert_close(host(db), dy.astype(np.float64).sum(axis=(0, 2, 3)), tol=1e-5, what="db nchw")
+        dyr = nhwc(dy)
+        db2 = ops.bias_grad(dev(dyr), shape[1], 1)
+        assert_close(host(db2), dy.astype(np.float64).sum(axis=(0, 2, 3)), tol=1e-5, what="db nhwc")
+
+
+def test_maxpool_matches_oracle(ops, oracle):
+    rng = np.random.default_rng(10)
+    for (shape, k, s, p) in [((2, 3, 8, 10), 2, 2, 0), ((2, 4, 9, 9), 3, 2, 1), ((1, 2, 7, 7), 3, 1, 1)]:
+        announce("maxpool", shape, k, s, p)
+        x = rng.standard_normal(shape).astype(np.float32)
+        x[0, 0, :2, :2] = 1.5  # ties: the first tap must win
+        y, idx = ops.max_pool_2d_fwd_nchw(dev(x), k, k, p, p, s, s)
+        y_ref, idx_ref = oracle.max_pool_2d_fwd_nchw(x, k, k, p, p, s, s)
+        assert np.array_equal(host(y), y_ref) and np.array_equal(host(idx), idx_ref)
+        dy = rng.standard_normal(y_ref.shape).astype(np.float32)
+        dx = ops.max_pool_2d_bwd_nchw(dev(dy), idx, *shape, k, k, p, p, s, s)
+        dx_ref = oracle.max_pool_2d_bwd_nchw(dy, idx_ref, *shape, k, k, p, p, s, s)
+        assert_close(host(dx), dx_ref, tol=1e-6, what="maxpool bwd")
+
+
+def test_sgd_momentum(ops, oracle):
+    rng = np.random.default_rng(11)
+    w, dw, v = [rng.standard_normal(1000).astype(np.float32) for _ in range(3)]
+    wd, vd = dev(w), dev(v)
+    ops.sgd_momentum(wd, dev(dw), vd, 0.01, 0.9, 1e-4, False)
+    w_ref, v_ref = oracle.sgd_update(w.copy(), dw, v.copy(), np.float32(0.01), np.float32(0.9), np.float32(1e-4))
+    assert_close(host(wd), w_ref, tol=1e-6, what="sgd w")
+    assert_close(host(vd), v_ref, tol=1e-6, what="sgd v")
+
+
+# ------------------------------------------------------------------ host-pointer compatibility ABI
+
+def test_libconvgemm_compat_abi_runs_like_the_reference_shim(oracle):
+    """Calls libconvGemm.so exactly the way pydtnn/backends/cpu/libs/conv_gemm.py:191-205, :299-307 does."""
+    from pydtnn_amd import native
+    lib = ctypes.CDLL(native.COMPAT_LIB_PATH)
+    ac, bc = ctypes.POINTER(ctypes.c_float)(), ctypes.POINTER(ctypes.c_float)()
+    lib.alloc_pack_buffs.restype = ctypes.c_int
+    assert lib.alloc_pack_buffs(ctypes.byref(ac), ctypes.byref(bc)) == 0
+    d = mid_grid[0]
+    announce("compat abi", d)
+    x, w, b, dy = case(d)
+    y = np.empty((d.b, d.kn, d.ho, d.wo), np.float32)
+    u = ctypes.c_uint
+    none = ctypes.c_void_p(None)
+    lib.sconvGemmNCHW(ctypes.c_char(b'N'), u(d.b), u(d.c), u(d.h), u(d.w), u(d.kn), u(d.kh), u(d.kw),
+                      u(d.vpadding), u(d.hpadding), u(d.vstride), u(d.hstride), u(d.vdilation), u(d.hdilation),
+                      ctypes.c_void_p(w.ctypes.data), ctypes.c_void_p(x.ctypes.data), ctypes.c_void_p(y.ctypes.data),
+                      ctypes.c_void_p(b.ctypes.data), none, none, none, none, ctypes.c_bool(True), ac, bc)
+    ref = np.maximum(_fwd_ref(oracle, x, w, b, d), 0)
+    assert_close(y, ref, what="compat fwd")
+    dw = np.empty(w.shape, np.float32)
+    lib.sconvGemmNCHW(ctypes.c_char(b'Y'), u(d.b), u(d.c), u(d.h), u(d.w), u(d.kn), u(d.kh), u(d.kw),
+                      u(d.vpadding), u(d.hpadding), u(d.vstride), u(d.hstride), u(d.vdilation), u(d.hdilation),
+                      ctypes.c_void_p(dy.ctypes.data), ctypes.c_void_p(x.ctypes.data),
+                      ctypes.c_void_p(dw.ctypes.data), none, none, none, none, none, ctypes.c_bool(False), ac, bc)
+    p = oracle.ConvParams(*d.geom())
+    _, x_cols = oracle.conv2d_forward_nchw_i2c(x, w, None, p)
+    dw_ref, _, dx_ref = oracle.conv2d_backward_nchw_i2c(dy, x_cols, w, x.shape, p)
+    assert_close(dw, dw_ref, what="compat dw")
+    dx = np.zeros(x.shape, np.float32)
+    lib.sconvGemmNCHW_back(u(d.b), u(d.c), u(d.h), u(d.w), u(d.kn), u(d.kh), u(d.kw), u(d.vstride), u(d.hstride),
+                           u(d.vpadding), u(d.hpadding), u(d.vdilation), u(d.hdilation),
+                           ctypes.c_void_p(w.ctypes.data), ctypes.c_void_p(dy.ctypes.data),
+                           ctypes.c_void_p(dx.ctypes.data), ac, bc)
+    assert_close(dx, dx_ref, what="compat dx")
+    libc = ctypes.CDLL("libc.so.6")
+    libc.free(ac)
+    libc.free(bc)

@@ -1,0 +1,332 @@
+"""GPU parity tests at the layer / model level: the PyDTNN layer protocol on top of the kernels.
+
+Pattern follows the reference's own layer tests: build the layer under a model, feed the same
+arrays to the CPU path (here: the oracle) and compare y, dw, db, dx
+(pydtnn/tests/conv2d_conv_gemm.py:114-200, check_tensor_format_models.py:66-162,
+check_conv_gemm_models.py:100-167: the CPU activations are fed to each layer under test).
+"""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import announce, assert_close, dev, host
+from shapes import D, small_grid
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def pd():
+    import pydtnn_amd
+    from pydtnn_amd import native
+    native.lib()
+    return pydtnn_amd
+
+
+def nhwc(a):
+    return np.ascontiguousarray(a.transpose(0, 2, 3, 1))
+
+
+def make_conv(pd, d, fmt, variant, need_dx=True, use_bias=True):
+    model = pd.Model(tensor_format=fmt, enable_conv_gemm=(variant == "cg"), batch_size=d.b)
+    model.mode = pd.TRAIN_MODE
+    layer = pd.Conv2D(nfilters=d.kn, filter_shape=(d.kh, d.kw), padding=(d.vpadding, d.hpadding),
+                      stride=(d.vstride, d.hstride), dilation=(d.vdilation, d.hdilation), use_bias=use_bias)
+    layer.set_model(model)
+    layer.initialize(prev_shape=(d.c, d.h, d.w) if fmt == "NCHW" else (d.h, d.w, d.c), need_dx=need_dx)
+    return model, layer
+
+
+layer_grid = small_grid[:8] + [D(4, 16, 20, 20, 40, 3, 3, 1, 1, 1, 1), D(3, 8, 17, 17, 12, 3, 3, 1, 1, 2, 2)]
+
+
+@pytest.mark.parametrize("variant", ["i2c", "cg"])
+@pytest.mark.parametrize("fmt", ["NCHW", "NHWC"])
+@pytest.mark.parametrize("d", layer_grid, ids=repr)
+def test_conv2d_layer_forward_backward(pd, oracle, d, fmt, variant):
+    announce("Conv2D layer", fmt, variant, d)
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((d.b, d.c, d.h, d.w)).astype(np.float32)
+    w = rng.standard_normal((d.kn, d.c, d.kh, d.kw)).astype(np.float32) * 0.2
+    b = rng.standard_normal(d.kn).astype(np.float32)
+    dy = rng.standard_normal((d.b, d.kn, d.ho, d.wo)).astype(np.float32)
+    model, layer = make_conv(pd, d, fmt, variant)
+    assert layer.forward.__name__ == f"_forward_{fmt.lower()}_{variant}"
+    p = oracle.ConvParams(*d.geom())
+    if fmt == "NCHW":
+        assert tuple(layer.weights.shape) == w.shape and layer.shape == (d.kn, d.ho, d.wo)
+        layer.weights, layer.biases = dev(w), dev(b)
+        y_ref, x_cols = oracle.conv2d_forward_nchw_i2c(x, w, b, p)
+        dw_ref, db_ref, dx_ref = oracle.conv2d_backward_nchw_i2c(dy, x_cols, w, x.shape, p)
+        y = layer.forward(dev(x))
+        dx = layer.backward(dev(dy))
+        if variant == "i2c":
+            assert np.array_equal(host(layer.x_cols), x_cols)  # the stored matrix is the reference's x_cols
+    else:
+        wr = np.ascontiguousarray(w.transpose(1, 2, 3, 0))
+        assert tuple(layer.weights.shape) == wr.shape and layer.shape == (d.ho, d.wo, d.kn)
+        layer.weights, layer.biases = dev(wr), dev(b)
+        y_ref, x_rows = oracle.conv2d_forward_nhwc_i2c(nhwc(x), wr, b, p)
+        dw_ref, db_ref, dx_ref = oracle.conv2d_backward_nhwc_i2c(nhwc(dy), x_rows, wr, nhwc(x).shape, p)
+        y = layer.forward(dev(nhwc(x)))
+        dx = layer.backward(dev(nhwc(dy)))
+        if variant == "i2c":
+            assert np.array_equal(host(layer.x_rows), x_rows)
+    assert_close(host(y), y_ref, what="y")
+    assert_close(host(layer.dw), dw_ref, what="dw")
+    assert tuple(layer.dw.shape) == tuple(layer.weights.shape)
+    assert_close(host(layer.db), db_ref, tol=1e-5, what="db")
+    assert_close(host(dx), dx_ref, what="dx")
+
+
+def test_first_layer_has_no_dx(pd):
+    d = small_grid[1]
+    model, layer = make_conv(pd, d, "NCHW", "cg", need_dx=False)
+    x = torch.randn((d.b, d.c, d.h, d.w), device="cuda")
+    y = layer.forward(x)
+    assert layer.backward(torch.ones_like(y)) is None and layer.dw is not None
+
+
+def test_grouped_convolutions_raise(pd):
+    model = pd.Model(tensor_format="NCHW")
+    layer = pd.Conv2D(nfilters=4, filter_shape=(3, 3), grouping="depthwise")
+    layer.set_model(model)
+    with pytest.raises(NotImplementedError):
+        layer.initialize(prev_shape=(4, 8, 8))
+
+
+def test_fc_layer(pd, oracle):
+    rng = np.random.default_rng(1)
+    for (bsz, nin, nout) in [(64, 300, 100), (5, 4100, 33)]:
+        announce("FC", bsz, nin, nout)
+        model = pd.Model(tensor_format="NCHW", batch_size=bsz)
+        model.mode = pd.TRAIN_MODE
+        fc = pd.FC(shape=(nout,))
+        fc.set_model(model)
+        fc.initialize(prev_shape=(nin,))
+        x = rng.standard_normal((bsz, nin)).astype(np.float32)
+        w = (rng.standard_normal((nin, nout)) / np.sqrt(nin)).astype(np.float32)
+        b = rng.standard_normal(nout).astype(np.float32)
+        dy = rng.standard_normal((bsz, nout)).astype(np.float32)
+        assert tuple(fc.weights.shape) == (nin, nout)
+        fc.weights, fc.biases = dev(w), dev(b)
+        y = fc.forward(dev(x))
+        dx = fc.backward(dev(dy))
+        dw_ref, db_ref, dx_ref = oracle.fc_backward(dy, x, w)
+        assert_close(host(y), oracle.fc_forward(x, w, b), what="fc y")
+        assert_close(host(fc.dw), dw_ref, what="fc dw")
+        assert_close(host(fc.db), db_ref, tol=1e-5, what="fc db")
+        assert_close(host(dx), dx_ref, what="fc dx")
+
+
+# ------------------------------------------------------------------ fusion
+
+def build_conv_bn_relu_model(pd, fmt, flags, shape_hwc=(12, 12, 6), seed=2):
+    model = pd.Model(tensor_format=fmt, **flags)
+    model.add(pd.Input(shape=shape_hwc))
+    model.add(pd.Conv2D(nfilters=10, filter_shape=(3, 3), padding=1))
+    model.add(pd.BatchNormalization())
+    model.add(pd.Relu())
+    model.add(pd.Conv2D(nfilters=7, filter_shape=(1, 1)))
+    model.add(pd.BatchNormalization())
+    model.add(pd.Conv2D(nfilters=5, filter_shape=(3, 3), stride=2, activation="relu"))
+    rng = np.random.default_rng(seed)
+    for layer in model.layers:
+        if layer.canonical_name == "BatchNormalization":
+            c = layer.gamma.numel()
+            layer.gamma = dev(rng.uniform(0.5, 1.5, c).astype(np.float32))
+            layer.beta = dev(rng.normal(0, 0.1, c).astype(np.float32))
+            layer.running_mean = dev(rng.normal(0, 0.1, c).astype(np.float32))
+            layer.running_var = dev(rng.uniform(0.5, 1.5, c).astype(np.float32))
+            layer.updated_running_var = True
+        elif layer.canonical_name == "Conv2D":
+            layer.weights = dev((rng.standard_normal(tuple(layer.weights.shape)) * 0.2).astype(np.float32))
+            layer.biases = dev(rng.standard_normal(layer.co).astype(np.float32))
+    return model
+
+
+@pytest.mark.parametrize("fmt", ["NCHW", "NHWC"])
+def test_fusion_rewrites_the_graph_and_keeps_the_numbers(pd, oracle, fmt):
+    announce("fusion", fmt)
+    flags = dict(enable_fused_conv_bn_relu=True, enable_fused_conv_bn=True, enable_fused_conv_relu=True,
+                 enable_fused_bn_relu=True)
+    plain = build_conv_bn_relu_model(pd, fmt, {})
+    fused = build_conv_bn_relu_model(pd, fmt, flags)
+    x = np.random.default_rng(3).standard_normal((4, 6, 12, 12)).astype(np.float32)
+    xin = dev(x if fmt == "NCHW" else nhwc(x))
+    y_plain = plain.evaluate_dataset_batch(xin)
+    y_fused = fused.evaluate_dataset_batch(xin)
+    names = [layer.canonical_name for layer in fused.layers]
+    assert names == ["Input", "Conv2DBatchNormalizationRelu", "Conv2DBatchNormalization", "Conv2DRelu"]
+    assert [layer.canonical_name for layer in plain.layers][1:4] == ["Conv2D", "BatchNormalization", "Relu"]
+    assert_close(host(y_fused), host(y_plain), tol=1e-6, what="fused vs layer-by-layer")
+    # against the oracle: conv -> bias -> BN -> ReLU composed from pinned parts
+    p1 = oracle.ConvParams(3, 3, 1, 1)
+    p2 = oracle.ConvParams(1, 1)
+    p3 = oracle.ConvParams(3, 3, 0, 0, 2, 2)
+    convs = [l for l in plain.layers if l.canonical_name == "Conv2D"]
+    bns = [l for l in plain.layers if l.canonical_name == "BatchNormalization"]
+    cur = x if fmt == "NCHW" else nhwc(x)
+    fwd = oracle.conv2d_forward_nchw_i2c if fmt == "NCHW" else oracle.conv2d_forward_nhwc_i2c
+    for conv, p, bn, relu in [(convs[0], p1, bns[0], True), (convs[1], p2, bns[1], False), (convs[2], p3, None, True)]:
+        cur, _ = fwd(cur, host(conv.weights), host(conv.biases), p)
+        bn_args = None
+        if bn is not None:
+            inv_std = (1.0 / np.sqrt(host(bn.running_var) + np.float32(bn.epsilon))).astype(np.float32)
+            bn_args = (host(bn.running_mean), inv_std, host(bn.gamma), host(bn.beta))
+        cur = oracle.fused_epilogue(cur, fmt, bn=bn_args, relu_flag=relu)
+    assert_close(host(y_fused), cur, what="fused vs oracle")
+
+
+def test_i2c_convolutions_are_not_fused(pd):
+    model = build_conv_bn_relu_model(pd, "NCHW", dict(enable_conv_gemm=False, enable_fused_conv_bn_relu=True))
+    model.apply_layer_fusion()
+    assert [l.canonical_name for l in model.layers][1:4] == ["Conv2D", "BatchNormalization", "Relu"]
+
+
+def test_fused_layers_refuse_training_and_backward(pd):
+    model = build_conv_bn_relu_model(pd, "NCHW", dict(enable_fused_conv_bn_relu=True))
+    model.apply_layer_fusion()
+    fused = model.layers[1]
+    model.mode = pd.TRAIN_MODE
+    with pytest.raises(RuntimeError):
+        fused.forward(torch.zeros((1, 6, 12, 12), device="cuda"))
+    with pytest.raises(RuntimeError):
+        fused.backward(torch.zeros((1, 10, 12, 12), device="cuda"))
+
+
+def test_residual_block_with_fusion(pd, oracle):
+    """A bottleneck shaped like pydtnn/models/resnet50_imagenet.py:41-59, NHWC, all fusions on."""
+    announce("bottleneck")
+    rng = np.random.default_rng(4)
+    cin, mid, hw, n = 16, 8, 10, 3
+
+    def build(flags):
+        model = pd.Model(tensor_format="NHWC", **flags)
+        model.add(pd.Input(shape=(hw, hw, cin)))
+        model.add(pd.AdditionBlock(
+            [pd.Conv2D(nfilters=mid, filter_shape=(1, 1)), pd.BatchNormalization(), pd.Relu(),
+             pd.Conv2D(nfilters=mid, filter_shape=(3, 3), padding=1), pd.BatchNormalization(), pd.Relu(),
+             pd.Conv2D(nfilters=cin, filter_shape=(1, 1)), pd.BatchNormalization()],
+            []))
+        model.add(pd.Relu())
+        return model
+
+    plain, fused = build({}), build(dict(enable_fused_conv_bn_relu=True, enable_fused_conv_bn=True))
+    r = np.random.default_rng(5)
+    for a, b in zip(plain.get_all_layers(), fused.get_all_layers()):
+        if a.canonical_name == "Conv2D":
+            a.weights = b.weights = dev((r.standard_normal(tuple(a.weights.shape)) * 0.3).astype(np.float32))
+        elif a.canonical_name == "BatchNormalization":
+            c = a.gamma.numel()
+            a.gamma = b.gamma = dev(r.uniform(0.5, 1.5, c).astype(np.float32))
+            a.beta = b.beta = dev(r.normal(0, 0.1, c).astype(np.float32))
+            a.running_mean = b.running_mean = dev(r.normal(0, 0.1, c).astype(np.float32))
+            a.running_var = b.running_var = dev(r.uniform(0.5, 1.5, c).astype(np.float32))
+            a.updated_running_var = b.updated_running_var = True
+    x = rng.standard_normal((n, hw, hw, cin)).astype(np.float32)
+    xd = dev(x)
+    y_plain = plain.evaluate_dataset_batch(xd)
+    y_fused = fused.evaluate_dataset_batch(xd)
+    block = fused.layers[1]
+    assert [l.canonical_name for l in block.paths[0]] == \
+        ["Conv2DBatchNormalizationRelu", "Conv2DBatchNormalizationRelu", "Conv2DBatchNormalization"]
+    assert np.array_equal(host(xd), x), "the block must not add into its input"
+    assert_close(host(y_fused), host(y_plain), tol=1e-6, what="bottleneck fused vs plain")
+    # oracle: relu(x + bn3(conv3(relu(bn2(conv2(relu(bn1(conv1(x)))))))))
+    convs = [l for l in plain.get_all_layers() if l.canonical_name == "Conv2D"]
+    bns = [l for l in plain.get_all_layers() if l.canonical_name == "BatchNormalization"]
+    cur = x
+    for conv, bn, relu, p in zip(convs, bns, (True, True, False),
+                                 (oracle.ConvParams(1, 1), oracle.ConvParams(3, 3, 1, 1), oracle.ConvParams(1, 1))):
+        cur, _ = oracle.conv2d_forward_nhwc_i2c(cur, host(conv.weights), host(conv.biases), p)
+        inv_std = (1.0 / np.sqrt(host(bn.running_var) + np.float32(bn.epsilon))).astype(np.float32)
+        cur = oracle.fused_epilogue(cur, "NHWC", bn=(host(bn.running_mean), inv_std, host(bn.gamma), host(bn.beta)),
+                                    relu_flag=relu)
+    ref, _ = oracle.relu(oracle.eltw_sum(np.ascontiguousarray(cur), x))
+    assert_close(host(y_fused), ref, what="bottleneck vs oracle")
+
+
+# ------------------------------------------------------------------ a small VGG-style training step
+
+def test_small_vgg_training_step_matches_the_oracle_chain(pd, oracle):
+    """conv-relu-conv-relu-pool-conv-relu-pool-flatten-fc-relu-fc-softmax, CCE, SGD momentum: one step,
+    every gradient and updated weight compared with the oracle run end to end on the CPU."""
+    announce("small vgg step")
+    rng = np.random.default_rng(6)
+    n, classes = 8, 10
+    model = pd.Model(tensor_format="NCHW", batch_size=n)
+    model.add(pd.Input(shape=(16, 16, 3)))
+    for nf in (8, 8):
+        model.add(pd.Conv2D(nfilters=nf, filter_shape=(3, 3), padding=1, activation="relu",
+                            weights_initializer="he_normal"))
+    model.add(pd.MaxPool2D(pool_shape=(2, 2), stride=2))
+    model.add(pd.Conv2D(nfilters=16, filter_shape=(3, 3), padding=1, activation="relu",
+                        weights_initializer="he_normal"))
+    model.add(pd.MaxPool2D(pool_shape=(2, 2), stride=2))
+    model.add(pd.Flatten())
+    model.add(pd.FC(shape=(32,), activation="relu", weights_initializer="he_normal"))
+    model.add(pd.FC(shape=(classes,), activation="softmax", weights_initializer="he_normal"))
+    assert model.layers[1].need_dx is False and model.layers[3].need_dx is True  # pydtnn/model.py:270
+    x = rng.random((n, 3, 16, 16)).astype(np.float32)
+    labels = rng.integers(0, classes, n)
+    y_targ = np.eye(classes, dtype=np.float32)[labels]
+    params = {l.id: (host(l.weights).copy(), host(l.biases).copy()) for l in model.layers if l.grad_vars}
+
+    loss = model.train_batch(dev(x), dev(y_targ), pd.CategoricalCrossEntropy(), pd.SGD(learning_rate=0.01, momentum=0.9))
+
+    # ---- oracle chain
+    p3 = oracle.ConvParams(3, 3, 1, 1)
+    acts, cur = [], x
+    for l in model.layers[1:]:
+        name = l.canonical_name
+        if name == "Conv2D":
+            w, b = params[l.id]
+            y, cols = oracle.conv2d_forward_nchw_i2c(cur, w, b, p3)
+            acts.append(("conv", l, cur.shape, cols))
+            cur = y
+        elif name == "Relu":
+            cur, mask = oracle.relu(cur)
+            acts.append(("relu", l, mask))
+        elif name == "MaxPool2D":
+            shp = cur.shape
+            cur, idx = oracle.max_pool_2d_fwd_nchw(cur, 2, 2, 0, 0, 2, 2)
+            acts.append(("pool", l, shp, idx))
+        elif name == "Flatten":
+            acts.append(("flat", l, cur.shape))
+            cur = cur.reshape(n, -1)
+        elif name == "FC":
+            w, b = params[l.id]
+            acts.append(("fc", l, cur))
+            cur = oracle.fc_forward(cur, w, b)
+        elif name == "Softmax":
+            cur = oracle.softmax_forward(cur)
+            acts.append(("softmax", l, cur))
+    loss_ref, dcur = oracle.categorical_cross_entropy(cur, y_targ, n)
+    assert abs(float(loss) - loss_ref) <= 1e-4 * abs(loss_ref)
+    for kind, l, *saved in reversed(acts):
+        if kind == "softmax":
+            dcur = oracle.softmax_backward(dcur, saved[0])
+        elif kind == "fc":
+            w, b = params[l.id]
+            dw, db, dcur = oracle.fc_backward(dcur, saved[0], w)
+            assert_close(host(l.dw), dw, what=f"{l} dw")
+            assert_close(host(l.db), db, tol=1e-5, what=f"{l} db")
+            w_new, _ = oracle.sgd_update(w.copy(), dw, np.zeros_like(w), np.float32(0.01), np.float32(0.9))
+            assert_close(host(l.weights), w_new, tol=1e-5, what=f"{l} updated weights")
+        elif kind == "flat":
+            dcur = dcur.reshape(saved[0])
+        elif kind == "pool":
+            shp, idx = saved
+            dcur = oracle.max_pool_2d_bwd_nchw(dcur, idx, *shp, 2, 2, 0, 0, 2, 2)
+        elif kind == "relu":
+            dcur = dcur * saved[0]
+        elif kind == "conv":
+            w, b = params[l.id]
+            shp, cols = saved
+            dw, db, dx = oracle.conv2d_backward_nchw_i2c(dcur, cols, w, shp, p3, need_dx=l.need_dx)
+            assert_close(host(l.dw), dw, what=f"{l} dw")
+            assert_close(host(l.db), db, tol=1e-5, what=f"{l} db")
+            w_new, _ = oracle.sgd_update(w.copy(), dw, np.zeros_like(w), np.float32(0.01), np.float32(0.9))
+            assert_close(host(l.weights), w_new, tol=1e-5, what=f"{l} updated weights")
+            dcur = dx
