@@ -121,21 +121,29 @@ inline bool bn_args_consistent(const float* mean, const float* inv_std, const fl
 }
 
 template <int BMN, bool SEG>
-inline PlainK<BMN, SEG> plain_k(const float* base, long ld, long image_stride, long extent, int seg_len)
+inline PlainK<BMN, SEG> plain_k(const float* base, long total, long ld, long image_stride, long extent, int seg_len)
 {
     PlainK<BMN, SEG> l;
-    l.base = base; l.ld = ld; l.image_stride = image_stride; l.extent = (int)extent;
+    l.base = base; l.total = total; l.ld = ld; l.image_stride = image_stride; l.extent = (int)extent;
     l.seg_len = seg_len; l.fd_seg = make_fastdiv((uint32_t)(seg_len > 0 ? seg_len : 1));
     return l;
 }
 
 template <int BMN>
-inline PlainMN<BMN> plain_mn(const float* base, long ld, long image_stride, long extent)
+inline PlainMN<BMN> plain_mn(const float* base, long total, long ld, long image_stride, long extent)
 {
     PlainMN<BMN> l;
-    l.base = base; l.ld = ld; l.image_stride = image_stride; l.extent = (int)extent;
+    l.base = base; l.total = total; l.ld = ld; l.image_stride = image_stride; l.extent = (int)extent;
     return l;
 }
+
+// Buffer descriptors span less than 2 GiB: a K-major operand needs its tile rows (plus the images of
+// one reduction group) inside that span, an MN-major operand one step of BK rows.
+inline bool span_ok_k(long tile_rows, long ld, long group_images, long image_stride)
+{
+    return (tile_rows * ld + group_images * image_stride) * 4 < kMaxSpanBytes;
+}
+inline bool span_ok_mn(long ld) { return (long)BK * ld * 4 < kMaxSpanBytes; }
 
 inline EpiPlain epi_plain(float* out, long ldc, long split_stride, long m, long n, const ChanEpilogue& chan)
 {
@@ -158,7 +166,8 @@ int conv_fwd_nchw(const ConvGeom& g, const float* w, const float* x, float* y, c
     const TileSel sel = pick_tile(g.kn, g.p);
     int rc = PYDTNN_HIP_OK;
     WITH_TILE(sel, {
-        auto al = plain_k<T::BM, false>(w, g.k, 0, g.kn, 0);
+        if (!span_ok_k(T::BM, g.k, 0, 0)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+        auto al = plain_k<T::BM, false>(w, (long)g.kn * g.k, g.k, 0, g.kn, 0);
         Im2colNchwMN<T::BN> bl;
         bl.x = x; bl.g = g;
         rc = launch<T>(al, bl, epi_nchw(y, g.kn, g.howo, g.p, chan), g.kn, g.p, no_split(g.k), 1, stream);
@@ -200,11 +209,14 @@ int conv_dw_nchw(const ConvGeom& g, const float* dy, const float* x, const float
     int rc = PYDTNN_HIP_OK;
     WITH_TILE(sel, {
         // A(m = filter, k = (image, pixel)) = dy[image][filter][pixel]
-        auto al = plain_k<T::BM, true>(dy, g.howo, (long)g.kn * g.howo, g.kn, g.howo);
+        const long dy_img = (long)g.kn * g.howo;
+        if (!span_ok_k(T::BM, g.howo, sp.si.ips, dy_img)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+        auto al = plain_k<T::BM, true>(dy, g.p * g.kn, g.howo, dy_img, g.kn, g.howo);
         const EpiPlain ep = epi_plain(ws, g.k, out_elems, g.kn, g.k, no_epilogue());
         if (cols) {
             // B(k = (image, pixel), n = row of cols) = cols[n][image*howo + pixel]
-            auto bl = plain_k<T::BN, true>(cols, g.p, g.howo, g.k, g.howo);
+            if (!span_ok_k(T::BN, g.p, sp.si.ips, g.howo)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+            auto bl = plain_k<T::BN, true>(cols, (long)g.k * g.p, g.p, g.howo, g.k, g.howo);
             rc = launch<T>(al, bl, ep, g.kn, g.k, sp.si, sp.splits, stream);
         } else {
             Im2colNchwK<T::BN> bl;
@@ -226,11 +238,11 @@ int conv_dw_nhwc(const ConvGeom& g, const float* dy, const float* x, const float
     int rc = PYDTNN_HIP_OK;
     WITH_TILE(sel, {
         // B(k = (image, pixel), n = filter) = dy[(image*howo + pixel)*kn + n]
-        auto bl = plain_mn<T::BN>(dy, g.kn, (long)g.howo * g.kn, g.kn);
+        auto bl = plain_mn<T::BN>(dy, g.p * g.kn, g.kn, (long)g.howo * g.kn, g.kn);
         const EpiPlain ep = epi_plain(ws, g.kn, out_elems, g.k, g.kn, no_epilogue());
         if (rows) {
             // A(m = column of rows, k) = rows[(image*howo + pixel)*K + m]
-            auto al = plain_mn<T::BM>(rows, g.k, (long)g.howo * g.k, g.k);
+            auto al = plain_mn<T::BM>(rows, g.p * g.k, g.k, (long)g.howo * g.k, g.k);
             rc = launch<T>(al, bl, ep, g.k, g.kn, sp.si, sp.splits, stream);
         } else {
             Im2rowNhwcMN<T::BM> al;
@@ -267,7 +279,7 @@ int conv_dx_i2c(const ConvGeom& g, int nhwc, const float* w, const float* dy, fl
         if (rc != PYDTNN_HIP_OK) return rc;
         const TileSel sel = pick_tile(g.k, g.p);
         WITH_TILE(sel, {
-            auto al = plain_mn<T::BM>(w, g.k, 0, g.k);
+            auto al = plain_mn<T::BM>(w, (long)g.kn * g.k, g.k, 0, g.k);
             Im2colNchwMN<T::BN> bl;
             bl.x = dy; bl.g = g1;
             rc = launch<T>(al, bl, epi_plain(ws, g.p, 0, g.k, g.p, no_epilogue()), g.k, g.p, no_split(g.kn), 1,
@@ -279,8 +291,8 @@ int conv_dx_i2c(const ConvGeom& g, int nhwc, const float* w, const float* dy, fl
     // res(P x K) = dy_rows (P x kn) * W_rows^T : B(kk = filter, n = k) = w[n*kn + kk]
     const TileSel sel = pick_tile(g.p, g.k);
     WITH_TILE(sel, {
-        auto al = plain_k<T::BM, false>(dy, g.kn, 0, g.p, 0);
-        auto bl = plain_k<T::BN, false>(w, g.kn, 0, g.k, 0);
+        auto al = plain_k<T::BM, false>(dy, g.p * g.kn, g.kn, 0, g.p, 0);
+        auto bl = plain_k<T::BN, false>(w, (long)g.k * g.kn, g.kn, 0, g.k, 0);
         rc = launch<T>(al, bl, epi_plain(ws, g.k, 0, g.p, g.k, no_epilogue()), g.p, g.k, no_split(g.kn), 1, stream);
     })
     if (rc != PYDTNN_HIP_OK) return rc;
@@ -424,20 +436,26 @@ int pydtnn_hip_sgemm(int transa, int transb, long m, long n, long k, const float
     }
     const hipStream_t st = as_stream(stream);
     int rc = PYDTNN_HIP_OK;
+    // floats reachable from each base pointer (last row may be shorter than its leading dimension)
+    const long a_total = transa ? (k - 1) * lda + m : (m - 1) * lda + k;
+    const long b_total = transb ? (n - 1) * ldb + k : (k - 1) * ldb + n;
     WITH_TILE(sel, {
         const EpiPlain ep = epi_plain(dst, dst_ld, m * n, m, n, gemm_chan);
+        if ((!transa && !span_ok_k(T::BM, lda, 0, 0)) || (transa && !span_ok_mn(lda)) ||
+            (transb && !span_ok_k(T::BN, ldb, 0, 0)) || (!transb && !span_ok_mn(ldb)))
+            return PYDTNN_HIP_ERR_UNSUPPORTED;
         if (!transa && !transb)
-            rc = launch<T>(plain_k<T::BM, false>(a, lda, 0, m, 0), plain_mn<T::BN>(b, ldb, 0, n), ep, m, n, sp.si,
-                           sp.splits, st);
+            rc = launch<T>(plain_k<T::BM, false>(a, a_total, lda, 0, m, 0), plain_mn<T::BN>(b, b_total, ldb, 0, n), ep,
+                           m, n, sp.si, sp.splits, st);
         else if (!transa && transb)
-            rc = launch<T>(plain_k<T::BM, false>(a, lda, 0, m, 0), plain_k<T::BN, false>(b, ldb, 0, n, 0), ep, m, n,
-                           sp.si, sp.splits, st);
+            rc = launch<T>(plain_k<T::BM, false>(a, a_total, lda, 0, m, 0),
+                           plain_k<T::BN, false>(b, b_total, ldb, 0, n, 0), ep, m, n, sp.si, sp.splits, st);
         else if (transa && !transb)
-            rc = launch<T>(plain_mn<T::BM>(a, lda, 0, m), plain_mn<T::BN>(b, ldb, 0, n), ep, m, n, sp.si, sp.splits,
-                           st);
+            rc = launch<T>(plain_mn<T::BM>(a, a_total, lda, 0, m), plain_mn<T::BN>(b, b_total, ldb, 0, n), ep, m, n,
+                           sp.si, sp.splits, st);
         else
-            rc = launch<T>(plain_mn<T::BM>(a, lda, 0, m), plain_k<T::BN, false>(b, ldb, 0, n, 0), ep, m, n, sp.si,
-                           sp.splits, st);
+            rc = launch<T>(plain_mn<T::BM>(a, a_total, lda, 0, m), plain_k<T::BN, false>(b, b_total, ldb, 0, n, 0), ep,
+                           m, n, sp.si, sp.splits, st);
     })
     if (rc != PYDTNN_HIP_OK || sp.splits == 1) return rc;
     if (ldc != n) return PYDTNN_HIP_ERR_UNSUPPORTED;  // the split reduction writes a dense C
@@ -528,13 +546,16 @@ int pydtnn_hip_conv_i2c_forward(int nhwc, int b, int c, int h, int w, int kn, in
     if (!nhwc) {
         const TileSel sel = pick_tile(g.kn, g.p);
         WITH_TILE(sel, {
-            rc = launch<T>(plain_k<T::BM, false>(weights, g.k, 0, g.kn, 0), plain_mn<T::BN>(mat, g.p, 0, g.p),
+            if (!span_ok_mn(g.p)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+            rc = launch<T>(plain_k<T::BM, false>(weights, (long)g.kn * g.k, g.k, 0, g.kn, 0),
+                           plain_mn<T::BN>(mat, (long)g.k * g.p, g.p, 0, g.p),
                            epi_nchw(y, g.kn, g.howo, g.p, chan), g.kn, g.p, no_split(g.k), 1, st);
         })
     } else {
         const TileSel sel = pick_tile(g.p, g.kn);
         WITH_TILE(sel, {
-            rc = launch<T>(plain_k<T::BM, false>(mat, g.k, 0, g.p, 0), plain_mn<T::BN>(weights, g.kn, 0, g.kn),
+            rc = launch<T>(plain_k<T::BM, false>(mat, g.p * g.k, g.k, 0, g.p, 0),
+                           plain_mn<T::BN>(weights, (long)g.k * g.kn, g.kn, 0, g.kn),
                            epi_plain(y, g.kn, 0, g.p, g.kn, chan), g.p, g.kn, no_split(g.k), 1, st);
         })
     }

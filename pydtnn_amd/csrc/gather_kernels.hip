@@ -185,9 +185,14 @@ int make_conv_geom(ConvGeom* g, int n, int c, int h, int w, int kn, int kh, int 
     g->p = (long)n * howo;
     // The kernels index x, y and one image's pixels with 32-bit ints and divide k, pixel and
     // channel indices with FastDiv; refuse extents those do not cover.
-    const long lim = 1l << 31;
+    // Tensors are addressed through buffer descriptors of less than 2 GiB (2^29 floats), and the
+    // loaders pack tap / pixel offsets into 16-bit fields.
+    const long lim = 1l << 29;
     if (k >= (1l << 24) || howo >= (1l << 24) || (long)n * c * h * w >= lim || g->p * kn >= lim ||
         (long)kn * k >= lim)
+        return PYDTNN_HIP_ERR_UNSUPPORTED;
+    if (h + 2 * vpadding >= 8192 || w + 2 * hpadding >= 8192 || (kh - 1) * vdilation >= 8192 ||
+        (kw - 1) * hdilation >= 8192)
         return PYDTNN_HIP_ERR_UNSUPPORTED;
     g->k = (int)k;
     g->howo = (int)howo;
