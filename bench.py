@@ -25,9 +25,10 @@ METRIC = "conv GFLOP/s & % fp32 MFMA peak (3x3 VGG layer); VGG16 train img/s, 1 
 FP32_MFMA_PEAK_TFLOPS = 157.3   # 256 CU x 2.4 GHz x 256 FLOP/clk/CU
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per launch of the forward kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
-# (see profiles/); None until measured for the workload.
-MEASURED_TRAFFIC_BYTES = {"cfg2": None}
+# HBM-side bytes per launch of the forward kernel, from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE), each
+# scaled by what the same counter reads for a 256 MiB copy (factors 2.000 and 1.000):
+# (191273.3 * 2.0 + 200704.0) KiB.  The summary of those runs is profiles/cfg2_conv3x3_pmc_counters.md.
+MEASURED_TRAFFIC_BYTES = {"cfg2": int((191273.3 * 2.0 + 200704.0) * 1024)}
 
 
 def parse_args():
@@ -38,6 +39,9 @@ def parse_args():
     ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-vgg16", action="store_true", help="skip the VGG16 training-step extra of the default run")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch a plain 256 MiB device copy (chan_eltwise_vec4_kernel with no epilogue) three "
+                         "times, so that rocprofv3 FETCH_SIZE / WRITE_SIZE readings can be scaled to bytes")
     return ap.parse_args()
 
 
@@ -159,26 +163,33 @@ def run_cfg2(torch, pd, args):
     return ms, step_flop / (ms * 1e-3) / 1e9, workload, roofline, extra
 
 
-def cpu_baseline_cfg2(sample_images=16):
+def cpu_baseline_cfg2(sample_images=64, reps=8):
     """The reference's CPU route (im2col -> NumPy @ -> bias add -> 1023 transpose; backward likewise) restated
-    by the oracle, timed on this host on `sample_images` of the 64 images."""
+    by the oracle and timed on this host.  BLAS and OpenMP are both held to `cores` threads."""
     import numpy as np
+    from threadpoolctl import threadpool_limits
     from oracle import cpu_ref
+    cores = int(os.environ.get("OMP_NUM_THREADS", min(16, os.cpu_count() or 1)))
     x, w, b, dy = make_cfg2(sample_images)
     p = cpu_ref.ConvParams(3, 3, 1, 1)
-    best = None
-    for it in range(3):
-        t0 = time.perf_counter()
-        y, x_cols = cpu_ref.conv2d_forward_nchw_i2c(x, w, b, p)
-        cpu_ref.conv2d_backward_nchw_i2c(dy, x_cols, w, x.shape, p)
-        dt = time.perf_counter() - t0
-        if it > 0:
-            best = dt if best is None else min(best, dt)
+    times = []
+    budget = time.perf_counter() + 30.0
+    with threadpool_limits(limits=cores):
+        for it in range(reps + 1):
+            t0 = time.perf_counter()
+            y, x_cols = cpu_ref.conv2d_forward_nchw_i2c(x, w, b, p)
+            cpu_ref.conv2d_backward_nchw_i2c(dy, x_cols, w, x.shape, p)
+            if it > 0:
+                times.append(time.perf_counter() - t0)
+            del y, x_cols
+            if time.perf_counter() > budget and times:
+                break
+    best = min(times)
     flop = 3 * 2.0 * 256 * 2304 * sample_images * 56 * 56
-    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
     return {"value": round(flop / best / 1e9, 1), "unit": "GFLOP/s", "cores": cores, "kind": "port",
-            "sample": f"{sample_images} of 64 images of cfg2, fwd+dW+db+dX, 1 warm-up then best of 2 "
-                      f"({best:.2f} s); C/OpenMP im2col+col2im, NumPy(OpenBLAS) matmul"}
+            "sample": f"{sample_images} of 64 images of cfg2, fwd+dW+db+dX, 1 warm-up then best of {len(times)} "
+                      f"({best:.2f} s each, {sum(times):.1f} s in all); C/OpenMP im2col+col2im and NumPy(OpenBLAS) "
+                      f"matmul limited to {cores} threads"}
 
 
 def build_vgg16(pd, n=64):
@@ -254,6 +265,15 @@ def main():
     else:
         from bench_configs import run_other
         ms, value, unit, workload, roofline, extra = run_other(torch, pd, args, Timer, timed_steps)
+
+    if args.copy_calibration:
+        from pydtnn_amd import ops
+        src = torch.ones(64 * 1024 * 1024, device="cuda")  # 256 MiB read + 256 MiB written per launch
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            ops.chan_eltwise(src, channels=1, inner=1, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
 
     cpu = None
     if not args.no_cpu_baseline and args.workload == "cfg2":
