@@ -11,11 +11,13 @@
 #define PYDTNN_HIP_ERR_LAUNCH 3       // HIP reported a launch/runtime error
 #define PYDTNN_HIP_ERR_UNSUPPORTED 4  // extents beyond what the index arithmetic covers
 
-// Division of a small unsigned by a run-time constant as one mul-hi.
+// Division of a small unsigned by a run-time constant as one mul-hi, branch-free.
 // Exact for every n with n * div < 2^32 (checked on the host before a launch).
+// div == 1 has no 32-bit multiplier; it is handled by mul = 0 and pass = all ones (q = 0 + n).
 struct FastDiv {
     uint32_t mul;
     uint32_t div;
+    uint32_t pass;
 };
 
 static inline FastDiv make_fastdiv(uint32_t d)
@@ -23,12 +25,13 @@ static inline FastDiv make_fastdiv(uint32_t d)
     FastDiv f;
     f.div = d;
     f.mul = d <= 1 ? 0u : (uint32_t)(((1ull << 32) + d - 1) / d);
+    f.pass = d <= 1 ? 0xffffffffu : 0u;
     return f;
 }
 
 __device__ __forceinline__ uint32_t fd_div(uint32_t n, const FastDiv f)
 {
-    return f.div == 1 ? n : __umulhi(n, f.mul);
+    return __umulhi(n, f.mul) + (n & f.pass);
 }
 
 // Geometry of one convolution. Names follow PyDTNN's Conv2D (vpadding = vertical padding, ...).

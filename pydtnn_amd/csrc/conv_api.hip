@@ -160,17 +160,47 @@ inline EpiNchw epi_nchw(float* out, int channels, int howo, long p, const ChanEp
 }
 
 // ---------------------------------------------------------------- forward (implicit)
-int conv_fwd_nchw(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan,
-                  hipStream_t stream)
+// The padding test works on tap masks of 31 usable bits: one word over i*kw + j when kh*kw <= 31,
+// otherwise one word per axis.
+inline bool taps_supported(const ConvGeom& g) { return g.kh <= 31 && g.kw <= 31; }
+inline bool taps_wide(const ConvGeom& g) { return g.khw > 31; }
+
+template <bool WIDE>
+int conv_fwd_nchw_t(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan,
+                    hipStream_t stream)
 {
     const TileSel sel = pick_tile(g.kn, g.p);
     int rc = PYDTNN_HIP_OK;
     WITH_TILE(sel, {
         if (!span_ok_k(T::BM, g.k, 0, 0)) return PYDTNN_HIP_ERR_UNSUPPORTED;
         auto al = plain_k<T::BM, false>(w, (long)g.kn * g.k, g.k, 0, g.kn, 0);
-        Im2colNchwMN<T::BN> bl;
+        Im2colNchwMN<T::BN, WIDE> bl;
         bl.x = x; bl.g = g;
         rc = launch<T>(al, bl, epi_nchw(y, g.kn, g.howo, g.p, chan), g.kn, g.p, no_split(g.k), 1, stream);
+    })
+    return rc;
+}
+
+int conv_fwd_nchw(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan,
+                  hipStream_t stream)
+{
+    if (!taps_supported(g)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+    return taps_wide(g) ? conv_fwd_nchw_t<true>(g, w, x, y, chan, stream)
+                        : conv_fwd_nchw_t<false>(g, w, x, y, chan, stream);
+}
+
+template <bool WIDE>
+int conv_fwd_nhwc_t(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan,
+                    hipStream_t stream)
+{
+    const TileSel sel = pick_tile(g.p, g.kn);
+    int rc = PYDTNN_HIP_OK;
+    WITH_TILE(sel, {
+        Im2rowNhwcK<T::BM, WIDE> al;
+        al.x = x; al.g = g;
+        FilterNhwcMN<T::BN> bl;
+        bl.w = w; bl.g = g;
+        rc = launch<T>(al, bl, epi_plain(y, g.kn, 0, g.p, g.kn, chan), g.p, g.kn, no_split(g.k), 1, stream);
     })
     return rc;
 }
@@ -178,16 +208,9 @@ int conv_fwd_nchw(const ConvGeom& g, const float* w, const float* x, float* y, c
 int conv_fwd_nhwc(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan,
                   hipStream_t stream)
 {
-    const TileSel sel = pick_tile(g.p, g.kn);
-    int rc = PYDTNN_HIP_OK;
-    WITH_TILE(sel, {
-        Im2rowNhwcK<T::BM> al;
-        al.x = x; al.g = g;
-        FilterNhwcMN<T::BN> bl;
-        bl.w = w; bl.g = g;
-        rc = launch<T>(al, bl, epi_plain(y, g.kn, 0, g.p, g.kn, chan), g.p, g.kn, no_split(g.k), 1, stream);
-    })
-    return rc;
+    if (!taps_supported(g)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+    return taps_wide(g) ? conv_fwd_nhwc_t<true>(g, w, x, y, chan, stream)
+                        : conv_fwd_nhwc_t<false>(g, w, x, y, chan, stream);
 }
 
 // ---------------------------------------------------------------- filter gradient

@@ -1,12 +1,14 @@
 // fp32 GEMM tile engine for gfx950 (CDNA4) on v_mfma_f32_32x32x2_f32.
 //
 // One workgroup = 256 threads = 4 wavefronts of 64 lanes.  It owns a BM x BN tile of C and walks
-// the reduction axis in steps of BK = 16.  A and B tiles are staged through LDS, double-buffered:
-// while the matrix cores consume tile t out of LDS, the global loads of tile t+1 are issued
-// *between* the MFMA groups of the same wavefront (a few loads after every four MFMAs), land in
-// registers, and are written to the other LDS buffer after the last MFMA, so there is one barrier
-// per step and a wavefront keeps the matrix pipe fed on its own.  Every wavefront owns a 64 x 64
-// sub-tile = 2 x 2 MFMA blocks of 32 x 32 (64 accumulator registers).
+// the reduction axis in steps of BK = 16.  A and B tiles are staged through LDS, double-buffered,
+// and through two register sets, so three tiles are in flight: while the matrix cores consume
+// tile t out of LDS, the global loads of tile t+2 are issued *between* the MFMA groups of the same
+// wavefront (a few loads after every four MFMAs) into one register set, and the other set -
+// tile t+1, loaded a whole step earlier - is written to the second LDS buffer after the last
+// MFMA.  There is one barrier per step, a load has a full step to arrive, and a wavefront keeps
+// the matrix pipe fed on its own.  Every wavefront owns a 64 x 64 sub-tile = 2 x 2 MFMA blocks of
+// 32 x 32 (64 accumulator registers).
 //
 // What A(m, k) and B(k, n) *are* is decided by loader policies: plain strided matrices, or an
 // implicit im2col / im2row view of an activation tensor that is never materialised.  What
@@ -20,8 +22,14 @@
 //     predicated: they only feed rows / columns of C that the epilogue never stores;
 //   * a descriptor never spans more than 2 GiB and its size is the true number of bytes left in
 //     the tensor, so a wrong offset reads 0 instead of faulting.
-// The loop body exists in a fast form (every reduction index of the step is valid) and a tail
-// form (predicated on k < kend); only the last step of a tile takes the tail form.
+// On this hardware a VALU instruction is not free next to MFMAs: each one takes matrix-pipe time
+// (8 per MFMA cost a quarter of the throughput), while scalar-ALU, LDS and memory instructions issue
+// beside them.  The loop is therefore written to need very few VALU instructions per step:
+//   * wave-uniform index arithmetic (tap decomposition of a reduction index) is done on the scalar ALU;
+//   * the padding test of an element is one bit-field extract from a per-thread tap mask that is
+//     computed once per tile, and invalid elements get their offset's top bit set with one more op;
+//   * MFMA operands are fetched from LDS with ds_read_b32 and 16-bit immediate offsets from one base
+//     register per operand (explicit instructions: the compiler would re-add a base per k-step).
 //
 // LDS tiles are kept as [k][m] and [k][n] with rows padded by 4 floats, so that an MFMA operand
 // fetch - lane l reads element (row l%32, k l/32) - is a conflict-free read of 32 consecutive
@@ -88,6 +96,61 @@ __device__ __forceinline__ float buf_load(rsrc_t r, uint32_t voff_bytes, uint32_
 
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
+// Byte offset for buf_load, pushed beyond every descriptor when `invalid_bit` is 1.
+__device__ __forceinline__ uint32_t guarded_offset(uint32_t invalid_bit, uint32_t byte_offset)
+{
+    return (invalid_bit << 31) | byte_offset;
+}
+
+// LDS byte address of a __shared__ object, and a read at a compile-time byte offset from it.  The
+// result may only be used after lds_wait().
+__device__ __forceinline__ uint32_t lds_addr(const float* p)
+{
+    return (uint32_t)(uintptr_t)((__attribute__((address_space(3))) const float*)p);
+}
+
+template <int OFF>
+__device__ __forceinline__ float lds_read(uint32_t addr)
+{
+    static_assert(OFF >= 0 && OFF < 65536, "ds_read_b32 takes a 16-bit byte offset");
+    float v;
+    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+    return v;
+}
+
+// Waits for every outstanding LDS read; the registers are passed through so that their uses cannot be
+// scheduled above the wait.
+template <int N>
+__device__ __forceinline__ void lds_wait(float (&a)[N])
+{
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]));
+#pragma unroll
+    for (int i = 1; i < N; ++i) asm volatile("" : "+v"(a[i]));
+}
+
+// Tap masks for the padding test.  Bit t of the returned word is 1 when tap t must read as zero.
+// Narrow form (kh*kw <= 31): one word over the combined tap index i*kw + j.  Wide form: one word over
+// i and one over j (kh, kw <= 31).  Bit 31 is always 1: reduction indices >= kend select it.
+__device__ __forceinline__ uint32_t tap_mask_combined(const ConvGeom& g, int ih0, int iw0)
+{
+    uint32_t inv = 0xffffffffu;
+    for (int t = 0; t < g.khw; ++t) {
+        const int ii = t / g.kw, jj = t - ii * g.kw;
+        const bool ok = (unsigned)(ih0 + ii * g.vdilation) < (unsigned)g.h &&
+                        (unsigned)(iw0 + jj * g.hdilation) < (unsigned)g.w;
+        if (ok) inv &= ~(1u << t);
+    }
+    return inv;
+}
+
+__device__ __forceinline__ uint32_t tap_mask_axis(int first, int taps, int dilation, int extent)
+{
+    uint32_t inv = 0xffffffffu;
+    for (int t = 0; t < taps; ++t)
+        if ((unsigned)(first + t * dilation) < (unsigned)extent) inv &= ~(1u << t);
+    return inv;
+}
+
 // ---------------------------------------------------------------- thread -> element maps
 // MapMN: lanes run along the m (or n) axis of the tile; the k row is uniform per wavefront.
 template <int BMN>
@@ -124,9 +187,12 @@ struct MapK {
 //   State            per-thread data fixed for the whole tile
 //   Iter             per-thread / per-wave data of one reduction step
 //   init(State&, origin, image0, tid)
-//   begin<TAIL>(State, Iter&, k0, kend)      prepare the step that starts at reduction index k0
-//   elem<TAIL, E>(State, Iter, k0, kend)     value of this thread's E-th element of that step
+//   begin(State, Iter&, k0, kend)            prepare the step that starts at reduction index k0
+//   elem<E>(State, Iter, k0, kend)           value of this thread's E-th element of that step
 //   store(lds, regs, tid)
+// Reduction indices >= kend read as zero.  That test is made once per step (it is folded into the
+// step's tap / offset computation or into the size of the step's descriptor), never per element, so
+// the loop body has a single form for full and partial steps.
 
 // ---------------------------------------------------------------- plain strided loaders
 // elem(mn, k) = base[(image0 + k / seg)*image_stride + mn*ld + k % seg]   (k contiguous inside a segment)
@@ -162,7 +228,6 @@ struct PlainK {
             s.rowoff[e] = (uint32_t)(row * ld + Map::kk(tid)) * 4u;
         }
     }
-    template <bool TAIL>
     __device__ __forceinline__ void begin(const State&, Iter& it, int k0, int kend) const
     {
         const int k = k0 + Map::kk(threadIdx.x);
@@ -173,9 +238,9 @@ struct PlainK {
             it.voff = 0;
         }
         it.soff = (uint32_t)k0 * 4u;
-        if (TAIL && k >= kend) it.voff = kOob;
+        if (k >= kend) it.voff = kOob;
     }
-    template <bool TAIL, int E>
+    template <int E>
     __device__ __forceinline__ float elem(const State& s, const Iter& it, int, int) const
     {
         return buf_load(s.rsrc, s.rowoff[E] + it.voff, it.soff);
@@ -184,7 +249,8 @@ struct PlainK {
 };
 
 // elem(mn, k) = base[image*image_stride + k*ld + mn]   (mn contiguous).  The descriptor is re-based to
-// row k0 at every step, so only BK*ld*4 < 2 GiB is needed (checked on the host).
+// row k0 at every step and sized to end with row kend-1, so rows of a partial step beyond the
+// reduction range read as zero; only BK*ld*4 < 2 GiB is needed (checked on the host).
 template <int BMN>
 struct PlainMN {
     using Map = MapMN<BMN>;
@@ -208,52 +274,28 @@ struct PlainMN {
         s.voff = (uint32_t)min(origin + Map::mn(tid), extent - 1) * 4u;
         s.krow = Map::krow(tid);
     }
-    template <bool TAIL>
-    __device__ __forceinline__ void begin(const State& s, Iter& it, int k0, int) const
+    __device__ __forceinline__ void begin(const State& s, Iter& it, int k0, int kend) const
     {
-        const long row0 = s.first + (long)(k0 + s.krow) * ld;
-        it.rsrc = make_rsrc(base + row0, total - row0);
+        const int krow0 = k0 + s.krow;
+        const long row0 = s.first + (long)krow0 * ld;
+        const long in_range = (long)(kend - krow0) * ld;  // <= 0 when the whole step lies beyond kend
+        const long in_tensor = total - row0;
+        it.rsrc = make_rsrc(base + row0, in_range < in_tensor ? in_range : in_tensor);
     }
-    template <bool TAIL, int E>
-    __device__ __forceinline__ float elem(const State& s, const Iter& it, int k0, int kend) const
+    template <int E>
+    __device__ __forceinline__ float elem(const State& s, const Iter& it, int, int) const
     {
-        const uint32_t soff = (uint32_t)(E * Map::kRowsPerPass) * (uint32_t)ld * 4u;
-        uint32_t voff = s.voff;
-        if (TAIL && k0 + s.krow + E * Map::kRowsPerPass >= kend) voff = kOob;
-        return buf_load(it.rsrc, voff, soff);
+        return buf_load(it.rsrc, s.voff + (uint32_t)(E * Map::kRowsPerPass) * (uint32_t)ld * 4u, 0);
     }
     __device__ __forceinline__ void store(float* lds, const float (&r)[NLD], int tid) const { Map::store(lds, r, tid); }
 };
 
 // ---------------------------------------------------------------- implicit im2col, NCHW
-// Taps of one reduction step, decomposed by the lanes of a wavefront in parallel: lane l holds the
-// tap with reduction index k0 + (l % 16); a wave-uniform tap is then fetched with v_readlane.
-struct TapLanes {
-    int off;  // c*h*w + (i*dv)*w + j*dh  (float offset of the tap inside one image)
-    int dij;  // (i*dv) << 16 | (j*dh)
-};
-
-template <bool TAIL>
-__device__ __forceinline__ TapLanes nchw_taps(const ConvGeom& g, int k0, int kend)
-{
-    const uint32_t k = (uint32_t)(k0 + (threadIdx.x & (BK - 1)));
-    const uint32_t cc = fd_div(k, g.fd_khw);
-    const uint32_t rem = k - cc * g.khw;
-    const uint32_t ii = fd_div(rem, g.fd_kw);
-    const uint32_t jj = rem - ii * g.kw;
-    int di = (int)ii * g.vdilation;
-    const int dj = (int)jj * g.hdilation;
-    TapLanes t;
-    t.off = ((int)cc * g.h + di) * g.w + dj;
-    if (TAIL && (int)k >= kend) di = 0x4000;  // fails every row bound test (h + padding < 8192)
-    t.dij = (di << 16) | dj;
-    return t;
-}
-
 // B(k = (c,i,j), n = (img,y,x)) = X[img, c, sv*y + dv*i - pv, sh*x + dh*j - ph]: the column matrix of
 // pydtnn/cython_modules/im2col_nchw_cython.pyx:104-124, never written to memory.
-// Lanes run along the pixel axis (contiguous in x for a fixed tap); the tap (c,i,j) is wave-uniform.
-template <int BN>
+// Lanes run along the pixel axis (contiguous in x for a fixed tap); the tap (c,i,j) of an element is
+// wave-uniform and is decomposed on the scalar ALU.  WIDE selects the two-word tap mask.
+template <int BN, bool WIDE = false>
 struct Im2colNchwMN {
     using Map = MapMN<BN>;
     static constexpr int NLD = Map::NLD;
@@ -261,13 +303,12 @@ struct Im2colNchwMN {
     ConvGeom g;
     struct State {
         rsrc_t rsrc;
-        int base;  // float index of (img, c=0, ih0, iw0); may be negative, only used with an in-range tap
-        int ih0, iw0;
+        uint32_t base;   // byte offset of (img, c=0, ih0, iw0), modulo 2^32; only used with a valid tap
+        uint32_t inv0;   // narrow: combined tap mask; wide: mask over i
+        uint32_t inv1;   // wide: mask over j
         int krow;
     };
-    struct Iter {
-        TapLanes taps;
-    };
+    struct Iter {};
     __device__ __forceinline__ void init(State& s, int origin, int /*image*/, int tid) const
     {
         s.rsrc = make_rsrc(x, (long)g.n * g.c * g.h * g.w);
@@ -276,25 +317,36 @@ struct Im2colNchwMN {
         const int img = (int)(n / g.howo);
         const int pp = (int)(n - (long)img * g.howo);
         const int yy = pp / g.wo, xx = pp - yy * g.wo;
-        s.ih0 = yy * g.vstride - g.vpadding;
-        s.iw0 = xx * g.hstride - g.hpadding;
+        const int ih0 = yy * g.vstride - g.vpadding;
+        const int iw0 = xx * g.hstride - g.hpadding;
         s.krow = Map::krow(tid);
-        s.base = (img * g.c * g.h + s.ih0) * g.w + s.iw0;
+        s.base = (uint32_t)((img * g.c * g.h + ih0) * g.w + iw0) * 4u;
+        if (WIDE) {
+            s.inv0 = tap_mask_axis(ih0, g.kh, g.vdilation, g.h);
+            s.inv1 = tap_mask_axis(iw0, g.kw, g.hdilation, g.w);
+        } else {
+            s.inv0 = tap_mask_combined(g, ih0, iw0);
+            s.inv1 = 0;
+        }
     }
-    template <bool TAIL>
-    __device__ __forceinline__ void begin(const State&, Iter& it, int k0, int kend) const
+    __device__ __forceinline__ void begin(const State&, Iter&, int, int) const {}
+    template <int E>
+    __device__ __forceinline__ float elem(const State& s, const Iter&, int k0, int kend) const
     {
-        it.taps = nchw_taps<TAIL>(g, k0, kend);
-    }
-    template <bool TAIL, int E>
-    __device__ __forceinline__ float elem(const State& s, const Iter& it, int, int) const
-    {
-        const int lane = s.krow + E * Map::kRowsPerPass;
-        const int off = __builtin_amdgcn_readlane(it.taps.off, lane);
-        const int dij = __builtin_amdgcn_readlane(it.taps.dij, lane);
-        const int di = dij >> 16, dj = dij & 0xffff;
-        const bool ok = (unsigned)(s.ih0 + di) < (unsigned)g.h && (unsigned)(s.iw0 + dj) < (unsigned)g.w;
-        return buf_load(s.rsrc, ok ? (uint32_t)(s.base + off) * 4u : kOob, 0);
+        // scalar: reduction index -> (c, i, j) -> float offset of the tap inside one image
+        const uint32_t k = (uint32_t)(k0 + s.krow + E * Map::kRowsPerPass);
+        const uint32_t cc = fd_div(k, g.fd_khw);
+        const uint32_t rem = k - cc * g.khw;
+        const uint32_t ii = fd_div(rem, g.fd_kw);
+        const uint32_t jj = rem - ii * g.kw;
+        const uint32_t off = (uint32_t)(((int)cc * g.h + (int)ii * g.vdilation) * g.w + (int)jj * g.hdilation) * 4u;
+        const bool live = (int)k < kend;
+        uint32_t invalid;
+        if (WIDE)
+            invalid = __builtin_amdgcn_ubfe(s.inv0, live ? ii : 31u, 1) | __builtin_amdgcn_ubfe(s.inv1, jj, 1);
+        else
+            invalid = __builtin_amdgcn_ubfe(s.inv0, live ? rem : 31u, 1);
+        return buf_load(s.rsrc, guarded_offset(invalid, s.base + off), 0);
     }
     __device__ __forceinline__ void store(float* lds, const float (&r)[NLD], int tid) const { Map::store(lds, r, tid); }
 };
@@ -331,7 +383,6 @@ struct Im2colNchwK {
             s.coff[e] = (cc * g.h + s.di[e]) * g.w + s.dj[e];
         }
     }
-    template <bool TAIL>
     __device__ __forceinline__ void begin(const State& s, Iter& it, int k0, int kend) const
     {
         const int k = k0 + Map::kk(threadIdx.x);  // (image within the group, pixel)
@@ -342,9 +393,9 @@ struct Im2colNchwK {
         it.ih0 = (int)yy * g.vstride - g.vpadding;
         it.iw0 = (int)xx * g.hstride - g.hpadding;
         it.base = ((s.image0 + (int)img) * g.c * g.h + it.ih0) * g.w + it.iw0;
-        if (TAIL && k >= kend) it.ih0 = -(1 << 20);  // fails every bound test
+        if (k >= kend) it.ih0 = -(1 << 20);  // fails every bound test
     }
-    template <bool TAIL, int E>
+    template <int E>
     __device__ __forceinline__ float elem(const State& s, const Iter& it, int, int) const
     {
         const bool ok = (unsigned)(it.ih0 + s.di[E]) < (unsigned)g.h && (unsigned)(it.iw0 + s.dj[E]) < (unsigned)g.w;
@@ -358,20 +409,23 @@ struct Im2colNchwK {
 // in (i, j, c) order so that lanes along k read consecutive channels.  The reference orders K as
 // (c, i, j) (pydtnn/cython_modules/im2row_nhwc_cython.pyx:96); a sum over K does not depend on the
 // order, and the filter loader below applies the same permutation to the rows of W.
-template <int BM>
+template <int BM, bool WIDE = false>
 struct Im2rowNhwcK {
     using Map = MapK<BM>;
     static constexpr int NLD = Map::NLD;
+    static constexpr int NMASK1 = WIDE ? NLD : 1;
     const float* x;
     ConvGeom g;
     struct State {
         rsrc_t rsrc;
-        int base[NLD];  // ((img*h + ih0)*w + iw0)*c, may be negative when padding reaches outside
-        int ih0[NLD], iw0[NLD];
+        uint32_t base[NLD];    // byte offset of ((img*h + ih0)*w + iw0)*c, modulo 2^32
+        uint32_t inv0[NLD];    // narrow: combined tap mask of the row's pixel; wide: mask over i
+        uint32_t inv1[NMASK1]; // wide: mask over j
     };
     struct Iter {
-        int koff;  // (di*w + dj)*c + channel
-        int di, dj;
+        uint32_t koff;  // byte offset of (di*w + dj)*c + channel
+        uint32_t bit0;  // narrow: combined tap index (31 beyond kend); wide: i (31 beyond kend)
+        uint32_t bit1;  // wide: j
     };
     __device__ __forceinline__ void init(State& s, int origin, int /*image*/, int tid) const
     {
@@ -383,12 +437,17 @@ struct Im2rowNhwcK {
             const int img = (int)(m / g.howo);
             const int pp = (int)(m - (long)img * g.howo);
             const int yy = pp / g.wo, xx = pp - yy * g.wo;
-            s.ih0[e] = yy * g.vstride - g.vpadding;
-            s.iw0[e] = xx * g.hstride - g.hpadding;
-            s.base[e] = ((img * g.h + s.ih0[e]) * g.w + s.iw0[e]) * g.c;
+            const int ih0 = yy * g.vstride - g.vpadding;
+            const int iw0 = xx * g.hstride - g.hpadding;
+            s.base[e] = (uint32_t)(((img * g.h + ih0) * g.w + iw0) * g.c) * 4u;
+            if (WIDE) {
+                s.inv0[e] = tap_mask_axis(ih0, g.kh, g.vdilation, g.h);
+                s.inv1[e] = tap_mask_axis(iw0, g.kw, g.hdilation, g.w);
+            } else {
+                s.inv0[e] = tap_mask_combined(g, ih0, iw0);
+            }
         }
     }
-    template <bool TAIL>
     __device__ __forceinline__ void begin(const State&, Iter& it, int k0, int kend) const
     {
         const uint32_t k = (uint32_t)(k0 + Map::kk(threadIdx.x));
@@ -396,16 +455,17 @@ struct Im2rowNhwcK {
         const uint32_t cc = k - ij * g.c;
         const uint32_t ii = fd_div(ij, g.fd_kw);
         const uint32_t jj = ij - ii * g.kw;
-        it.di = (int)ii * g.vdilation;
-        it.dj = (int)jj * g.hdilation;
-        it.koff = (it.di * g.w + it.dj) * g.c + (int)cc;
-        if (TAIL && (int)k >= kend) it.di = 1 << 20;
+        it.koff = (uint32_t)(((int)ii * g.vdilation * g.w + (int)jj * g.hdilation) * g.c + (int)cc) * 4u;
+        const bool live = (int)k < kend;
+        it.bit0 = live ? (WIDE ? ii : ij) : 31u;
+        it.bit1 = jj;
     }
-    template <bool TAIL, int E>
+    template <int E>
     __device__ __forceinline__ float elem(const State& s, const Iter& it, int, int) const
     {
-        const bool ok = (unsigned)(s.ih0[E] + it.di) < (unsigned)g.h && (unsigned)(s.iw0[E] + it.dj) < (unsigned)g.w;
-        return buf_load(s.rsrc, ok ? (uint32_t)(s.base[E] + it.koff) * 4u : kOob, 0);
+        uint32_t invalid = __builtin_amdgcn_ubfe(s.inv0[E], it.bit0, 1);
+        if (WIDE) invalid |= __builtin_amdgcn_ubfe(s.inv1[E], it.bit1, 1);
+        return buf_load(s.rsrc, guarded_offset(invalid, s.base[E] + it.koff), 0);
     }
     __device__ __forceinline__ void store(float* lds, const float (&r)[NLD], int tid) const { Map::store(lds, r, tid); }
 };
@@ -422,31 +482,23 @@ struct FilterNhwcMN {
         uint32_t voff;
         int krow;
     };
-    struct Iter {
-        int row;  // per lane: filter row c*kh*kw + i*kw + j of reduction index k0 + lane%16
-    };
+    struct Iter {};
     __device__ __forceinline__ void init(State& s, int origin, int /*image*/, int tid) const
     {
         s.rsrc = make_rsrc(w, (long)g.k * g.kn);
         s.voff = (uint32_t)min(origin + Map::mn(tid), g.kn - 1) * 4u;
         s.krow = Map::krow(tid);
     }
-    template <bool TAIL>
-    __device__ __forceinline__ void begin(const State&, Iter& it, int k0, int) const
+    __device__ __forceinline__ void begin(const State&, Iter&, int, int) const {}
+    template <int E>
+    __device__ __forceinline__ float elem(const State& s, const Iter&, int k0, int kend) const
     {
-        const uint32_t k = (uint32_t)(k0 + (threadIdx.x & (BK - 1)));
+        // scalar: reduction index in (i,j,c) order -> filter row c*kh*kw + i*kw + j
+        const uint32_t k = (uint32_t)(k0 + s.krow + E * Map::kRowsPerPass);
         const uint32_t ij = fd_div(k, g.fd_c);
         const uint32_t cc = k - ij * g.c;
-        it.row = (int)(cc * g.khw + ij);
-    }
-    template <bool TAIL, int E>
-    __device__ __forceinline__ float elem(const State& s, const Iter& it, int k0, int kend) const
-    {
-        const int lane = s.krow + E * Map::kRowsPerPass;
-        const uint32_t row = (uint32_t)__builtin_amdgcn_readlane(it.row, lane);
-        uint32_t voff = s.voff;
-        if (TAIL && k0 + lane >= kend) voff = kOob;
-        return buf_load(s.rsrc, voff, row * (uint32_t)g.kn * 4u);
+        const uint32_t rowoff = (int)k < kend ? (cc * g.khw + ij) * (uint32_t)g.kn * 4u : kOob;
+        return buf_load(s.rsrc, s.voff + rowoff, 0);
     }
     __device__ __forceinline__ void store(float* lds, const float (&r)[NLD], int tid) const { Map::store(lds, r, tid); }
 };
@@ -466,10 +518,7 @@ struct Im2rowNhwcMN {
         int krow;
         int image0;
     };
-    struct Iter {
-        int pix;  // per lane: (img*h + ih0)*w + iw0 of reduction index k0 + lane%16 (may be negative)
-        int ihw;  // per lane: (ih0 + 0x4000) << 16 | (iw0 + 0x4000)
-    };
+    struct Iter {};
     __device__ __forceinline__ void init(State& s, int origin, int image0, int tid) const
     {
         s.rsrc = make_rsrc(x, (long)g.n * g.c * g.h * g.w);
@@ -482,27 +531,19 @@ struct Im2rowNhwcMN {
         s.krow = Map::krow(tid);
         s.image0 = image0;
     }
-    template <bool TAIL>
-    __device__ __forceinline__ void begin(const State& s, Iter& it, int k0, int kend) const
+    __device__ __forceinline__ void begin(const State&, Iter&, int, int) const {}
+    template <int E>
+    __device__ __forceinline__ float elem(const State& s, const Iter&, int k0, int kend) const
     {
-        const uint32_t k = (uint32_t)(k0 + (threadIdx.x & (BK - 1)));  // (image within the group, pixel)
+        // scalar: reduction index -> (image within the group, y, x) -> first input row / column of the window
+        const uint32_t k = (uint32_t)(k0 + s.krow + E * Map::kRowsPerPass);
         const uint32_t img = fd_div(k, g.fd_howo);
         const uint32_t pp = k - img * g.howo;
         const uint32_t yy = fd_div(pp, g.fd_wo);
         const uint32_t xx = pp - yy * g.wo;
-        int ih0 = (int)yy * g.vstride - g.vpadding;
+        const int ih0 = (int)k < kend ? (int)yy * g.vstride - g.vpadding : 0x2000;  // beyond kend: fails the row test
         const int iw0 = (int)xx * g.hstride - g.hpadding;
-        it.pix = ((s.image0 + (int)img) * g.h + ih0) * g.w + iw0;
-        if (TAIL && (int)k >= kend) ih0 = 0x2000;  // fails every row bound test (h < 8192)
-        it.ihw = ((ih0 + 0x4000) << 16) | (iw0 + 0x4000);
-    }
-    template <bool TAIL, int E>
-    __device__ __forceinline__ float elem(const State& s, const Iter& it, int, int) const
-    {
-        const int lane = s.krow + E * Map::kRowsPerPass;
-        const int pix = __builtin_amdgcn_readlane(it.pix, lane);
-        const int ihw = __builtin_amdgcn_readlane(it.ihw, lane);
-        const int ih0 = (ihw >> 16) - 0x4000, iw0 = (ihw & 0xffff) - 0x4000;
+        const int pix = ((s.image0 + (int)img) * g.h + ih0) * g.w + iw0;
         const bool ok = (unsigned)(ih0 + s.di) < (unsigned)g.h && (unsigned)(iw0 + s.dj) < (unsigned)g.w;
         return buf_load(s.rsrc, ok ? (uint32_t)(pix * g.c + s.moff) * 4u : kOob, 0);
     }
@@ -579,83 +620,90 @@ __device__ __forceinline__ int xcd_remap(int bid, int nblocks)
 
 // Loads of one reduction step are spread over the BK/2 MFMA groups of the step: group J issues the
 // elements E with E*(BK/2)/NLD == J.
-template <bool TAIL, int J, int E, class L>
+template <int J, int E, class L>
 __device__ __forceinline__ void group_load(const L& l, const typename L::State& s, const typename L::Iter& it,
                                            float (&r)[L::NLD], int k0, int kend)
 {
     if constexpr (E < L::NLD) {
-        if constexpr (E * (BK / 2) / L::NLD == J) r[E] = l.template elem<TAIL, E>(s, it, k0, kend);
-        group_load<TAIL, J, E + 1, L>(l, s, it, r, k0, kend);
+        if constexpr (E * (BK / 2) / L::NLD == J) r[E] = l.template elem<E>(s, it, k0, kend);
+        group_load<J, E + 1, L>(l, s, it, r, k0, kend);
     }
 }
 
-template <bool TAIL, int E, class L>
+template <int E, class L>
 __device__ __forceinline__ void load_all(const L& l, const typename L::State& s, const typename L::Iter& it,
                                          float (&r)[L::NLD], int k0, int kend)
 {
     if constexpr (E < L::NLD) {
-        r[E] = l.template elem<TAIL, E>(s, it, k0, kend);
-        load_all<TAIL, E + 1, L>(l, s, it, r, k0, kend);
+        r[E] = l.template elem<E>(s, it, k0, kend);
+        load_all<E + 1, L>(l, s, it, r, k0, kend);
     }
 }
 
-// One MFMA group (k-step J of the LDS tile) and everything scheduled around it.
-// LOADS: 0 = last step of the tile (nothing to prefetch), 1 = prefetch a full step, 2 = prefetch the tail step
-template <class T, int LOADS, int J, class AL, class BL>
+// MFMA operands of k-step J out of LDS buffer BUF: lane (r, h) of a wavefront holds A[m = 32*i + r][k = 2*J + h]
+// and B[k = 2*J + h][n = 32*j + r].  `a_base` / `b_base` are the LDS byte addresses of this lane's element of
+// buffer 0 at J = 0, i = j = 0; everything else is an immediate offset.
+template <class T, int BUF, int J>
+__device__ __forceinline__ void request_operands(uint32_t a_base, uint32_t b_base, float (&af)[T::TM], float (&bf)[T::TN])
+{
+    constexpr int a_off = (BUF * BK * (T::BM + kPad) + 2 * J * (T::BM + kPad)) * 4;
+    constexpr int b_off = (BUF * BK * (T::BN + kPad) + 2 * J * (T::BN + kPad)) * 4;
+    if constexpr (T::TM >= 1) af[0] = lds_read<a_off>(a_base);
+    if constexpr (T::TM >= 2) af[1] = lds_read<a_off + 128>(a_base);
+    if constexpr (T::TM >= 3) af[2] = lds_read<a_off + 256>(a_base);
+    if constexpr (T::TM >= 4) af[3] = lds_read<a_off + 384>(a_base);
+    if constexpr (T::TN >= 1) bf[0] = lds_read<b_off>(b_base);
+    if constexpr (T::TN >= 2) bf[1] = lds_read<b_off + 128>(b_base);
+    if constexpr (T::TN >= 3) bf[2] = lds_read<b_off + 256>(b_base);
+    if constexpr (T::TN >= 4) bf[3] = lds_read<b_off + 384>(b_base);
+    static_assert(T::TM <= 4 && T::TN <= 4, "operand fetch is written for up to 4 blocks per axis");
+}
+
+// One MFMA group (k-step J of the LDS tile) and everything scheduled around it: wait for its operands,
+// start the first MFMA, request the next group's operands, issue this group's share of the global loads,
+// then the remaining MFMAs.
+template <class T, int BUF, int J, class AL, class BL>
 __device__ __forceinline__ void mfma_groups(const AL& al, const BL& bl, const typename AL::State& as,
                                             const typename BL::State& bs, const typename AL::Iter& ai,
                                             const typename BL::Iter& bi, float (&ra)[AL::NLD], float (&rb)[BL::NLD],
-                                            const float* a_lds, const float* b_lds, floatx16 (&acc)[T::TM][T::TN],
+                                            uint32_t a_base, uint32_t b_base, floatx16 (&acc)[T::TM][T::TN],
                                             float (&af)[2][T::TM], float (&bf)[2][T::TN], int knext, int kend)
 {
     constexpr int G = BK / 2;
     if constexpr (J < G) {
-        if constexpr (J + 1 < G) {  // operands of the next group are fetched before this group's MFMAs issue
-#pragma unroll
-            for (int i = 0; i < T::TM; ++i) af[(J + 1) & 1][i] = a_lds[2 * (J + 1) * (T::BM + kPad) + i * 32];
-#pragma unroll
-            for (int j = 0; j < T::TN; ++j) bf[(J + 1) & 1][j] = b_lds[2 * (J + 1) * (T::BN + kPad) + j * 32];
-        }
-        if constexpr (LOADS == 1) {
-            group_load<false, J, 0, AL>(al, as, ai, ra, knext, kend);
-            group_load<false, J, 0, BL>(bl, bs, bi, rb, knext, kend);
-        } else if constexpr (LOADS == 2) {
-            group_load<true, J, 0, AL>(al, as, ai, ra, knext, kend);
-            group_load<true, J, 0, BL>(bl, bs, bi, rb, knext, kend);
-        }
+        lds_wait(af[J & 1]);
+        lds_wait(bf[J & 1]);
+        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[J & 1][0], bf[J & 1][0], acc[0][0], 0, 0, 0);
+        if constexpr (J + 1 < G) request_operands<T, BUF, J + 1>(a_base, b_base, af[(J + 1) & 1], bf[(J + 1) & 1]);
+        group_load<J, 0, AL>(al, as, ai, ra, knext, kend);
+        group_load<J, 0, BL>(bl, bs, bi, rb, knext, kend);
 #pragma unroll
         for (int i = 0; i < T::TM; ++i)
 #pragma unroll
             for (int j = 0; j < T::TN; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[J & 1][i], bf[J & 1][j], acc[i][j], 0, 0, 0);
+                if (i + j > 0)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[J & 1][i], bf[J & 1][j], acc[i][j], 0, 0, 0);
         // keep this group's LDS fetches, global loads and MFMAs together: the instruction scheduler
         // must not sink the loads to the end of the step
         __builtin_amdgcn_sched_barrier(0);
-        mfma_groups<T, LOADS, J + 1, AL, BL>(al, bl, as, bs, ai, bi, ra, rb, a_lds, b_lds, acc, af, bf, knext, kend);
+        mfma_groups<T, BUF, J + 1, AL, BL>(al, bl, as, bs, ai, bi, ra, rb, a_base, b_base, acc, af, bf, knext, kend);
     }
 }
 
-template <class T, int LOADS, class AL, class BL>
+// Consumes LDS buffer BUF and loads the tile that starts at reduction index knext into (ra, rb).
+template <class T, int BUF, class AL, class BL>
 __device__ __forceinline__ void step(const AL& al, const BL& bl, const typename AL::State& as,
                                      const typename BL::State& bs, float (&ra)[AL::NLD], float (&rb)[BL::NLD],
-                                     const float* a_lds, const float* b_lds, floatx16 (&acc)[T::TM][T::TN], int knext,
+                                     uint32_t a_base, uint32_t b_base, floatx16 (&acc)[T::TM][T::TN], int knext,
                                      int kend)
 {
     typename AL::Iter ai;
     typename BL::Iter bi;
-    if constexpr (LOADS == 1) {
-        al.template begin<false>(as, ai, knext, kend);
-        bl.template begin<false>(bs, bi, knext, kend);
-    } else if constexpr (LOADS == 2) {
-        al.template begin<true>(as, ai, knext, kend);
-        bl.template begin<true>(bs, bi, knext, kend);
-    }
     float af[2][T::TM], bf[2][T::TN];
-#pragma unroll
-    for (int i = 0; i < T::TM; ++i) af[0][i] = a_lds[i * 32];
-#pragma unroll
-    for (int j = 0; j < T::TN; ++j) bf[0][j] = b_lds[j * 32];
-    mfma_groups<T, LOADS, 0, AL, BL>(al, bl, as, bs, ai, bi, ra, rb, a_lds, b_lds, acc, af, bf, knext, kend);
+    request_operands<T, BUF, 0>(a_base, b_base, af[0], bf[0]);
+    al.begin(as, ai, knext, kend);
+    bl.begin(bs, bi, knext, kend);
+    mfma_groups<T, BUF, 0, AL, BL>(al, bl, as, bs, ai, bi, ra, rb, a_base, b_base, acc, af, bf, knext, kend);
 }
 
 template <class T, class AL, class BL, class EP>
@@ -681,7 +729,9 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(AL al, BL bl, EP ep, int
     al.init(as, m0, image, tid);
     bl.init(bs, n0, image, tid);
 
-    float ra[AL::NLD], rb[BL::NLD];
+    // Register sets: during step s the loads of tile s+2 go to set (s & 1) while set ((s+1) & 1),
+    // filled during step s-1 with tile s+1, is stored to LDS at the end of the step.
+    float ra0[AL::NLD], rb0[BL::NLD], ra1[AL::NLD], rb1[BL::NLD];
     floatx16 acc[T::TM][T::TN];
 #pragma unroll
     for (int i = 0; i < T::TM; ++i)
@@ -693,45 +743,36 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(AL al, BL bl, EP ep, int
     const int wave = tid >> 6, lane = tid & 63;
     const int wm0 = (wave % T::WGM) * T::WM, wn0 = (wave / T::WGM) * T::WN;
     const int frag_r = lane & 31, frag_k = lane >> 5;
+    const uint32_t a_base = lds_addr(&As[0][frag_k * (T::BM + kPad) + wm0 + frag_r]);
+    const uint32_t b_base = lds_addr(&Bs[0][frag_k * (T::BN + kPad) + wn0 + frag_r]);
 
-    {   // first tile: tail form (correct for any kend, including an empty range)
+    {   // tiles 0 and 1 (any kend, including an empty range: everything reads as zero)
         typename AL::Iter ai;
         typename BL::Iter bi;
-        al.template begin<true>(as, ai, kbeg, kend);
-        bl.template begin<true>(bs, bi, kbeg, kend);
-        load_all<true, 0, AL>(al, as, ai, ra, kbeg, kend);
-        load_all<true, 0, BL>(bl, bs, bi, rb, kbeg, kend);
+        al.begin(as, ai, kbeg, kend);
+        bl.begin(bs, bi, kbeg, kend);
+        load_all<0, AL>(al, as, ai, ra0, kbeg, kend);
+        load_all<0, BL>(bl, bs, bi, rb0, kbeg, kend);
+        al.begin(as, ai, kbeg + BK, kend);
+        bl.begin(bs, bi, kbeg + BK, kend);
+        load_all<0, AL>(al, as, ai, ra1, kbeg + BK, kend);
+        load_all<0, BL>(bl, bs, bi, rb1, kbeg + BK, kend);
     }
-    al.store(As[0], ra, tid);
-    bl.store(Bs[0], rb, tid);
+    al.store(As[0], ra0, tid);
+    bl.store(Bs[0], rb0, tid);
     __syncthreads();
 
-    // Steady state: the step being prefetched is a full one, so the loop body exists in one form.
-    int cur = 0;
-    int k0 = kbeg;
-    for (; k0 + 2 * BK <= kend; k0 += BK) {
-        const float* a_lds = As[cur] + frag_k * (T::BM + kPad) + wm0 + frag_r;
-        const float* b_lds = Bs[cur] + frag_k * (T::BN + kPad) + wn0 + frag_r;
-        step<T, 1>(al, bl, as, bs, ra, rb, a_lds, b_lds, acc, k0 + BK, kend);
-        al.store(As[cur ^ 1], ra, tid);
-        bl.store(Bs[cur ^ 1], rb, tid);
+    // Two steps per trip so that the register sets are named statically.  A reduction range with an
+    // odd number of steps runs one extra step on a tile that lies beyond kend and therefore is zero.
+    for (int k0 = kbeg; k0 < kend; k0 += 2 * BK) {
+        step<T, 0>(al, bl, as, bs, ra0, rb0, a_base, b_base, acc, k0 + 2 * BK, kend);
+        al.store(As[1], ra1, tid);
+        bl.store(Bs[1], rb1, tid);
         __syncthreads();
-        cur ^= 1;
-    }
-    if (k0 + BK < kend) {  // the next step is the partial one at the end of the reduction range
-        const float* a_lds = As[cur] + frag_k * (T::BM + kPad) + wm0 + frag_r;
-        const float* b_lds = Bs[cur] + frag_k * (T::BN + kPad) + wn0 + frag_r;
-        step<T, 2>(al, bl, as, bs, ra, rb, a_lds, b_lds, acc, k0 + BK, kend);
-        al.store(As[cur ^ 1], ra, tid);
-        bl.store(Bs[cur ^ 1], rb, tid);
+        step<T, 1>(al, bl, as, bs, ra1, rb1, a_base, b_base, acc, k0 + 3 * BK, kend);
+        al.store(As[0], ra0, tid);
+        bl.store(Bs[0], rb0, tid);
         __syncthreads();
-        cur ^= 1;
-        k0 += BK;
-    }
-    if (k0 < kend) {  // last step: nothing left to prefetch
-        const float* a_lds = As[cur] + frag_k * (T::BM + kPad) + wm0 + frag_r;
-        const float* b_lds = Bs[cur] + frag_k * (T::BN + kPad) + wn0 + frag_r;
-        step<T, 0>(al, bl, as, bs, ra, rb, a_lds, b_lds, acc, k0 + BK, kend);
     }
 
     // Accumulator layout of v_mfma_f32_32x32x2_f32: register v of lane l holds
