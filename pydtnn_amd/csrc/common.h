@@ -34,6 +34,13 @@ __device__ __forceinline__ uint32_t fd_div(uint32_t n, const FastDiv f)
     return __umulhi(n, f.mul) + (n & f.pass);
 }
 
+// The same quotient where the host could not prove n * div < 2^32: `exact` is a launch-wide flag,
+// so the branch is uniform and the hardware division is only paid by shapes that need it.
+__device__ __forceinline__ uint32_t fd_div_checked(uint32_t n, const FastDiv f, int exact)
+{
+    return exact ? fd_div(n, f) : n / f.div;
+}
+
 // Geometry of one convolution. Names follow PyDTNN's Conv2D (vpadding = vertical padding, ...).
 // Output extent: ho = (h + 2*vpadding - vdilation*(kh-1) - 1) / vstride + 1 (pydtnn/layers/conv_2d.py:75-76).
 struct ConvGeom {
@@ -46,6 +53,7 @@ struct ConvGeom {
     int howo;           // ho*wo
     long p;             // n*ho*wo  (pixels = GEMM columns in NCHW, rows in NHWC)
     FastDiv fd_khw, fd_kw, fd_wo, fd_c, fd_howo;
+    FastDiv fd_w, fd_kh, fd_vs, fd_hs;  // used by the streaming kernels (input-plane pixel, pool index, strides)
 };
 
 static inline int conv_out_dim(int in, int pad, int dil, int k, int stride)

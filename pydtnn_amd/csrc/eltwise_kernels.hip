@@ -56,24 +56,50 @@ __global__ void __launch_bounds__(kThreads) chan_eltwise_vec4_kernel(const float
 
 // ---------------------------------------------------------------- ReLU with mask
 // pydtnn/cython_modules/relu_cython.pyx:52-59 (strict x > 0); pydtnn/backends/cpu/activations/relu_cpu.py:38-40.
+// Four elements per thread (one 16-byte load, one 16-byte store, one 4-byte mask store) when the
+// pointers allow it; the last thread finishes a tail of up to three elements.
+template <bool VEC4>
 __global__ void __launch_bounds__(kThreads) relu_fwd_kernel(const float* __restrict__ x, float* __restrict__ y,
                                                            int8_t* __restrict__ mask, long total)
 {
-    const long idx = (long)blockIdx.x * kThreads + threadIdx.x;
+    const long idx = ((long)blockIdx.x * kThreads + threadIdx.x) * (VEC4 ? 4 : 1);
     if (idx >= total) return;
-    const float v = x[idx];
-    const bool pos = v > 0.0f;
-    y[idx] = pos ? v : 0.0f;
-    if (mask) mask[idx] = pos ? 1 : 0;
+    if (VEC4 && idx + 4 <= total) {
+        const float4 v = *reinterpret_cast<const float4*>(x + idx);
+        const bool p0 = v.x > 0.0f, p1 = v.y > 0.0f, p2 = v.z > 0.0f, p3 = v.w > 0.0f;
+        *reinterpret_cast<float4*>(y + idx) =
+            make_float4(p0 ? v.x : 0.0f, p1 ? v.y : 0.0f, p2 ? v.z : 0.0f, p3 ? v.w : 0.0f);
+        if (mask)
+            *reinterpret_cast<uint32_t*>(mask + idx) =
+                (uint32_t)p0 | ((uint32_t)p1 << 8) | ((uint32_t)p2 << 16) | ((uint32_t)p3 << 24);
+        return;
+    }
+    const long end = VEC4 ? total : idx + 1;
+    for (long i = idx; i < end; ++i) {
+        const float v = x[i];
+        const bool pos = v > 0.0f;
+        y[i] = pos ? v : 0.0f;
+        if (mask) mask[i] = pos ? 1 : 0;
+    }
 }
 
+template <bool VEC4>
 __global__ void __launch_bounds__(kThreads) relu_bwd_kernel(const float* __restrict__ dy,
                                                            const int8_t* __restrict__ mask,
                                                            float* __restrict__ dx, long total)
 {
-    const long idx = (long)blockIdx.x * kThreads + threadIdx.x;
+    const long idx = ((long)blockIdx.x * kThreads + threadIdx.x) * (VEC4 ? 4 : 1);
     if (idx >= total) return;
-    dx[idx] = dy[idx] * (float)mask[idx];
+    if (VEC4 && idx + 4 <= total) {
+        const float4 v = *reinterpret_cast<const float4*>(dy + idx);
+        const uint32_t m = *reinterpret_cast<const uint32_t*>(mask + idx);
+        *reinterpret_cast<float4*>(dx + idx) =
+            make_float4(v.x * (float)(int8_t)(m & 0xff), v.y * (float)(int8_t)((m >> 8) & 0xff),
+                        v.z * (float)(int8_t)((m >> 16) & 0xff), v.w * (float)(int8_t)(m >> 24));
+        return;
+    }
+    const long end = VEC4 ? total : idx + 1;
+    for (long i = idx; i < end; ++i) dx[i] = dy[i] * (float)mask[i];
 }
 
 // ---------------------------------------------------------------- bias gradient
@@ -198,67 +224,92 @@ __global__ void __launch_bounds__(kThreads) flip_filter_nhwc_kernel(const float*
 
 // ---------------------------------------------------------------- MaxPool2D NCHW
 // Forward: pydtnn/cython_modules/max_pool_2d_nchw_cython.pyx:86-110 (first maximum wins, index ii*kw+jj).
+// grid.x * 256 threads walk one (n, c) plane of the output, grid.y walks the planes.
 __global__ void __launch_bounds__(kThreads) max_pool_fwd_nchw_kernel(const float* __restrict__ x,
                                                                     float* __restrict__ y,
                                                                     int32_t* __restrict__ idx_max, ConvGeom g)
 {
-    const long idx = (long)blockIdx.x * kThreads + threadIdx.x;
-    const long total = (long)g.n * g.c * g.howo;
-    if (idx >= total) return;
-    const int ox = (int)(idx % g.wo);
-    long t = idx / g.wo;
-    const int oy = (int)(t % g.ho);
-    const long plane = t / g.ho;  // n*c + c
-    const float* src = x + plane * g.h * g.w;
-    float maxval = -3.402823466e+38f;
-    int best = 0;
-    for (int ii = 0; ii < g.kh; ++ii) {
-        const int x_x = g.vstride * oy + g.vdilation * ii - g.vpadding;
-        if ((unsigned)x_x >= (unsigned)g.h) continue;
-        for (int jj = 0; jj < g.kw; ++jj) {
-            const int x_y = g.hstride * ox + g.hdilation * jj - g.hpadding;
-            if ((unsigned)x_y >= (unsigned)g.w) continue;
-            const float val = src[x_x * g.w + x_y];
-            if (val > maxval) { maxval = val; best = ii * g.kw + jj; }
+    const uint32_t pix = blockIdx.x * kThreads + threadIdx.x;
+    if (pix >= (uint32_t)g.howo) return;
+    const int oy = (int)fd_div(pix, g.fd_wo);
+    const int ox = (int)pix - oy * g.wo;
+    const uint32_t planes = (uint32_t)(g.n * g.c);
+    const int y0 = g.vstride * oy - g.vpadding, x0 = g.hstride * ox - g.hpadding;
+    for (uint32_t plane = blockIdx.y; plane < planes; plane += gridDim.y) {
+        const float* src = x + (long)plane * g.h * g.w;
+        float maxval = -3.402823466e+38f;
+        int best = 0;
+        for (int ii = 0; ii < g.kh; ++ii) {
+            const int x_x = y0 + g.vdilation * ii;
+            if ((unsigned)x_x >= (unsigned)g.h) continue;
+            for (int jj = 0; jj < g.kw; ++jj) {
+                const int x_y = x0 + g.hdilation * jj;
+                if ((unsigned)x_y >= (unsigned)g.w) continue;
+                const float val = src[x_x * g.w + x_y];
+                if (val > maxval) { maxval = val; best = ii * g.kw + jj; }
+            }
         }
+        y[(long)plane * g.howo + pix] = maxval;
+        idx_max[(long)plane * g.howo + pix] = best;
     }
-    y[idx] = maxval;
-    idx_max[idx] = best;
 }
 
 // Backward in gather form: one thread per dx element sums dy of every window whose recorded
 // maximum decodes to this element.  The decode is the reference's own
 // (ii = idx / kh, jj = idx % kw, max_pool_2d_nchw_cython.pyx:204-205).  Windows are visited in
 // ascending (oy, ox), the order of the reference's scatter loop.
+// TILED: windows do not overlap and have no padding or dilation (kh == vstride, kw == hstride),
+// so each element lies in at most one window and the tap loops collapse to one lookup.
+template <bool TILED>
 __global__ void __launch_bounds__(kThreads) max_pool_bwd_nchw_kernel(const float* __restrict__ dy,
                                                                     const int32_t* __restrict__ idx_max,
                                                                     float* __restrict__ dx, ConvGeom g)
 {
-    const long idx = (long)blockIdx.x * kThreads + threadIdx.x;
-    const long total = (long)g.n * g.c * g.h * g.w;
-    if (idx >= total) return;
-    const int ww = (int)(idx % g.w);
-    long t = idx / g.w;
-    const int hh = (int)(t % g.h);
-    const long plane = t / g.h;
-    const float* gy = dy + plane * g.howo;
-    const int32_t* gi = idx_max + plane * g.howo;
-    float acc = 0.0f;
-    for (int ii = g.kh - 1; ii >= 0; --ii) {
-        const int ty = hh + g.vpadding - g.vdilation * ii;
-        if (ty < 0) continue;
-        const int oy = ty / g.vstride;
-        if (oy * g.vstride != ty || oy >= g.ho) continue;
-        for (int jj = g.kw - 1; jj >= 0; --jj) {
-            const int tx = ww + g.hpadding - g.hdilation * jj;
-            if (tx < 0) continue;
-            const int ox = tx / g.hstride;
-            if (ox * g.hstride != tx || ox >= g.wo) continue;
-            const int rec = gi[oy * g.wo + ox];
-            if (rec / g.kh == ii && rec % g.kw == jj) acc += gy[oy * g.wo + ox];
+    const uint32_t hw = (uint32_t)(g.h * g.w);
+    const uint32_t pix = blockIdx.x * kThreads + threadIdx.x;
+    if (pix >= hw) return;
+    const int hh = (int)fd_div(pix, g.fd_w);
+    const int ww = (int)pix - hh * g.w;
+    const uint32_t planes = (uint32_t)(g.n * g.c);
+    if (TILED) {
+        const int oy = (int)fd_div((uint32_t)hh, g.fd_vs), ox = (int)fd_div((uint32_t)ww, g.fd_hs);
+        const int ii = hh - oy * g.vstride, jj = ww - ox * g.hstride;
+        const bool inside = oy < g.ho && ox < g.wo;
+        const int win = oy * g.wo + ox;
+        for (uint32_t plane = blockIdx.y; plane < planes; plane += gridDim.y) {
+            float acc = 0.0f;
+            if (inside) {
+                const uint32_t rec = (uint32_t)idx_max[(long)plane * g.howo + win];
+                const uint32_t ri = fd_div(rec, g.fd_kh);
+                const uint32_t rj = rec - fd_div(rec, g.fd_kw) * g.kw;
+                if ((int)ri == ii && (int)rj == jj) acc = 0.0f + dy[(long)plane * g.howo + win];
+            }
+            dx[(long)plane * hw + pix] = acc;
         }
+        return;
     }
-    dx[idx] = acc;
+    for (uint32_t plane = blockIdx.y; plane < planes; plane += gridDim.y) {
+        const float* gy = dy + (long)plane * g.howo;
+        const int32_t* gi = idx_max + (long)plane * g.howo;
+        float acc = 0.0f;
+        for (int ii = g.kh - 1; ii >= 0; --ii) {
+            const int ty = hh + g.vpadding - g.vdilation * ii;
+            if (ty < 0) continue;
+            const int oy = (int)fd_div((uint32_t)ty, g.fd_vs);
+            if (oy * g.vstride != ty || oy >= g.ho) continue;
+            for (int jj = g.kw - 1; jj >= 0; --jj) {
+                const int tx = ww + g.hpadding - g.hdilation * jj;
+                if (tx < 0) continue;
+                const int ox = (int)fd_div((uint32_t)tx, g.fd_hs);
+                if (ox * g.hstride != tx || ox >= g.wo) continue;
+                const uint32_t rec = (uint32_t)gi[oy * g.wo + ox];
+                const uint32_t ri = fd_div(rec, g.fd_kh);
+                const uint32_t rj = rec - fd_div(rec, g.fd_kw) * g.kw;
+                if ((int)ri == ii && (int)rj == jj) acc += gy[oy * g.wo + ox];
+            }
+        }
+        dx[(long)plane * hw + pix] = acc;
+    }
 }
 
 // ---------------------------------------------------------------- SGD with momentum
@@ -302,7 +353,14 @@ int launch_chan_eltwise(const float* x, const float* residual, float* y, long to
 int launch_relu_fwd(const float* x, float* y, int8_t* mask, long total, hipStream_t stream)
 {
     if (total <= 0) return PYDTNN_HIP_ERR_INVALID;
-    hipLaunchKernelGGL(relu_fwd_kernel, dim3(blocks_for(total)), dim3(kThreads), 0, stream, x, y, mask, total);
+    const bool vec = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0 &&
+                     (reinterpret_cast<uintptr_t>(mask) & 3) == 0;
+    if (vec)
+        hipLaunchKernelGGL(relu_fwd_kernel<true>, dim3(blocks_for((total + 3) / 4)), dim3(kThreads), 0, stream, x, y,
+                           mask, total);
+    else
+        hipLaunchKernelGGL(relu_fwd_kernel<false>, dim3(blocks_for(total)), dim3(kThreads), 0, stream, x, y, mask,
+                           total);
     HIP_RETURN_IF_LAUNCH_FAILED();
     return PYDTNN_HIP_OK;
 }
@@ -310,7 +368,14 @@ int launch_relu_fwd(const float* x, float* y, int8_t* mask, long total, hipStrea
 int launch_relu_bwd(const float* dy, const int8_t* mask, float* dx, long total, hipStream_t stream)
 {
     if (total <= 0) return PYDTNN_HIP_ERR_INVALID;
-    hipLaunchKernelGGL(relu_bwd_kernel, dim3(blocks_for(total)), dim3(kThreads), 0, stream, dy, mask, dx, total);
+    const bool vec = ((reinterpret_cast<uintptr_t>(dy) | reinterpret_cast<uintptr_t>(dx)) & 15) == 0 &&
+                     (reinterpret_cast<uintptr_t>(mask) & 3) == 0;
+    if (vec)
+        hipLaunchKernelGGL(relu_bwd_kernel<true>, dim3(blocks_for((total + 3) / 4)), dim3(kThreads), 0, stream, dy,
+                           mask, dx, total);
+    else
+        hipLaunchKernelGGL(relu_bwd_kernel<false>, dim3(blocks_for(total)), dim3(kThreads), 0, stream, dy, mask, dx,
+                           total);
     HIP_RETURN_IF_LAUNCH_FAILED();
     return PYDTNN_HIP_OK;
 }
@@ -375,8 +440,9 @@ int launch_flip_filter(const float* w, float* wf, int nhwc, int kn, int c, int k
 
 int launch_max_pool_fwd_nchw(const float* x, float* y, int32_t* idx_max, const ConvGeom& g, hipStream_t stream)
 {
-    const long total = (long)g.n * g.c * g.howo;
-    hipLaunchKernelGGL(max_pool_fwd_nchw_kernel, dim3(blocks_for(total)), dim3(kThreads), 0, stream, x, y, idx_max, g);
+    const long planes = (long)g.n * g.c;
+    dim3 grid(blocks_for(g.howo), (unsigned)(planes < 65535 ? planes : 65535));
+    hipLaunchKernelGGL(max_pool_fwd_nchw_kernel, grid, dim3(kThreads), 0, stream, x, y, idx_max, g);
     HIP_RETURN_IF_LAUNCH_FAILED();
     return PYDTNN_HIP_OK;
 }
@@ -384,9 +450,14 @@ int launch_max_pool_fwd_nchw(const float* x, float* y, int32_t* idx_max, const C
 int launch_max_pool_bwd_nchw(const float* dy, const int32_t* idx_max, float* dx, const ConvGeom& g,
                              hipStream_t stream)
 {
-    const long total = (long)g.n * g.c * g.h * g.w;
-    hipLaunchKernelGGL(max_pool_bwd_nchw_kernel, dim3(blocks_for(total)), dim3(kThreads), 0, stream, dy, idx_max, dx,
-                       g);
+    const long planes = (long)g.n * g.c;
+    dim3 grid(blocks_for((long)g.h * g.w), (unsigned)(planes < 65535 ? planes : 65535));
+    const bool tiled = g.kh == g.vstride && g.kw == g.hstride && g.vpadding == 0 && g.hpadding == 0 &&
+                       g.vdilation == 1 && g.hdilation == 1;
+    if (tiled)
+        hipLaunchKernelGGL(max_pool_bwd_nchw_kernel<true>, grid, dim3(kThreads), 0, stream, dy, idx_max, dx, g);
+    else
+        hipLaunchKernelGGL(max_pool_bwd_nchw_kernel<false>, grid, dim3(kThreads), 0, stream, dy, idx_max, dx, g);
     HIP_RETURN_IF_LAUNCH_FAILED();
     return PYDTNN_HIP_OK;
 }

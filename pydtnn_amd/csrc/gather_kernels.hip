@@ -20,40 +20,41 @@ namespace {
 constexpr int kThreads = 256;
 
 // ---------------------------------------------------------------- im2col NCHW
-// grid.y = matrix row (c,i,j); grid.x * 256 threads * 4 columns walk the row.
+// grid.y = matrix row (c,i,j); grid.x * 256 threads * 4 columns walk the row.  All index
+// arithmetic is 32-bit (tensors hold fewer than 2^29 floats) and the two per-thread divisions are
+// multiply-high: these kernels are bound by the vector ALU long before HBM if they divide.
 template <bool VEC4>
 __global__ void __launch_bounds__(kThreads) im2col_nchw_kernel(const float* __restrict__ x,
-                                                              float* __restrict__ cols, ConvGeom g)
+                                                              float* __restrict__ cols, ConvGeom g, int p_exact)
 {
-    const int row = blockIdx.y;
-    const int cc = row / g.khw;
-    const int rem = row - cc * g.khw;
-    const int ii = rem / g.kw;
-    const int jj = rem - ii * g.kw;
-    const int di = g.vdilation * ii - g.vpadding;
-    const int dj = g.hdilation * jj - g.hpadding;
+    const uint32_t row = blockIdx.y;
+    const uint32_t cc = fd_div(row, g.fd_khw);
+    const uint32_t rem = row - cc * g.khw;
+    const uint32_t ii = fd_div(rem, g.fd_kw);
+    const uint32_t jj = rem - ii * g.kw;
+    const int di = g.vdilation * (int)ii - g.vpadding;
+    const int dj = g.hdilation * (int)jj - g.hpadding;
 
-    const long col0 = ((long)blockIdx.x * kThreads + threadIdx.x) * 4;
-    if (col0 >= g.p) return;
-    int nn = (int)(col0 / g.howo);
-    int pp = (int)(col0 - (long)nn * g.howo);
-    int yy = pp / g.wo;
-    int xx = pp - yy * g.wo;
+    const uint32_t p = (uint32_t)g.p;
+    const uint32_t col0 = (blockIdx.x * kThreads + threadIdx.x) * 4;
+    if (col0 >= p) return;
+    uint32_t nn = fd_div_checked(col0, g.fd_howo, p_exact);
+    const uint32_t pp = col0 - nn * g.howo;
+    uint32_t yy = fd_div(pp, g.fd_wo);
+    uint32_t xx = pp - yy * g.wo;
 
     float v[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         float val = 0.0f;
-        if (col0 + e < g.p) {
-            const int x_x = g.vstride * yy + di;
-            const int x_y = g.hstride * xx + dj;
-            if ((unsigned)x_x < (unsigned)g.h && (unsigned)x_y < (unsigned)g.w)
-                val = x[(((long)nn * g.c + cc) * g.h + x_x) * g.w + x_y];
-        }
+        const int x_x = g.vstride * (int)yy + di;
+        const int x_y = g.hstride * (int)xx + dj;
+        if (col0 + e < p && (unsigned)x_x < (unsigned)g.h && (unsigned)x_y < (unsigned)g.w)
+            val = x[((nn * g.c + cc) * g.h + x_x) * g.w + x_y];
         v[e] = val;
-        if (++xx == g.wo) {
+        if (++xx == (uint32_t)g.wo) {
             xx = 0;
-            if (++yy == g.ho) { yy = 0; ++nn; }
+            if (++yy == (uint32_t)g.ho) { yy = 0; ++nn; }
         }
     }
     float* dst = cols + (long)row * g.p + col0;
@@ -62,106 +63,124 @@ __global__ void __launch_bounds__(kThreads) im2col_nchw_kernel(const float* __re
     } else {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-            if (col0 + e < g.p) dst[e] = v[e];
+            if (col0 + e < p) dst[e] = v[e];
     }
+}
+
+// Output coordinate reached from input coordinate t = in + pad - dil*tap: t / stride when that is
+// exact and inside [0, limit).  UNIT skips the division for stride 1.
+template <bool UNIT>
+__device__ __forceinline__ bool out_coord(int t, int stride, const FastDiv fd, int limit, int* out)
+{
+    if (t < 0) return false;
+    int o = t;
+    if (!UNIT) {
+        o = (int)fd_div((uint32_t)t, fd);
+        if (o * stride != t) return false;
+    }
+    *out = o;
+    return o < limit;
 }
 
 // ---------------------------------------------------------------- col2im NCHW (gather form)
-// One thread per dx element; lanes along w.
+// grid.x * 256 threads walk one (n, c) plane of dx, grid.y walks the planes; lanes along w.
+template <bool UNIT>
 __global__ void __launch_bounds__(kThreads) col2im_nchw_kernel(const float* __restrict__ cols,
                                                               float* __restrict__ dx, ConvGeom g)
 {
-    const long idx = (long)blockIdx.x * kThreads + threadIdx.x;
-    const long total = (long)g.n * g.c * g.h * g.w;
-    if (idx >= total) return;
-    const int ww = (int)(idx % g.w);
-    long t = idx / g.w;
-    const int hh = (int)(t % g.h);
-    t /= g.h;
-    const int cc = (int)(t % g.c);
-    const int nn = (int)(t / g.c);
-
-    float acc = 0.0f;
-    for (int ii = 0; ii < g.kh; ++ii) {
-        const int ty = hh + g.vpadding - g.vdilation * ii;
-        if (ty < 0) continue;
-        const int oy = ty / g.vstride;
-        if (oy * g.vstride != ty || oy >= g.ho) continue;
-        for (int jj = 0; jj < g.kw; ++jj) {
-            const int tx = ww + g.hpadding - g.hdilation * jj;
-            if (tx < 0) continue;
-            const int ox = tx / g.hstride;
-            if (ox * g.hstride != tx || ox >= g.wo) continue;
-            const long row = (long)cc * g.khw + ii * g.kw + jj;
-            const long col = (long)nn * g.howo + oy * g.wo + ox;
-            acc += cols[row * g.p + col];
+    const uint32_t hw = (uint32_t)(g.h * g.w);
+    const uint32_t pix = blockIdx.x * kThreads + threadIdx.x;
+    if (pix >= hw) return;
+    const int hh = (int)fd_div(pix, g.fd_w);
+    const int ww = (int)pix - hh * g.w;
+    const uint32_t planes = (uint32_t)(g.n * g.c);
+    for (uint32_t plane = blockIdx.y; plane < planes; plane += gridDim.y) {
+        const uint32_t nn = plane / (uint32_t)g.c;
+        const uint32_t cc = plane - nn * g.c;
+        const float* src = cols + (long)cc * g.khw * g.p + (long)nn * g.howo;
+        float acc = 0.0f;
+        for (int ii = 0; ii < g.kh; ++ii) {
+            int oy;
+            if (!out_coord<UNIT>(hh + g.vpadding - g.vdilation * ii, g.vstride, g.fd_vs, g.ho, &oy)) continue;
+            for (int jj = 0; jj < g.kw; ++jj) {
+                int ox;
+                if (!out_coord<UNIT>(ww + g.hpadding - g.hdilation * jj, g.hstride, g.fd_hs, g.wo, &ox)) continue;
+                acc += src[(long)(ii * g.kw + jj) * g.p + oy * g.wo + ox];
+            }
         }
+        dx[(long)plane * hw + pix] = acc;
     }
-    dx[idx] = acc;
 }
 
 // ---------------------------------------------------------------- im2row NHWC
-// One thread per matrix element; lanes along the K axis (c,i,j) of one pixel row.
+// One block owns `rpb` consecutive pixel rows of the matrix (a contiguous run of rpb*k floats) and
+// its threads walk that run, so stores are fully coalesced; the block's first pixel is decomposed
+// once with scalar arithmetic and each element only needs multiply-high divisions.
 __global__ void __launch_bounds__(kThreads) im2row_nhwc_kernel(const float* __restrict__ x,
-                                                              float* __restrict__ rows, ConvGeom g)
+                                                              float* __restrict__ rows, ConvGeom g, int rpb,
+                                                              FastDiv fd_k)
 {
-    const long idx = (long)blockIdx.x * kThreads + threadIdx.x;
-    const long total = g.p * g.k;
-    if (idx >= total) return;
-    const int col = (int)(idx % g.k);
-    const long row = idx / g.k;
-    const int cc = col / g.khw;
-    const int rem = col - cc * g.khw;
-    const int ii = rem / g.kw;
-    const int jj = rem - ii * g.kw;
-    const int nn = (int)(row / g.howo);
-    const int pp = (int)(row - (long)nn * g.howo);
-    const int yy = pp / g.wo;
-    const int xx = pp - yy * g.wo;
-    const int x_x = g.vstride * yy + g.vdilation * ii - g.vpadding;
-    const int x_y = g.hstride * xx + g.hdilation * jj - g.hpadding;
-    float val = 0.0f;
-    if ((unsigned)x_x < (unsigned)g.h && (unsigned)x_y < (unsigned)g.w)
-        val = x[(((long)nn * g.h + x_x) * g.w + x_y) * g.c + cc];
-    rows[idx] = val;
+    const uint32_t row0 = blockIdx.x * (uint32_t)rpb;
+    const uint32_t left = (uint32_t)g.p - row0;
+    const uint32_t nrows = left < (uint32_t)rpb ? left : (uint32_t)rpb;
+    const uint32_t n0 = row0 / (uint32_t)g.howo;
+    const uint32_t pp0 = row0 - n0 * g.howo;
+    const uint32_t count = nrows * (uint32_t)g.k;
+    float* dst = rows + (long)row0 * g.k;
+    for (uint32_t e = threadIdx.x; e < count; e += kThreads) {
+        const uint32_t r = rpb > 1 ? fd_div(e, fd_k) : 0u;
+        const uint32_t col = e - r * g.k;
+        uint32_t pp = pp0 + r, nn = n0;
+        if (pp >= (uint32_t)g.howo) { pp -= g.howo; ++nn; }  // rpb <= howo: at most one wrap
+        const uint32_t yy = fd_div(pp, g.fd_wo);
+        const uint32_t xx = pp - yy * g.wo;
+        const uint32_t cc = fd_div(col, g.fd_khw);
+        const uint32_t rem = col - cc * g.khw;
+        const uint32_t ii = fd_div(rem, g.fd_kw);
+        const uint32_t jj = rem - ii * g.kw;
+        const int x_x = g.vstride * (int)yy + g.vdilation * (int)ii - g.vpadding;
+        const int x_y = g.hstride * (int)xx + g.hdilation * (int)jj - g.hpadding;
+        float val = 0.0f;
+        if ((unsigned)x_x < (unsigned)g.h && (unsigned)x_y < (unsigned)g.w)
+            val = x[((nn * g.h + x_x) * g.w + x_y) * g.c + cc];
+        dst[e] = val;
+    }
 }
 
 // ---------------------------------------------------------------- row2im NHWC (gather form)
-// One thread per dx element; lanes along c.
+// grid.x * 256 threads walk one image of dx (h*w*c floats, lanes along c), grid.y walks the images.
+template <bool UNIT>
 __global__ void __launch_bounds__(kThreads) row2im_nhwc_kernel(const float* __restrict__ rows,
-                                                              float* __restrict__ dx, ConvGeom g)
+                                                              float* __restrict__ dx, ConvGeom g, int c_exact)
 {
-    const long idx = (long)blockIdx.x * kThreads + threadIdx.x;
-    const long total = (long)g.n * g.h * g.w * g.c;
-    if (idx >= total) return;
-    const int cc = (int)(idx % g.c);
-    long t = idx / g.c;
-    const int ww = (int)(t % g.w);
-    t /= g.w;
-    const int hh = (int)(t % g.h);
-    const int nn = (int)(t / g.h);
-
-    float acc = 0.0f;
-    // ascending output pixel (oy, ox) == descending tap (ii, jj): the order of the reference's n,y,x-major loop
-    for (int ii = g.kh - 1; ii >= 0; --ii) {
-        const int ty = hh + g.vpadding - g.vdilation * ii;
-        if (ty < 0) continue;
-        const int oy = ty / g.vstride;
-        if (oy * g.vstride != ty || oy >= g.ho) continue;
-        for (int jj = g.kw - 1; jj >= 0; --jj) {
-            const int tx = ww + g.hpadding - g.hdilation * jj;
-            if (tx < 0) continue;
-            const int ox = tx / g.hstride;
-            if (ox * g.hstride != tx || ox >= g.wo) continue;
-            const long row = (long)nn * g.howo + oy * g.wo + ox;
-            const long col = (long)cc * g.khw + ii * g.kw + jj;
-            acc += rows[row * g.k + col];
+    const uint32_t hwc = (uint32_t)(g.h * g.w * g.c);
+    const uint32_t e = blockIdx.x * kThreads + threadIdx.x;
+    if (e >= hwc) return;
+    const uint32_t t = fd_div_checked(e, g.fd_c, c_exact);
+    const uint32_t cc = e - t * g.c;
+    const int hh = (int)fd_div(t, g.fd_w);
+    const int ww = (int)t - hh * g.w;
+    for (uint32_t nn = blockIdx.y; nn < (uint32_t)g.n; nn += gridDim.y) {
+        const float* src = rows + (long)nn * g.howo * g.k + cc * g.khw;
+        float acc = 0.0f;
+        // ascending output pixel (oy, ox) == descending tap (ii, jj): the order of the reference's n,y,x-major loop
+        for (int ii = g.kh - 1; ii >= 0; --ii) {
+            int oy;
+            if (!out_coord<UNIT>(hh + g.vpadding - g.vdilation * ii, g.vstride, g.fd_vs, g.ho, &oy)) continue;
+            for (int jj = g.kw - 1; jj >= 0; --jj) {
+                int ox;
+                if (!out_coord<UNIT>(ww + g.hpadding - g.hdilation * jj, g.hstride, g.fd_hs, g.wo, &ox)) continue;
+                acc += src[(long)(oy * g.wo + ox) * g.k + ii * g.kw + jj];
+            }
         }
+        dx[(long)nn * hwc + e] = acc;
     }
-    dx[idx] = acc;
 }
 
 inline unsigned blocks_for(long total) { return (unsigned)((total + kThreads - 1) / kThreads); }
+inline unsigned grid_y_for(long count) { return (unsigned)(count < 65535 ? count : 65535); }
+// fd_div(n, d) is exact for every n below `bound` when bound * d < 2^32.
+inline int fd_exact(unsigned long bound, unsigned long d) { return bound * d < (1ul << 32); }
 
 }  // namespace
 
@@ -205,6 +224,13 @@ int make_conv_geom(ConvGeom* g, int n, int c, int h, int w, int kn, int kh, int 
     g->fd_wo = make_fastdiv((uint32_t)g->wo);
     g->fd_c = make_fastdiv((uint32_t)c);
     g->fd_howo = make_fastdiv((uint32_t)g->howo);
+    // Streaming kernels: pixel index of one input plane by w; pool index by kh; coordinates by the strides.
+    if ((unsigned long)((long)h * w + 1024) * w >= two32 || vstride >= 65536 || hstride >= 65536)
+        return PYDTNN_HIP_ERR_UNSUPPORTED;
+    g->fd_w = make_fastdiv((uint32_t)w);
+    g->fd_kh = make_fastdiv((uint32_t)kh);
+    g->fd_vs = make_fastdiv((uint32_t)vstride);
+    g->fd_hs = make_fastdiv((uint32_t)hstride);
     return PYDTNN_HIP_OK;
 }
 
@@ -213,35 +239,49 @@ int launch_im2col_nchw(const float* x, float* cols, const ConvGeom& g, hipStream
     if (g.k > 65535) return PYDTNN_HIP_ERR_UNSUPPORTED;
     dim3 grid((unsigned)((g.p + (long)kThreads * 4 - 1) / ((long)kThreads * 4)), (unsigned)g.k);
     const bool vec = (g.p % 4 == 0) && ((reinterpret_cast<uintptr_t>(cols) & 15) == 0);
+    const int p_exact = fd_exact((unsigned long)g.p + 4 * kThreads, (unsigned long)g.howo);
     if (vec)
-        hipLaunchKernelGGL(im2col_nchw_kernel<true>, grid, dim3(kThreads), 0, stream, x, cols, g);
+        hipLaunchKernelGGL(im2col_nchw_kernel<true>, grid, dim3(kThreads), 0, stream, x, cols, g, p_exact);
     else
-        hipLaunchKernelGGL(im2col_nchw_kernel<false>, grid, dim3(kThreads), 0, stream, x, cols, g);
+        hipLaunchKernelGGL(im2col_nchw_kernel<false>, grid, dim3(kThreads), 0, stream, x, cols, g, p_exact);
     HIP_RETURN_IF_LAUNCH_FAILED();
     return PYDTNN_HIP_OK;
 }
 
 int launch_col2im_nchw(const float* cols, float* dx, const ConvGeom& g, hipStream_t stream)
 {
-    const long total = (long)g.n * g.c * g.h * g.w;
-    hipLaunchKernelGGL(col2im_nchw_kernel, dim3(blocks_for(total)), dim3(kThreads), 0, stream, cols, dx, g);
+    dim3 grid(blocks_for((long)g.h * g.w), grid_y_for((long)g.n * g.c));
+    if (g.vstride == 1 && g.hstride == 1)
+        hipLaunchKernelGGL(col2im_nchw_kernel<true>, grid, dim3(kThreads), 0, stream, cols, dx, g);
+    else
+        hipLaunchKernelGGL(col2im_nchw_kernel<false>, grid, dim3(kThreads), 0, stream, cols, dx, g);
     HIP_RETURN_IF_LAUNCH_FAILED();
     return PYDTNN_HIP_OK;
 }
 
 int launch_im2row_nhwc(const float* x, float* rows, const ConvGeom& g, hipStream_t stream)
 {
-    const long total = g.p * g.k;
-    if ((total + kThreads - 1) / kThreads >= (1l << 31)) return PYDTNN_HIP_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL(im2row_nhwc_kernel, dim3(blocks_for(total)), dim3(kThreads), 0, stream, x, rows, g);
+    // About 2048 matrix elements per block, never more rows than one image holds.
+    int rpb = 2048 / g.k;
+    if (rpb > g.howo) rpb = g.howo;
+    if (rpb < 1) rpb = 1;
+    if (rpb > 1 && !fd_exact((unsigned long)rpb * g.k + kThreads, (unsigned long)g.k)) rpb = 1;
+    const long blocks = (g.p + rpb - 1) / rpb;
+    hipLaunchKernelGGL(im2row_nhwc_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, stream, x, rows, g, rpb,
+                       make_fastdiv((uint32_t)g.k));
     HIP_RETURN_IF_LAUNCH_FAILED();
     return PYDTNN_HIP_OK;
 }
 
 int launch_row2im_nhwc(const float* rows, float* dx, const ConvGeom& g, hipStream_t stream)
 {
-    const long total = (long)g.n * g.h * g.w * g.c;
-    hipLaunchKernelGGL(row2im_nhwc_kernel, dim3(blocks_for(total)), dim3(kThreads), 0, stream, rows, dx, g);
+    const long hwc = (long)g.h * g.w * g.c;
+    dim3 grid(blocks_for(hwc), grid_y_for(g.n));
+    const int c_exact = fd_exact((unsigned long)hwc + kThreads, (unsigned long)g.c);
+    if (g.vstride == 1 && g.hstride == 1)
+        hipLaunchKernelGGL(row2im_nhwc_kernel<true>, grid, dim3(kThreads), 0, stream, rows, dx, g, c_exact);
+    else
+        hipLaunchKernelGGL(row2im_nhwc_kernel<false>, grid, dim3(kThreads), 0, stream, rows, dx, g, c_exact);
     HIP_RETURN_IF_LAUNCH_FAILED();
     return PYDTNN_HIP_OK;
 }
