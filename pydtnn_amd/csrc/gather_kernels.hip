@@ -20,12 +20,81 @@ namespace {
 constexpr int kThreads = 256;
 
 // ---------------------------------------------------------------- im2col NCHW
-// grid.y = matrix row (c,i,j); grid.x * 256 threads * 4 columns walk the row.  All index
-// arithmetic is 32-bit (tensors hold fewer than 2^29 floats) and the two per-thread divisions are
-// multiply-high: these kernels are bound by the vector ALU long before HBM if they divide.
+// The matrix is kh*kw times larger than the image, so the kernel is a store stream and anything
+// it re-reads from L2 competes with that stream for the same fabric.  A block therefore stages
+// the input rows its pixels need in LDS once (coalesced loads of one contiguous piece of an
+// (n, c) plane) and produces all kh*kw matrix rows of its channel from there.
+//   grid.x = image * chunks + chunk (a chunk is `chunk_px` consecutive output pixels of one image)
+//   grid.y = input channel;  256 threads * 4 consecutive pixels each.
+// Index arithmetic is 32-bit (tensors hold fewer than 2^29 floats) with multiply-high divisions.
 template <bool VEC4>
-__global__ void __launch_bounds__(kThreads) im2col_nchw_kernel(const float* __restrict__ x,
-                                                              float* __restrict__ cols, ConvGeom g, int p_exact)
+__global__ void __launch_bounds__(kThreads) im2col_nchw_lds_kernel(const float* __restrict__ x,
+                                                                  float* __restrict__ cols, ConvGeom g,
+                                                                  int chunks, int chunk_px)
+{
+    extern __shared__ float win[];
+    const uint32_t cc = blockIdx.y;
+    const uint32_t nn = blockIdx.x / (uint32_t)chunks;
+    const uint32_t chunk = blockIdx.x - nn * chunks;
+    const uint32_t pp_begin = chunk * (uint32_t)chunk_px;
+    const uint32_t pp_stop = pp_begin + chunk_px;
+    const uint32_t pp_end = pp_stop < (uint32_t)g.howo ? pp_stop : (uint32_t)g.howo;
+    if (pp_begin >= pp_end) return;  // uniform
+
+    // Input rows touched by output rows y0..y1, clipped to the image.
+    const int y0 = (int)(pp_begin / (uint32_t)g.wo), y1 = (int)((pp_end - 1) / (uint32_t)g.wo);
+    int r0 = g.vstride * y0 - g.vpadding;
+    int r1 = g.vstride * y1 + g.vdilation * (g.kh - 1) - g.vpadding;
+    r0 = r0 < 0 ? 0 : r0;
+    r1 = r1 > g.h - 1 ? g.h - 1 : r1;
+    const float* plane = x + (size_t)(nn * g.c + cc) * g.h * g.w;
+    const int start = r0 * g.w, end = (r1 + 1) * g.w;
+    for (int i = start + (int)threadIdx.x; i < end; i += kThreads) win[i - start] = plane[i];
+    __syncthreads();
+
+    const uint32_t pp = pp_begin + threadIdx.x * 4;
+    if (pp >= pp_end) return;
+    uint32_t yy = fd_div(pp, g.fd_wo);
+    uint32_t xx = pp - yy * g.wo;
+    int iy0[4], ix0[4];
+    bool live[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        iy0[e] = g.vstride * (int)yy - g.vpadding;
+        ix0[e] = g.hstride * (int)xx - g.hpadding;
+        live[e] = pp + e < pp_end;
+        if (++xx == (uint32_t)g.wo) { xx = 0; ++yy; }
+    }
+    float* dst = cols + (size_t)cc * g.khw * g.p + (size_t)nn * g.howo + pp;
+    for (int ii = 0; ii < g.kh; ++ii) {
+        for (int jj = 0; jj < g.kw; ++jj) {
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int x_x = iy0[e] + g.vdilation * ii;
+                const int x_y = ix0[e] + g.hdilation * jj;
+                const bool ok = live[e] && (unsigned)x_x < (unsigned)g.h && (unsigned)x_y < (unsigned)g.w;
+                const float val = win[ok ? (x_x - r0) * g.w + x_y : 0];
+                v[e] = ok ? val : 0.0f;
+            }
+            if (VEC4) {
+                *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (live[e]) dst[e] = v[e];
+            }
+            dst += g.p;
+        }
+    }
+}
+
+// Fallback without staging, for windows that do not fit in LDS (large strides or filters on wide
+// images): grid.y = matrix row (c,i,j); grid.x * 256 threads * 4 columns walk the row.
+template <bool VEC4>
+__global__ void __launch_bounds__(kThreads) im2col_nchw_direct_kernel(const float* __restrict__ x,
+                                                                     float* __restrict__ cols, ConvGeom g,
+                                                                     int p_exact)
 {
     const uint32_t row = blockIdx.y;
     const uint32_t cc = fd_div(row, g.fd_khw);
@@ -46,12 +115,11 @@ __global__ void __launch_bounds__(kThreads) im2col_nchw_kernel(const float* __re
     float v[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-        float val = 0.0f;
         const int x_x = g.vstride * (int)yy + di;
         const int x_y = g.hstride * (int)xx + dj;
-        if (col0 + e < p && (unsigned)x_x < (unsigned)g.h && (unsigned)x_y < (unsigned)g.w)
-            val = x[((nn * g.c + cc) * g.h + x_x) * g.w + x_y];
-        v[e] = val;
+        const bool ok = col0 + e < p && (unsigned)x_x < (unsigned)g.h && (unsigned)x_y < (unsigned)g.w;
+        const float val = x[ok ? ((nn * g.c + cc) * g.h + x_x) * g.w + x_y : 0u];
+        v[e] = ok ? val : 0.0f;
         if (++xx == (uint32_t)g.wo) {
             xx = 0;
             if (++yy == (uint32_t)g.ho) { yy = 0; ++nn; }
@@ -72,19 +140,23 @@ __global__ void __launch_bounds__(kThreads) im2col_nchw_kernel(const float* __re
 template <bool UNIT>
 __device__ __forceinline__ bool out_coord(int t, int stride, const FastDiv fd, int limit, int* out)
 {
-    if (t < 0) return false;
     int o = t;
+    bool ok = t >= 0;
     if (!UNIT) {
-        o = (int)fd_div((uint32_t)t, fd);
-        if (o * stride != t) return false;
+        o = (int)fd_div((uint32_t)(ok ? t : 0), fd);
+        ok = ok && o * stride == t;
     }
     *out = o;
-    return o < limit;
+    return ok && o < limit;
 }
 
 // ---------------------------------------------------------------- col2im NCHW (gather form)
 // grid.x * 256 threads walk one (n, c) plane of dx, grid.y walks the planes; lanes along w.
-template <bool UNIT>
+// Every tap is a clamped load followed by a select, so the loads of one element do not wait for
+// each other; adding +0 for a tap outside the matrix leaves the sum unchanged (the accumulator
+// starts at +0 and can therefore never hold -0).  KH, KW > 0 fix the filter at compile time so
+// that the tap loops unroll; 0 keeps them as run-time loops.
+template <bool UNIT, int KH, int KW>
 __global__ void __launch_bounds__(kThreads) col2im_nchw_kernel(const float* __restrict__ cols,
                                                               float* __restrict__ dx, ConvGeom g)
 {
@@ -93,19 +165,24 @@ __global__ void __launch_bounds__(kThreads) col2im_nchw_kernel(const float* __re
     if (pix >= hw) return;
     const int hh = (int)fd_div(pix, g.fd_w);
     const int ww = (int)pix - hh * g.w;
+    const int kh = KH > 0 ? KH : g.kh, kw = KW > 0 ? KW : g.kw;
     const uint32_t planes = (uint32_t)(g.n * g.c);
     for (uint32_t plane = blockIdx.y; plane < planes; plane += gridDim.y) {
         const uint32_t nn = plane / (uint32_t)g.c;
         const uint32_t cc = plane - nn * g.c;
-        const float* src = cols + (long)cc * g.khw * g.p + (long)nn * g.howo;
+        const float* src = cols + (long)cc * (kh * kw) * g.p + (long)nn * g.howo;
         float acc = 0.0f;
-        for (int ii = 0; ii < g.kh; ++ii) {
-            int oy;
-            if (!out_coord<UNIT>(hh + g.vpadding - g.vdilation * ii, g.vstride, g.fd_vs, g.ho, &oy)) continue;
-            for (int jj = 0; jj < g.kw; ++jj) {
-                int ox;
-                if (!out_coord<UNIT>(ww + g.hpadding - g.hdilation * jj, g.hstride, g.fd_hs, g.wo, &ox)) continue;
-                acc += src[(long)(ii * g.kw + jj) * g.p + oy * g.wo + ox];
+#pragma unroll
+        for (int ii = 0; ii < kh; ++ii) {
+            int oy = 0;
+            const bool row_ok = out_coord<UNIT>(hh + g.vpadding - g.vdilation * ii, g.vstride, g.fd_vs, g.ho, &oy);
+#pragma unroll
+            for (int jj = 0; jj < kw; ++jj) {
+                int ox = 0;
+                const bool ok =
+                    out_coord<UNIT>(ww + g.hpadding - g.hdilation * jj, g.hstride, g.fd_hs, g.wo, &ox) && row_ok;
+                const float val = src[(long)(ii * kw + jj) * g.p + (ok ? oy * g.wo + ox : 0)];
+                acc += ok ? val : 0.0f;
             }
         }
         dx[(long)plane * hw + pix] = acc;
@@ -236,14 +313,31 @@ int make_conv_geom(ConvGeom* g, int n, int c, int h, int w, int kn, int kh, int 
 
 int launch_im2col_nchw(const float* x, float* cols, const ConvGeom& g, hipStream_t stream)
 {
+    const bool aligned = (reinterpret_cast<uintptr_t>(cols) & 15) == 0;
+    // Staged form: chunks of at most 1024 pixels, equal within an image and a multiple of 4 long.
+    const int chunks = (g.howo + 1023) / 1024;
+    const int chunk_px = ((g.howo + chunks - 1) / chunks + 3) & ~3;
+    const long rows_out = (chunk_px + g.wo - 2) / g.wo + 1;  // output rows a chunk can straddle
+    const long rows_in = (long)g.vstride * (rows_out - 1) + (long)g.vdilation * (g.kh - 1) + 1;
+    const long lds_bytes = (rows_in < g.h ? rows_in : g.h) * g.w * 4;
+    if (lds_bytes <= 48 * 1024 && g.c <= 65535) {
+        dim3 grid((unsigned)((long)g.n * chunks), (unsigned)g.c);
+        if (aligned && g.howo % 4 == 0)
+            hipLaunchKernelGGL(im2col_nchw_lds_kernel<true>, grid, dim3(kThreads), (size_t)lds_bytes, stream, x, cols,
+                               g, chunks, chunk_px);
+        else
+            hipLaunchKernelGGL(im2col_nchw_lds_kernel<false>, grid, dim3(kThreads), (size_t)lds_bytes, stream, x, cols,
+                               g, chunks, chunk_px);
+        HIP_RETURN_IF_LAUNCH_FAILED();
+        return PYDTNN_HIP_OK;
+    }
     if (g.k > 65535) return PYDTNN_HIP_ERR_UNSUPPORTED;
     dim3 grid((unsigned)((g.p + (long)kThreads * 4 - 1) / ((long)kThreads * 4)), (unsigned)g.k);
-    const bool vec = (g.p % 4 == 0) && ((reinterpret_cast<uintptr_t>(cols) & 15) == 0);
     const int p_exact = fd_exact((unsigned long)g.p + 4 * kThreads, (unsigned long)g.howo);
-    if (vec)
-        hipLaunchKernelGGL(im2col_nchw_kernel<true>, grid, dim3(kThreads), 0, stream, x, cols, g, p_exact);
+    if (aligned && g.p % 4 == 0)
+        hipLaunchKernelGGL(im2col_nchw_direct_kernel<true>, grid, dim3(kThreads), 0, stream, x, cols, g, p_exact);
     else
-        hipLaunchKernelGGL(im2col_nchw_kernel<false>, grid, dim3(kThreads), 0, stream, x, cols, g, p_exact);
+        hipLaunchKernelGGL(im2col_nchw_direct_kernel<false>, grid, dim3(kThreads), 0, stream, x, cols, g, p_exact);
     HIP_RETURN_IF_LAUNCH_FAILED();
     return PYDTNN_HIP_OK;
 }
@@ -251,10 +345,13 @@ int launch_im2col_nchw(const float* x, float* cols, const ConvGeom& g, hipStream
 int launch_col2im_nchw(const float* cols, float* dx, const ConvGeom& g, hipStream_t stream)
 {
     dim3 grid(blocks_for((long)g.h * g.w), grid_y_for((long)g.n * g.c));
-    if (g.vstride == 1 && g.hstride == 1)
-        hipLaunchKernelGGL(col2im_nchw_kernel<true>, grid, dim3(kThreads), 0, stream, cols, dx, g);
+    const bool unit = g.vstride == 1 && g.hstride == 1;
+    if (unit && g.kh == 3 && g.kw == 3)
+        hipLaunchKernelGGL((col2im_nchw_kernel<true, 3, 3>), grid, dim3(kThreads), 0, stream, cols, dx, g);
+    else if (unit)
+        hipLaunchKernelGGL((col2im_nchw_kernel<true, 0, 0>), grid, dim3(kThreads), 0, stream, cols, dx, g);
     else
-        hipLaunchKernelGGL(col2im_nchw_kernel<false>, grid, dim3(kThreads), 0, stream, cols, dx, g);
+        hipLaunchKernelGGL((col2im_nchw_kernel<false, 0, 0>), grid, dim3(kThreads), 0, stream, cols, dx, g);
     HIP_RETURN_IF_LAUNCH_FAILED();
     return PYDTNN_HIP_OK;
 }
