@@ -155,6 +155,17 @@ def run_cfg2(torch, pd, args):
     extra["im2col_pct_hbm_peak"] = round(100 * extra["im2col_gbs"] / HBM_PEAK_GBS, 1)
     extra["col2im_pct_hbm_peak"] = round(100 * extra["col2im_gbs"] / HBM_PEAK_GBS, 1)
     del cols
+    # the NHWC pair on the same layer (x viewed as N,56,56,256; the values do not matter for a stream)
+    xh = xd.view(n, 56, 56, 256)
+    rows_t, r2i_t = Timer(torch), Timer(torch)
+    for i in range(4):
+        rows = ops.im2row_nhwc(xh, *geom) if i == 0 else rows_t(ops.im2row_nhwc, xh, *geom)
+        back = ops.row2im_nhwc(rows, n, 56, 56, 256, *geom) if i == 0 else r2i_t(ops.row2im_nhwc, rows, n, 56, 56,
+                                                                                256, *geom)
+        del back, rows
+    torch.cuda.synchronize()
+    extra["im2row_gbs"] = round(stream_bytes / (rows_t.mean_ms() * 1e-3) / 1e9, 1)
+    extra["row2im_gbs"] = round(stream_bytes / (r2i_t.mean_ms() * 1e-3) / 1e9, 1)
     roofline = {"bound": "mfma", "kernel": "gemm_kernel<128x128, PlainK, Im2colNchwMN, EpiNchw> (forward)",
                 "achieved": round(achieved, 3), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES["cfg2"]}

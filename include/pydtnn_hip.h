@@ -85,6 +85,11 @@ int pydtnn_hip_sgemm(int transa, int transb, long m, long n, long k, const float
  *                  + bias_vector -> ((v - bn_running_mean) * bn_inv_std) * bn_gamma + bn_beta -> ReLU,
  *                  each stage skipped when its pointer is NULL / relu is false.  The BN stage is
  *                  applied when bn_running_mean is non-NULL and then needs all four vectors.
+ *                  The workspace is optional here: with
+ *                  pydtnn_hip_conv_workspace_bytes(PYDTNN_HIP_OP_FWD, ...) bytes the launch is
+ *                  balanced over the compute units (tiles that do not fill the chip evenly are
+ *                  cut along the reduction axis and summed in a fixed order); with less, or
+ *                  NULL, the result is computed by a plain grid of tiles.
  *   trans == 'Y' : filter gradient.  in1 = dy (layout of y), out = dw (layout of weights);
  *                  epilogue arguments must be NULL / false.  Needs a workspace of
  *                  pydtnn_hip_conv_workspace_bytes(PYDTNN_HIP_OP_DW, ...) bytes.

@@ -66,7 +66,7 @@ class ConvGemm:
             "The input matrices must have the same type of data as the one specified when " \
             "this class was instantiated!"
         geom = (b, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
-        ws, ws_bytes = native.conv_workspace(native.OP_DW, 0, geom) if trans else (None, 0)
+        ws, ws_bytes = native.conv_workspace(native.OP_DW if trans else native.OP_FWD, 0, geom)
         check(lib().pydtnn_hip_sconvGemmNCHW(
             b'Y' if trans else b'N', b, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation,
             hdilation, f32(weights), f32(x), f32(biases), f32(biases_vector), f32(bn_running_mean), f32(bn_inv_std),
@@ -97,7 +97,7 @@ class ConvGemm:
         assert ck == c, "Number of channels in weights and x should be the same!"
         assert weights.dtype == x.dtype == biases.dtype, "All the matrices must have the same type of data!"
         geom = (b, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
-        ws, ws_bytes = native.conv_workspace(native.OP_DW, 1, geom) if trans else (None, 0)
+        ws, ws_bytes = native.conv_workspace(native.OP_DW if trans else native.OP_FWD, 1, geom)
         check(lib().pydtnn_hip_sconvGemmNHWC(
             b'Y' if trans else b'N', b, h, w, c, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation,
             hdilation, f32(weights), f32(x), f32(biases), f32(biases_vector), f32(bn_running_mean), f32(bn_inv_std),

@@ -165,9 +165,14 @@ inline EpiNchw epi_nchw(float* out, int channels, int howo, long p, const ChanEp
 inline bool taps_supported(const ConvGeom& g) { return g.kh <= 31 && g.kw <= 31; }
 inline bool taps_wide(const ConvGeom& g) { return g.khw > 31; }
 
+// Workspace of the balanced launch (gemm::launch_balanced): two accumulator tiles per resident
+// workgroup, sized for the most this part can hold (4 per CU on 256 CUs) so that the query needs no device.
+constexpr int kMaxResident = 1024;
+constexpr size_t kBalanceBytes = (size_t)2 * kMaxResident * 128 * 128 * 4;
+
 template <bool WIDE>
-int conv_fwd_nchw_t(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan,
-                    hipStream_t stream)
+int conv_fwd_nchw_t(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan, float* ws,
+                    size_t ws_bytes, hipStream_t stream)
 {
     const TileSel sel = pick_tile(g.kn, g.p);
     int rc = PYDTNN_HIP_OK;
@@ -176,22 +181,23 @@ int conv_fwd_nchw_t(const ConvGeom& g, const float* w, const float* x, float* y,
         auto al = plain_k<T::BM, false>(w, (long)g.kn * g.k, g.k, 0, g.kn, 0);
         Im2colNchwMN<T::BN, WIDE> bl;
         bl.x = x; bl.g = g;
-        rc = launch<T>(al, bl, epi_nchw(y, g.kn, g.howo, g.p, chan), g.kn, g.p, no_split(g.k), 1, stream);
+        rc = launch_balanced<T>(al, bl, epi_nchw(y, g.kn, g.howo, g.p, chan), g.kn, g.p, g.k, ws, ws_bytes, stream);
     })
     return rc;
 }
 
-int conv_fwd_nchw(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan,
-                  hipStream_t stream)
+// `ws` is optional: without it (or with less than kBalanceBytes) the launch is a plain grid of tiles.
+int conv_fwd_nchw(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan, float* ws,
+                  size_t ws_bytes, hipStream_t stream)
 {
     if (!taps_supported(g)) return PYDTNN_HIP_ERR_UNSUPPORTED;
-    return taps_wide(g) ? conv_fwd_nchw_t<true>(g, w, x, y, chan, stream)
-                        : conv_fwd_nchw_t<false>(g, w, x, y, chan, stream);
+    return taps_wide(g) ? conv_fwd_nchw_t<true>(g, w, x, y, chan, ws, ws_bytes, stream)
+                        : conv_fwd_nchw_t<false>(g, w, x, y, chan, ws, ws_bytes, stream);
 }
 
 template <bool WIDE>
-int conv_fwd_nhwc_t(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan,
-                    hipStream_t stream)
+int conv_fwd_nhwc_t(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan, float* ws,
+                    size_t ws_bytes, hipStream_t stream)
 {
     const TileSel sel = pick_tile(g.p, g.kn);
     int rc = PYDTNN_HIP_OK;
@@ -200,17 +206,18 @@ int conv_fwd_nhwc_t(const ConvGeom& g, const float* w, const float* x, float* y,
         al.x = x; al.g = g;
         FilterNhwcMN<T::BN> bl;
         bl.w = w; bl.g = g;
-        rc = launch<T>(al, bl, epi_plain(y, g.kn, 0, g.p, g.kn, chan), g.p, g.kn, no_split(g.k), 1, stream);
+        rc = launch_balanced<T>(al, bl, epi_plain(y, g.kn, 0, g.p, g.kn, chan), g.p, g.kn, g.k, ws, ws_bytes,
+                                stream);
     })
     return rc;
 }
 
-int conv_fwd_nhwc(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan,
-                  hipStream_t stream)
+int conv_fwd_nhwc(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan, float* ws,
+                  size_t ws_bytes, hipStream_t stream)
 {
     if (!taps_supported(g)) return PYDTNN_HIP_ERR_UNSUPPORTED;
-    return taps_wide(g) ? conv_fwd_nhwc_t<true>(g, w, x, y, chan, stream)
-                        : conv_fwd_nhwc_t<false>(g, w, x, y, chan, stream);
+    return taps_wide(g) ? conv_fwd_nhwc_t<true>(g, w, x, y, chan, ws, ws_bytes, stream)
+                        : conv_fwd_nhwc_t<false>(g, w, x, y, chan, ws, ws_bytes, stream);
 }
 
 // ---------------------------------------------------------------- filter gradient
@@ -335,8 +342,12 @@ int conv_dx(const ConvGeom& g, int nhwc, const float* w, const float* dy, float*
                         g.hdilation * (g.kw - 1) - g.hpadding, 1, 1, g.vdilation, g.hdilation);
     if (rc != PYDTNN_HIP_OK) return rc;
     if (gb.ho != g.h || gb.wo != g.w) return PYDTNN_HIP_ERR_INVALID;
-    return nhwc ? conv_fwd_nhwc(gb, ws, dy, dx, no_epilogue(), stream)
-                : conv_fwd_nchw(gb, ws, dy, dx, no_epilogue(), stream);
+    // what is left of the workspace after the flipped filter balances the launch
+    const size_t used = (need + 255) & ~(size_t)255;
+    float* rest = ws_bytes > used ? ws + used / 4 : nullptr;
+    const size_t rest_bytes = ws_bytes > used ? ws_bytes - used : 0;
+    return nhwc ? conv_fwd_nhwc(gb, ws, dy, dx, no_epilogue(), rest, rest_bytes, stream)
+                : conv_fwd_nchw(gb, ws, dy, dx, no_epilogue(), rest, rest_bytes, stream);
 }
 
 int geom_from_args(ConvGeom* g, long b, long c, long h, long w, long kn, long kh, long kw, long vpadding,
@@ -358,7 +369,8 @@ int sconv_gemm(int nhwc, char trans, const ConvGeom& g, const float* in1, const 
     if (trans == 'N') {
         if (!bn_args_consistent(mean, inv_std, gamma, beta)) return PYDTNN_HIP_ERR_INVALID;
         const ChanEpilogue chan = make_chan(bias, mean, inv_std, gamma, beta, relu ? 1 : 0);
-        return nhwc ? conv_fwd_nhwc(g, in1, x, out, chan, stream) : conv_fwd_nchw(g, in1, x, out, chan, stream);
+        return nhwc ? conv_fwd_nhwc(g, in1, x, out, chan, (float*)ws, ws_bytes, stream)
+                    : conv_fwd_nchw(g, in1, x, out, chan, (float*)ws, ws_bytes, stream);
     }
     if (trans == 'Y') {
         if (bias || mean || inv_std || gamma || beta || relu) return PYDTNN_HIP_ERR_INVALID;
@@ -494,8 +506,10 @@ size_t pydtnn_hip_conv_workspace_bytes(int op, int nhwc, int b, int c, int h, in
     if (geom_from_args(&g, GEOM_ARGS) != PYDTNN_HIP_OK) return 0;
     switch (op) {
         case PYDTNN_HIP_OP_DW: return (size_t)plan_dw(g, nhwc).splits * g.kn * g.k * 4;
+        case PYDTNN_HIP_OP_FWD: return kBalanceBytes;  // optional: a smaller or absent workspace only costs speed
         case PYDTNN_HIP_OP_DX:
-            return dx_as_forward(g) ? (size_t)g.kn * g.k * 4 : (size_t)g.k * g.p * 4;
+            return dx_as_forward(g) ? (((size_t)g.kn * g.k * 4 + 255) & ~(size_t)255) + kBalanceBytes
+                                    : (size_t)g.k * g.p * 4;
         case PYDTNN_HIP_OP_DX_I2C: return (size_t)g.k * g.p * 4;
         case PYDTNN_HIP_OP_DB: return bias_grad_workspace_floats(g.n, g.kn) * 4;
         default: return 0;

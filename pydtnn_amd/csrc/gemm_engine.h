@@ -706,6 +706,96 @@ __device__ __forceinline__ void step(const AL& al, const BL& bl, const typename 
     mfma_groups<T, BUF, 0, AL, BL>(al, bl, as, bs, ai, bi, ra, rb, a_base, b_base, acc, af, bf, knext, kend);
 }
 
+// The reduction loop of one tile over [kbeg, kend): adds into `acc`.  Leaves LDS free for reuse
+// (every wavefront has passed the barrier that follows the last operand fetch).
+template <class T, class AL, class BL>
+__device__ __forceinline__ void tile_mainloop(const AL& al, const BL& bl, int m0, int n0, int image, int kbeg,
+                                              int kend, float* As0, float* As1, float* Bs0, float* Bs1,
+                                              uint32_t a_base, uint32_t b_base, floatx16 (&acc)[T::TM][T::TN], int tid)
+{
+    typename AL::State as;
+    typename BL::State bs;
+    al.init(as, m0, image, tid);
+    bl.init(bs, n0, image, tid);
+
+    // Register sets: during step s the loads of tile s+2 go to set (s & 1) while set ((s+1) & 1),
+    // filled during step s-1 with tile s+1, is stored to LDS at the end of the step.
+    float ra0[AL::NLD], rb0[BL::NLD], ra1[AL::NLD], rb1[BL::NLD];
+    {   // tiles 0 and 1 (any kend, including an empty range: everything reads as zero)
+        typename AL::Iter ai;
+        typename BL::Iter bi;
+        al.begin(as, ai, kbeg, kend);
+        bl.begin(bs, bi, kbeg, kend);
+        load_all<0, AL>(al, as, ai, ra0, kbeg, kend);
+        load_all<0, BL>(bl, bs, bi, rb0, kbeg, kend);
+        al.begin(as, ai, kbeg + BK, kend);
+        bl.begin(bs, bi, kbeg + BK, kend);
+        load_all<0, AL>(al, as, ai, ra1, kbeg + BK, kend);
+        load_all<0, BL>(bl, bs, bi, rb1, kbeg + BK, kend);
+    }
+    al.store(As0, ra0, tid);
+    bl.store(Bs0, rb0, tid);
+    __syncthreads();
+
+    // Two steps per trip so that the register sets are named statically.  A reduction range with an
+    // odd number of steps runs one extra step on a tile that lies beyond kend and therefore is zero.
+    for (int k0 = kbeg; k0 < kend; k0 += 2 * BK) {
+        step<T, 0>(al, bl, as, bs, ra0, rb0, a_base, b_base, acc, k0 + 2 * BK, kend);
+        al.store(As1, ra1, tid);
+        bl.store(Bs1, rb1, tid);
+        __syncthreads();
+        step<T, 1>(al, bl, as, bs, ra1, rb1, a_base, b_base, acc, k0 + 3 * BK, kend);
+        al.store(As0, ra0, tid);
+        bl.store(Bs0, rb0, tid);
+        __syncthreads();
+    }
+}
+
+template <class T>
+__device__ __forceinline__ void clear_acc(floatx16 (&acc)[T::TM][T::TN])
+{
+#pragma unroll
+    for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < T::TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+}
+
+// Accumulator layout of v_mfma_f32_32x32x2_f32: register v of lane l holds
+// C[8*(v/4) + 4*(l/32) + v%4][l%32] of the 32x32 block.
+template <class T, class EP>
+__device__ __forceinline__ void store_tile(const EP& ep, const floatx16 (&acc)[T::TM][T::TN], int m0, int n0,
+                                           int split, int tid)
+{
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm0 = (wave % T::WGM) * T::WM, wn0 = (wave / T::WGM) * T::WN;
+    const int frag_r = lane & 31, frag_k = lane >> 5;
+#pragma unroll
+    for (int j = 0; j < T::TN; ++j) {
+        const typename EP::Col col = ep.column(n0 + wn0 + j * 32 + frag_r, split);
+#pragma unroll
+        for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int m = m0 + wm0 + i * 32 + 8 * (v / 4) + 4 * frag_k + (v % 4);
+                ep.store(col, m, acc[i][j][v]);
+            }
+    }
+}
+
+// LDS byte addresses of this lane's MFMA operand elements of buffer 0 at k-step 0, block (0, 0).
+template <class T>
+__device__ __forceinline__ void operand_bases(const float* As0, const float* Bs0, int tid, uint32_t* a_base,
+                                              uint32_t* b_base)
+{
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm0 = (wave % T::WGM) * T::WM, wn0 = (wave / T::WGM) * T::WN;
+    const int frag_r = lane & 31, frag_k = lane >> 5;
+    *a_base = lds_addr(&As0[frag_k * (T::BM + kPad) + wm0 + frag_r]);
+    *b_base = lds_addr(&Bs0[frag_k * (T::BN + kPad) + wn0 + frag_r]);
+}
+
 template <class T, class AL, class BL, class EP>
 __global__ void __launch_bounds__(kThreads) gemm_kernel(AL al, BL bl, EP ep, int tiles_m, SplitInfo si)
 {
@@ -724,70 +814,12 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(AL al, BL bl, EP ep, int
     const int kbeg = chunk_idx * si.chunk;
     const int kend = min(k_total, kbeg + si.chunk);
 
-    typename AL::State as;
-    typename BL::State bs;
-    al.init(as, m0, image, tid);
-    bl.init(bs, n0, image, tid);
-
-    // Register sets: during step s the loads of tile s+2 go to set (s & 1) while set ((s+1) & 1),
-    // filled during step s-1 with tile s+1, is stored to LDS at the end of the step.
-    float ra0[AL::NLD], rb0[BL::NLD], ra1[AL::NLD], rb1[BL::NLD];
+    uint32_t a_base, b_base;
+    operand_bases<T>(As[0], Bs[0], tid, &a_base, &b_base);
     floatx16 acc[T::TM][T::TN];
-#pragma unroll
-    for (int i = 0; i < T::TM; ++i)
-#pragma unroll
-        for (int j = 0; j < T::TN; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-
-    const int wave = tid >> 6, lane = tid & 63;
-    const int wm0 = (wave % T::WGM) * T::WM, wn0 = (wave / T::WGM) * T::WN;
-    const int frag_r = lane & 31, frag_k = lane >> 5;
-    const uint32_t a_base = lds_addr(&As[0][frag_k * (T::BM + kPad) + wm0 + frag_r]);
-    const uint32_t b_base = lds_addr(&Bs[0][frag_k * (T::BN + kPad) + wn0 + frag_r]);
-
-    {   // tiles 0 and 1 (any kend, including an empty range: everything reads as zero)
-        typename AL::Iter ai;
-        typename BL::Iter bi;
-        al.begin(as, ai, kbeg, kend);
-        bl.begin(bs, bi, kbeg, kend);
-        load_all<0, AL>(al, as, ai, ra0, kbeg, kend);
-        load_all<0, BL>(bl, bs, bi, rb0, kbeg, kend);
-        al.begin(as, ai, kbeg + BK, kend);
-        bl.begin(bs, bi, kbeg + BK, kend);
-        load_all<0, AL>(al, as, ai, ra1, kbeg + BK, kend);
-        load_all<0, BL>(bl, bs, bi, rb1, kbeg + BK, kend);
-    }
-    al.store(As[0], ra0, tid);
-    bl.store(Bs[0], rb0, tid);
-    __syncthreads();
-
-    // Two steps per trip so that the register sets are named statically.  A reduction range with an
-    // odd number of steps runs one extra step on a tile that lies beyond kend and therefore is zero.
-    for (int k0 = kbeg; k0 < kend; k0 += 2 * BK) {
-        step<T, 0>(al, bl, as, bs, ra0, rb0, a_base, b_base, acc, k0 + 2 * BK, kend);
-        al.store(As[1], ra1, tid);
-        bl.store(Bs[1], rb1, tid);
-        __syncthreads();
-        step<T, 1>(al, bl, as, bs, ra1, rb1, a_base, b_base, acc, k0 + 3 * BK, kend);
-        al.store(As[0], ra0, tid);
-        bl.store(Bs[0], rb0, tid);
-        __syncthreads();
-    }
-
-    // Accumulator layout of v_mfma_f32_32x32x2_f32: register v of lane l holds
-    // C[8*(v/4) + 4*(l/32) + v%4][l%32] of the 32x32 block.
-#pragma unroll
-    for (int j = 0; j < T::TN; ++j) {
-        const typename EP::Col col = ep.column(n0 + wn0 + j * 32 + frag_r, split);
-#pragma unroll
-        for (int i = 0; i < T::TM; ++i)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int m = m0 + wm0 + i * 32 + 8 * (v / 4) + 4 * frag_k + (v % 4);
-                ep.store(col, m, acc[i][j][v]);
-            }
-    }
+    clear_acc<T>(acc);
+    tile_mainloop<T>(al, bl, m0, n0, image, kbeg, kend, As[0], As[1], Bs[0], Bs[1], a_base, b_base, acc, tid);
+    store_tile<T>(ep, acc, m0, n0, split, tid);
 }
 
 template <class T, class AL, class BL, class EP>
@@ -799,6 +831,192 @@ inline int launch(const AL& al, const BL& bl, const EP& ep, long m, long n, cons
     dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)splits);
     hipLaunchKernelGGL((gemm_kernel<T, AL, BL, EP>), grid, dim3(kThreads), 0, stream, al, bl, ep, (int)tiles_m, si);
     HIP_RETURN_IF_LAUNCH_FAILED();
+    return PYDTNN_HIP_OK;
+}
+
+// ---------------------------------------------------------------- balanced ("stream-K") form
+// A grid of whole tiles leaves compute units idle whenever the tile count is not a multiple of
+// what the chip holds at once: 3136 tiles on 256 CUs is 12.25 per CU, so the launch lasts as long
+// as 13.  Here the grid is exactly the number of workgroups the chip holds (`gridDim.x`), and
+//   * the tiles [0, sk_tiles), sk_tiles = tiles mod gridDim.x, are cut along the reduction axis
+//     into units of 2*BK and the units are dealt out evenly: workgroup g takes units
+//     [g*U/G, (g+1)*U/G) of the U = sk_tiles*units in all, crossing tile borders as they come;
+//   * the remaining tiles, a multiple of the grid, go round-robin, whole.
+// A workgroup that holds a tile's whole reduction range stores it through the epilogue; otherwise it
+// stores the raw accumulators to one of its two slots of `partial` (a range touches at most two
+// tiles partially: slot 0 for the piece that starts at the workgroup's first unit, slot 1 for the
+// other), and streamk_fixup_kernel adds a tile's pieces in ascending reduction order and applies
+// the epilogue.  No workgroup waits for another, and the result does not depend on timing.
+struct StreamK {
+    int tiles;      // all tiles of the GEMM
+    int sk_tiles;   // tiles cut into units
+    int sk_blocks;  // workgroups that take part in the unit phase (each gets at least a few units)
+    int units;      // units of 2*BK per tile
+    int k;          // reduction length
+    float* partial; // 2 * gridDim.x slots of BM*BN floats
+};
+
+__host__ __device__ inline long sk_first_unit(int g, long total_units, int sk_blocks)
+{
+    return (long)g * total_units / sk_blocks;
+}
+
+template <class T, class AL, class BL, class EP>
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))) gemm_streamk_kernel(AL al, BL bl, EP ep, int tiles_m, StreamK sk)
+{
+    __shared__ float As[2][BK * (T::BM + kPad)];
+    __shared__ float Bs[2][BK * (T::BN + kPad)];
+
+    const int tid = threadIdx.x;
+    const int g = xcd_remap(blockIdx.x, gridDim.x);
+    uint32_t a_base, b_base;
+    operand_bases<T>(As[0], Bs[0], tid, &a_base, &b_base);
+
+    const long total = (long)sk.sk_tiles * sk.units;
+    long u = 0, u_end = 0;
+    if (g < sk.sk_blocks) {
+        u = sk_first_unit(g, total, sk.sk_blocks);
+        u_end = sk_first_unit(g + 1, total, sk.sk_blocks);
+    }
+    const long u_first = u;
+    // Workgroups that share a compute unit would otherwise run in lockstep (all of them in their
+    // prologue or their epilogue at once, with the matrix cores idle).  They are launched a third of
+    // the grid apart, so each third takes its units after a different number of whole tiles.
+    int whole_before_units = (int)((long)blockIdx.x * 3 / gridDim.x);
+    int whole_tile = sk.sk_tiles + g;
+    for (;;) {
+        int tile, kbeg, kend;
+        bool whole;
+        float* slot = nullptr;
+        const bool units_left = u < u_end, tiles_left = whole_tile < sk.tiles;
+        if (units_left && (whole_before_units <= 0 || !tiles_left)) {
+            tile = (int)(u / sk.units);
+            const int ku0 = (int)(u - (long)tile * sk.units);
+            const long left = u_end - u;
+            const int ku1 = left < sk.units - ku0 ? ku0 + (int)left : sk.units;
+            kbeg = ku0 * 2 * BK;
+            kend = min(sk.k, ku1 * 2 * BK);
+            whole = ku0 == 0 && ku1 == sk.units;
+            // slot 0 for the piece that starts at this workgroup's first unit, slot 1 for a piece that
+            // starts at a tile border
+            slot = sk.partial + (size_t)(2 * g + (u == u_first ? 0 : 1)) * (T::BM * T::BN);
+            u += ku1 - ku0;
+        } else if (tiles_left) {
+            tile = whole_tile;
+            kbeg = 0;
+            kend = sk.k;
+            whole = true;
+            whole_tile += gridDim.x;
+            --whole_before_units;
+        } else {
+            break;
+        }
+        const int tm_idx = tile % tiles_m, tn_idx = tile / tiles_m;
+        const int m0 = tm_idx * T::BM, n0 = tn_idx * T::BN;
+        floatx16 acc[T::TM][T::TN];
+        clear_acc<T>(acc);
+        tile_mainloop<T>(al, bl, m0, n0, 0, kbeg, kend, As[0], As[1], Bs[0], Bs[1], a_base, b_base, acc, tid);
+        if (whole) {
+            store_tile<T>(ep, acc, m0, n0, 0, tid);
+        } else {
+            float* dst = slot + tid;
+#pragma unroll
+            for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+                for (int j = 0; j < T::TN; ++j)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) dst[((i * T::TN + j) * 16 + v) * kThreads] = acc[i][j][v];
+        }
+    }
+}
+
+// grid (sk_tiles, TM*TN*4): a workgroup owns four of the 16*TM*TN accumulator registers of one
+// tile; if the tile was cut, it adds their pieces in ascending reduction order and stores them.
+template <class T, class EP>
+__global__ void __launch_bounds__(kThreads) streamk_fixup_kernel(EP ep, int tiles_m, StreamK sk)
+{
+    const int tid = threadIdx.x;
+    const int tile = blockIdx.x;
+    const int quad = blockIdx.y;  // registers [4*quad, 4*quad + 4) in (i, j, v) order
+    const long total = (long)sk.sk_tiles * sk.units;
+    const long a = (long)tile * sk.units, b = a + sk.units;
+    // the workgroup whose range holds unit a
+    int g = (int)(((a + 1) * sk.sk_blocks - 1) / total);
+    while (g > 0 && sk_first_unit(g, total, sk.sk_blocks) > a) --g;
+    while (g + 1 < sk.sk_blocks && sk_first_unit(g + 1, total, sk.sk_blocks) <= a) ++g;
+    if (sk_first_unit(g + 1, total, sk.sk_blocks) >= b) return;  // it held the whole tile and stored it
+
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (; g < sk.sk_blocks; ++g) {
+        const long s0 = sk_first_unit(g, total, sk.sk_blocks), s1 = sk_first_unit(g + 1, total, sk.sk_blocks);
+        if (s0 >= b) break;
+        const long piece0 = s0 > a ? s0 : a, piece1 = s1 < b ? s1 : b;
+        if (piece1 <= piece0) continue;
+        const float* src =
+            sk.partial + (size_t)(2 * g + (piece0 == s0 ? 0 : 1)) * (T::BM * T::BN) + quad * 4 * kThreads + tid;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) acc[q] += src[q * kThreads];
+    }
+    const int ij = quad >> 2, i = ij / T::TN, j = ij - i * T::TN, v0 = (quad & 3) * 4;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm0 = (wave % T::WGM) * T::WM, wn0 = (wave / T::WGM) * T::WN;
+    const int frag_r = lane & 31, frag_k = lane >> 5;
+    const int m0 = (tile % tiles_m) * T::BM, n0 = (tile / tiles_m) * T::BN;
+    const typename EP::Col col = ep.column(n0 + wn0 + j * 32 + frag_r, 0);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) ep.store(col, m0 + wm0 + i * 32 + 8 * ((v0 + q) / 4) + 4 * frag_k + ((v0 + q) % 4), acc[q]);
+}
+
+// Workgroups of gemm_streamk_kernel<T, ...> the device holds at once.
+template <class T, class AL, class BL, class EP>
+inline int resident_workgroups()
+{
+    static int cached = 0;
+    if (cached == 0) {
+        int dev = 0, cus = 0, per_cu = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+            hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_streamk_kernel<T, AL, BL, EP>, kThreads, 0) !=
+                hipSuccess ||
+            cus <= 0 || per_cu <= 0)
+            return 0;
+        cached = cus * per_cu;
+    }
+    return cached;
+}
+
+inline size_t streamk_workspace_bytes(int resident, int bm, int bn) { return (size_t)2 * resident * bm * bn * 4; }
+
+// C = A*B over the full reduction range [0, k), balanced as described above when that pays and
+// `partial` is large enough; otherwise the plain grid of whole tiles.
+template <class T, class AL, class BL, class EP>
+inline int launch_balanced(const AL& al, const BL& bl, const EP& ep, long m, long n, int k, float* partial,
+                           size_t partial_bytes, hipStream_t stream)
+{
+    const long tiles_m = (m + T::BM - 1) / T::BM, tiles_n = (n + T::BN - 1) / T::BN;
+    const long tiles = tiles_m * tiles_n;
+    if (tiles >= (1l << 31)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+    const int resident = resident_workgroups<T, AL, BL, EP>();
+    const int units = (k + 2 * BK - 1) / (2 * BK);
+    bool balanced = resident > 0 && partial && partial_bytes >= streamk_workspace_bytes(resident, T::BM, T::BN) &&
+                    tiles % resident != 0 && tiles < 16l * resident && units >= 8;
+    if (!balanced) return launch<T>(al, bl, ep, m, n, no_split(k), 1, stream);
+    StreamK sk;
+    sk.tiles = (int)tiles;
+    sk.sk_tiles = (int)(tiles % resident);
+    sk.units = units;
+    sk.k = k;
+    sk.partial = partial;
+    const long total = (long)sk.sk_tiles * units;
+    sk.sk_blocks = (int)(total / 4 < resident ? (total / 4 > 0 ? total / 4 : 1) : resident);
+    hipLaunchKernelGGL((gemm_streamk_kernel<T, AL, BL, EP>), dim3((unsigned)resident), dim3(kThreads), 0, stream, al,
+                       bl, ep, (int)tiles_m, sk);
+    HIP_RETURN_IF_LAUNCH_FAILED();
+    if (sk.sk_tiles > 0) {
+        hipLaunchKernelGGL((streamk_fixup_kernel<T, EP>), dim3((unsigned)sk.sk_tiles, T::TM * T::TN * 4), dim3(kThreads), 0,
+                           stream, ep, (int)tiles_m, sk);
+        HIP_RETURN_IF_LAUNCH_FAILED();
+    }
     return PYDTNN_HIP_OK;
 }
 

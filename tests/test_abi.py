@@ -57,8 +57,12 @@ def test_workspace_queries_are_pure_host_code(native):
     kn_k = 256 * 2304 * 4
     dw = lib.pydtnn_hip_conv_workspace_bytes(native.OP_DW, 0, *cfg2)
     assert dw % kn_k == 0 and 1 <= dw // kn_k <= 64 * 4
-    # stride 1: dX only needs the flipped filter; strided: the (K x P) matrix of the explicit route
-    assert lib.pydtnn_hip_conv_workspace_bytes(native.OP_DX, 0, *cfg2) == kn_k
+    # forward: optional scratch of the balanced launch, two 128x128 accumulator tiles for each of 1024 workgroups
+    balance = 2 * 1024 * 128 * 128 * 4
+    assert lib.pydtnn_hip_conv_workspace_bytes(native.OP_FWD, 0, *cfg2) == balance
+    # stride 1: dX needs the flipped filter and runs as a forward launch; strided: the (K x P) matrix of the
+    # explicit route
+    assert lib.pydtnn_hip_conv_workspace_bytes(native.OP_DX, 0, *cfg2) == kn_k + balance
     strided = (8, 3, 32, 32, 16, 3, 3, 1, 1, 2, 2, 1, 1)
     assert lib.pydtnn_hip_conv_workspace_bytes(native.OP_DX, 0, *strided) == 27 * 8 * 16 * 16 * 4
     assert lib.pydtnn_hip_conv_workspace_bytes(native.OP_DX_I2C, 1, *cfg2) == 2304 * 64 * 56 * 56 * 4
