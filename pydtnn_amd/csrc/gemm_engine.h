@@ -302,8 +302,8 @@ struct Im2colNchwMN {
     const float* x;
     ConvGeom g;
     struct State {
-        rsrc_t rsrc;
-        uint32_t base;   // byte offset of (img, c=0, ih0, iw0), modulo 2^32; only used with a valid tap
+        rsrc_t rsrc;     // starts `lead` floats before x, so that every thread's base offset is >= 0
+        uint32_t base;   // byte offset of (img, c=0, ih0, iw0) from there
         uint32_t inv0;   // narrow: combined tap mask; wide: mask over i
         uint32_t inv1;   // wide: mask over j
         int krow;
@@ -311,7 +311,11 @@ struct Im2colNchwMN {
     struct Iter {};
     __device__ __forceinline__ void init(State& s, int origin, int /*image*/, int tid) const
     {
-        s.rsrc = make_rsrc(x, (long)g.n * g.c * g.h * g.w);
+        // ih0*w + iw0 >= -(vpadding*w + hpadding): shifting the descriptor back by that much keeps the
+        // per-thread offset unsigned, and the tap's own offset (>= 0) can then ride in the scalar offset
+        // operand of the load, which the hardware adds after its range check of the vector offset.
+        const int lead = g.vpadding * g.w + g.hpadding;
+        s.rsrc = make_rsrc(x - lead, (long)g.n * g.c * g.h * g.w + lead);
         long n = (long)origin + Map::mn(tid);
         n = n < g.p ? n : g.p - 1;
         const int img = (int)(n / g.howo);
@@ -320,7 +324,7 @@ struct Im2colNchwMN {
         const int ih0 = yy * g.vstride - g.vpadding;
         const int iw0 = xx * g.hstride - g.hpadding;
         s.krow = Map::krow(tid);
-        s.base = (uint32_t)((img * g.c * g.h + ih0) * g.w + iw0) * 4u;
+        s.base = (uint32_t)((img * g.c * g.h + ih0) * g.w + iw0 + lead) * 4u;
         if (WIDE) {
             s.inv0 = tap_mask_axis(ih0, g.kh, g.vdilation, g.h);
             s.inv1 = tap_mask_axis(iw0, g.kw, g.hdilation, g.w);
@@ -333,7 +337,7 @@ struct Im2colNchwMN {
     template <int E>
     __device__ __forceinline__ float elem(const State& s, const Iter&, int k0, int kend) const
     {
-        // scalar: reduction index -> (c, i, j) -> float offset of the tap inside one image
+        // scalar: reduction index -> (c, i, j) -> byte offset of the tap inside one image
         const uint32_t k = (uint32_t)(k0 + s.krow + E * Map::kRowsPerPass);
         const uint32_t cc = fd_div(k, g.fd_khw);
         const uint32_t rem = k - cc * g.khw;
@@ -341,12 +345,14 @@ struct Im2colNchwMN {
         const uint32_t jj = rem - ii * g.kw;
         const uint32_t off = (uint32_t)(((int)cc * g.h + (int)ii * g.vdilation) * g.w + (int)jj * g.hdilation) * 4u;
         const bool live = (int)k < kend;
-        uint32_t invalid;
-        if (WIDE)
-            invalid = __builtin_amdgcn_ubfe(s.inv0, live ? ii : 31u, 1) | __builtin_amdgcn_ubfe(s.inv1, jj, 1);
-        else
-            invalid = __builtin_amdgcn_ubfe(s.inv0, live ? rem : 31u, 1);
-        return buf_load(s.rsrc, guarded_offset(invalid, s.base + off), 0);
+        if (WIDE) {
+            const uint32_t invalid =
+                __builtin_amdgcn_ubfe(s.inv0, live ? ii : 31u, 1) | __builtin_amdgcn_ubfe(s.inv1, jj, 1);
+            return buf_load(s.rsrc, guarded_offset(invalid, s.base), off);
+        }
+        // two vector instructions per element: move the tap's mask bit to bit 31, merge it into the offset
+        const uint32_t bit = live ? rem : 31u;
+        return buf_load(s.rsrc, ((s.inv0 << (31u - bit)) & kOob) | s.base, off);
     }
     __device__ __forceinline__ void store(float* lds, const float (&r)[NLD], int tid) const { Map::store(lds, r, tid); }
 };
