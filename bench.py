@@ -27,8 +27,9 @@ HBM_PEAK_GBS = 8000.0
 
 # HBM-side bytes per launch of the forward kernel, from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE), each
 # scaled by what the same counter reads for a 256 MiB copy (factors 2.000 and 1.000):
-# (191273.3 * 2.0 + 200704.0) KiB.  The summary of those runs is profiles/cfg2_conv3x3_pmc_counters.md.
-MEASURED_TRAFFIC_BYTES = {"cfg2": int((191273.3 * 2.0 + 200704.0) * 1024)}
+# main launch (194063.3 * 2.0 + 245760.0) KiB plus the fixup launch of its cut tiles (24631.4 * 2.0 + 4096.0) KiB.
+# The summary of those runs is profiles/cfg2_conv3x3_pmc_counters.md.
+MEASURED_TRAFFIC_BYTES = {"cfg2": int((194063.3 * 2.0 + 245760.0 + 24631.4 * 2.0 + 4096.0) * 1024)}
 
 
 def parse_args():
@@ -166,7 +167,7 @@ def run_cfg2(torch, pd, args):
     torch.cuda.synchronize()
     extra["im2row_gbs"] = round(stream_bytes / (rows_t.mean_ms() * 1e-3) / 1e9, 1)
     extra["row2im_gbs"] = round(stream_bytes / (r2i_t.mean_ms() * 1e-3) / 1e9, 1)
-    roofline = {"bound": "mfma", "kernel": "gemm_kernel<128x128, PlainK, Im2colNchwMN, EpiNchw> (forward)",
+    roofline = {"bound": "mfma", "kernel": "gemm_streamk_kernel<128x128, PlainK, Im2colNchwMN, EpiNchw> + streamk_fixup_kernel (forward)",
                 "achieved": round(achieved, 3), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES["cfg2"]}
     workload = ("cfg2: VGG16-style 3x3 conv layer fwd+dW+db+dX, fp32 NCHW, N=64, 256->256, 56x56, stride 1, pad 1, "
