@@ -188,6 +188,21 @@ int pydtnn_hip_max_pool_2d_bwd_nchw(const float *dy, const int32_t *idx_max, flo
                                     int kh, int kw, int vpadding, int hpadding, int vstride, int hstride,
                                     int vdilation, int hdilation, void *stream);
 
+/* Softmax over the rows of a (rows, cols) matrix and its backward
+ * (pydtnn/backends/cpu/activations/softmax_cpu.py:32-39):
+ *   y = exp(x - max(x, axis=1)) / sum(...);   dx = y * (dy - sum(dy * y, axis=1)). */
+int pydtnn_hip_softmax_fwd(const float *x, float *y, int rows, int cols, void *stream);
+int pydtnn_hip_softmax_bwd(const float *dy, const float *y, float *dx, int rows, int cols, void *stream);
+
+/* Categorical cross-entropy and its gradient
+ * (pydtnn/backends/cpu/losses/categorical_cross_entropy_cpu.py:28-35): with a = first argmax of
+ * y_targ[row] and p = clip(y_pred[row, a], eps, 1 - eps) (bounds rounded to float32),
+ *   loss[0] = -sum_rows log(p) / rows;   dx = y_targ except dx[row, a] = y_targ[row, a] / (-p * global_batch).
+ * Workspace: rows * 4 bytes. */
+int pydtnn_hip_categorical_cross_entropy(const float *y_pred, const float *y_targ, float *dx, float *loss, int rows,
+                                         int cols, double eps, int global_batch, void *workspace,
+                                         size_t workspace_bytes, void *stream);
+
 /* SGD with momentum, in place (pydtnn/backends/cpu/optimizers/sgd_cpu.py:28-41). */
 int pydtnn_hip_sgd_momentum(float *w, const float *dw, float *velocity, long total, float lr, float momentum,
                             float decay, int nesterov, void *stream);

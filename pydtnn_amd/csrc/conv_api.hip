@@ -14,6 +14,9 @@ size_t bias_grad_workspace_floats(long, int);
 int launch_bias_grad(const float*, float*, long, int, int, float*, hipStream_t);
 int launch_splitk_reduce(const float*, float*, long, int, long, int, int, int, const ChanEpilogue&, hipStream_t);
 int launch_flip_filter(const float*, float*, int, int, int, int, int, hipStream_t);
+int launch_softmax_fwd(const float*, float*, int, int, hipStream_t);
+int launch_softmax_bwd(const float*, const float*, float*, int, int, hipStream_t);
+int launch_cce(const float*, const float*, float*, float*, float*, int, int, float, float, float, hipStream_t);
 int launch_max_pool_fwd_nchw(const float*, float*, int32_t*, const ConvGeom&, hipStream_t);
 int launch_max_pool_bwd_nchw(const float*, const int32_t*, float*, const ConvGeom&, hipStream_t);
 int launch_sgd_momentum(float*, const float*, float*, long, float, float, float, int, hipStream_t);
@@ -675,6 +678,29 @@ int pydtnn_hip_max_pool_2d_bwd_nchw(const float* dy, const int32_t* idx_max, flo
     const int kn = 1;
     const int rc = geom_from_args(&g, GEOM_ARGS);
     return rc != PYDTNN_HIP_OK ? rc : launch_max_pool_bwd_nchw(dy, idx_max, dx, g, as_stream(stream));
+}
+
+int pydtnn_hip_softmax_fwd(const float* x, float* y, int rows, int cols, void* stream)
+{
+    if (!x || !y) return PYDTNN_HIP_ERR_INVALID;
+    return launch_softmax_fwd(x, y, rows, cols, as_stream(stream));
+}
+
+int pydtnn_hip_softmax_bwd(const float* dy, const float* y, float* dx, int rows, int cols, void* stream)
+{
+    if (!dy || !y || !dx) return PYDTNN_HIP_ERR_INVALID;
+    return launch_softmax_bwd(dy, y, dx, rows, cols, as_stream(stream));
+}
+
+int pydtnn_hip_categorical_cross_entropy(const float* y_pred, const float* y_targ, float* dx, float* loss, int rows,
+                                         int cols, double eps, int global_batch, void* workspace,
+                                         size_t workspace_bytes, void* stream)
+{
+    if (!y_pred || !y_targ || !dx || !loss || global_batch <= 0) return PYDTNN_HIP_ERR_INVALID;
+    if (!workspace || workspace_bytes < (size_t)(rows > 0 ? rows : 0) * 4) return PYDTNN_HIP_ERR_WORKSPACE;
+    // the reference clips a float32 array with float64 bounds: the bounds are rounded to float32 first
+    return launch_cce(y_pred, y_targ, dx, loss, (float*)workspace, rows, cols, (float)eps, (float)(1.0 - eps),
+                      (float)global_batch, as_stream(stream));
 }
 
 int pydtnn_hip_sgd_momentum(float* w, const float* dw, float* velocity, long total, float lr, float momentum,

@@ -328,6 +328,112 @@ __global__ void __launch_bounds__(kThreads) sgd_momentum_kernel(float* __restric
     velocity[idx] = v;
 }
 
+// ---------------------------------------------------------------- softmax and categorical cross-entropy
+// Rows of a (rows, cols) matrix, one workgroup per row.
+template <class Op>
+__device__ __forceinline__ float block_reduce(float v, Op op, float* red)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = op(v, __shfl_xor(v, off, 64));
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __syncthreads();  // red may still be read from a previous call
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    float r = red[0];
+#pragma unroll
+    for (int i = 1; i < kThreads / 64; ++i) r = op(r, red[i]);
+    return r;  // the same value in every thread
+}
+
+struct MaxOp { __device__ float operator()(float a, float b) const { return a > b ? a : b; } };
+struct SumOp { __device__ float operator()(float a, float b) const { return a + b; } };
+
+// pydtnn/backends/cpu/activations/softmax_cpu.py:32-35: y = exp(x - max(x)); y /= sum(y)
+__global__ void __launch_bounds__(kThreads) softmax_fwd_kernel(const float* __restrict__ x, float* __restrict__ y,
+                                                              int cols)
+{
+    __shared__ float red[kThreads / 64];
+    const float* xr = x + (long)blockIdx.x * cols;
+    float* yr = y + (long)blockIdx.x * cols;
+    float m = -3.402823466e+38f;
+    for (int c = threadIdx.x; c < cols; c += kThreads) m = fmaxf(m, xr[c]);
+    m = block_reduce(m, MaxOp(), red);
+    float sum = 0.0f;
+    for (int c = threadIdx.x; c < cols; c += kThreads) {
+        const float e = expf(xr[c] - m);
+        yr[c] = e;
+        sum += e;
+    }
+    sum = block_reduce(sum, SumOp(), red);
+    for (int c = threadIdx.x; c < cols; c += kThreads) yr[c] = yr[c] / sum;
+}
+
+// softmax_cpu.py:37-39: dx = y * (dy - sum(dy * y))
+__global__ void __launch_bounds__(kThreads) softmax_bwd_kernel(const float* __restrict__ dy,
+                                                              const float* __restrict__ y, float* __restrict__ dx,
+                                                              int cols)
+{
+    __shared__ float red[kThreads / 64];
+    const long base = (long)blockIdx.x * cols;
+    float dot = 0.0f;
+    for (int c = threadIdx.x; c < cols; c += kThreads) dot += dy[base + c] * y[base + c];
+    dot = block_reduce(dot, SumOp(), red);
+    for (int c = threadIdx.x; c < cols; c += kThreads) dx[base + c] = y[base + c] * (dy[base + c] - dot);
+}
+
+// pydtnn/backends/cpu/losses/categorical_cross_entropy_cpu.py:28-35, one row per workgroup:
+//   a = first argmax of y_targ[row];  p = clip(y_pred[row, a], lo, hi);  row_loss[row] = log(p);
+//   dx[row] = y_targ[row] except dx[row, a] = y_targ[row, a] / (-p * global_batch)
+__global__ void __launch_bounds__(kThreads) cce_rows_kernel(const float* __restrict__ y_pred,
+                                                           const float* __restrict__ y_targ, float* __restrict__ dx,
+                                                           float* __restrict__ row_loss, int cols, float lo, float hi,
+                                                           float global_batch)
+{
+    __shared__ float best_v[kThreads];
+    __shared__ int best_i[kThreads];
+    const long base = (long)blockIdx.x * cols;
+    float bv = -3.402823466e+38f;
+    int bi = 0x7fffffff;
+    for (int c = threadIdx.x; c < cols; c += kThreads) {
+        const float v = y_targ[base + c];
+        dx[base + c] = v;
+        if (bi == 0x7fffffff || v > bv) { bv = v; bi = c; }
+    }
+    best_v[threadIdx.x] = bv;
+    best_i[threadIdx.x] = bi;
+    __syncthreads();
+    for (int off = kThreads / 2; off > 0; off >>= 1) {
+        if ((int)threadIdx.x < off) {
+            const float ov = best_v[threadIdx.x + off];
+            const int oi = best_i[threadIdx.x + off];
+            const float mv = best_v[threadIdx.x];
+            const int mi = best_i[threadIdx.x];
+            // larger value wins; on a tie the smaller column (numpy.argmax returns the first maximum)
+            if (oi != 0x7fffffff && (mi == 0x7fffffff || ov > mv || (ov == mv && oi < mi))) {
+                best_v[threadIdx.x] = ov;
+                best_i[threadIdx.x] = oi;
+            }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        const int a = best_i[0];
+        float p = y_pred[base + a];
+        p = p < lo ? lo : (p > hi ? hi : p);
+        row_loss[blockIdx.x] = logf(p);
+        dx[base + a] = best_v[0] / (-p * global_batch);
+    }
+}
+
+// loss = -sum(row_loss) / rows, rows added in ascending order by one thread.
+__global__ void cce_loss_kernel(const float* __restrict__ row_loss, float* __restrict__ loss, int rows)
+{
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    float acc = 0.0f;
+    for (int r = 0; r < rows; ++r) acc += row_loss[r];
+    loss[0] = -acc / (float)rows;
+}
+
 }  // namespace
 
 // Algorithmic bytes: 2 * 4 * total (+ 4 * total when a residual is read).
@@ -468,6 +574,34 @@ int launch_sgd_momentum(float* w, const float* dw, float* velocity, long total, 
     if (total <= 0) return PYDTNN_HIP_ERR_INVALID;
     hipLaunchKernelGGL(sgd_momentum_kernel, dim3(blocks_for(total)), dim3(kThreads), 0, stream, w, dw, velocity, total,
                        lr, momentum, decay, nesterov);
+    HIP_RETURN_IF_LAUNCH_FAILED();
+    return PYDTNN_HIP_OK;
+}
+
+int launch_softmax_fwd(const float* x, float* y, int rows, int cols, hipStream_t stream)
+{
+    if (rows <= 0 || cols <= 0) return PYDTNN_HIP_ERR_INVALID;
+    hipLaunchKernelGGL(softmax_fwd_kernel, dim3(rows), dim3(kThreads), 0, stream, x, y, cols);
+    HIP_RETURN_IF_LAUNCH_FAILED();
+    return PYDTNN_HIP_OK;
+}
+
+int launch_softmax_bwd(const float* dy, const float* y, float* dx, int rows, int cols, hipStream_t stream)
+{
+    if (rows <= 0 || cols <= 0) return PYDTNN_HIP_ERR_INVALID;
+    hipLaunchKernelGGL(softmax_bwd_kernel, dim3(rows), dim3(kThreads), 0, stream, dy, y, dx, cols);
+    HIP_RETURN_IF_LAUNCH_FAILED();
+    return PYDTNN_HIP_OK;
+}
+
+int launch_cce(const float* y_pred, const float* y_targ, float* dx, float* loss, float* row_loss, int rows, int cols,
+               float lo, float hi, float global_batch, hipStream_t stream)
+{
+    if (rows <= 0 || cols <= 0) return PYDTNN_HIP_ERR_INVALID;
+    hipLaunchKernelGGL(cce_rows_kernel, dim3(rows), dim3(kThreads), 0, stream, y_pred, y_targ, dx, row_loss, cols, lo,
+                       hi, global_batch);
+    HIP_RETURN_IF_LAUNCH_FAILED();
+    hipLaunchKernelGGL(cce_loss_kernel, dim3(1), dim3(64), 0, stream, row_loss, loss, rows);
     HIP_RETURN_IF_LAUNCH_FAILED();
     return PYDTNN_HIP_OK;
 }

@@ -165,7 +165,7 @@ class Relu(Layer):
 
 
 class Softmax(Layer):
-    """pydtnn/backends/cpu/activations/softmax_cpu.py:25-39 (a (batch, classes) matrix; torch ops)."""
+    """pydtnn/backends/cpu/activations/softmax_cpu.py:25-39 (a (batch, classes) matrix)."""
 
     def __init__(self, shape=(1,)):
         super().__init__(shape)
@@ -176,13 +176,12 @@ class Softmax(Layer):
         self.shape = prev_shape
 
     def forward(self, x):
-        self.y = torch.exp(x - torch.max(x, dim=1, keepdim=True).values)
-        self.y /= torch.sum(self.y, dim=1, keepdim=True)
+        self.y = ops.softmax(x)
         return self.y
 
     def backward(self, dy):
         if self.need_dx:
-            return self.y * (dy - (dy * self.y).sum(dim=1, keepdim=True))
+            return ops.softmax_backward(dy, self.y)
 
 
 activations = {"relu": Relu, "softmax": Softmax}

@@ -207,6 +207,41 @@ def max_pool_2d_bwd_nchw(dy, idx_max, n, c, h, w, kh, kw, vpadding, hpadding, vs
     return dx
 
 
+def softmax(x):
+    """pydtnn/backends/cpu/activations/softmax_cpu.py:32-35 on a (batch, classes) matrix."""
+    _need_f32(x)
+    if x.dim() != 2:
+        raise ValueError("softmax expects a (batch, classes) matrix")
+    x = x.contiguous()
+    y = torch.empty_like(x)
+    check(lib().pydtnn_hip_softmax_fwd(f32(x), f32(y), x.shape[0], x.shape[1], stream_ptr()), "softmax_fwd")
+    return y
+
+
+def softmax_backward(dy, y):
+    """pydtnn/backends/cpu/activations/softmax_cpu.py:37-39"""
+    _need_f32(dy, y)
+    dy, y = dy.contiguous(), y.contiguous()
+    dx = torch.empty_like(y)
+    check(lib().pydtnn_hip_softmax_bwd(f32(dy), f32(y), f32(dx), y.shape[0], y.shape[1], stream_ptr()),
+          "softmax_bwd")
+    return dx
+
+
+def categorical_cross_entropy(y_pred, y_targ, global_batch_size, eps=1e-8):
+    """pydtnn/backends/cpu/losses/categorical_cross_entropy_cpu.py:28-35.  Returns (loss as a 0-d tensor, dx)."""
+    _need_f32(y_pred, y_targ)
+    y_pred, y_targ = y_pred.contiguous(), y_targ.contiguous()
+    rows, cols = y_pred.shape
+    dx = torch.empty_like(y_targ)
+    loss = torch.empty(1, dtype=torch.float32, device=y_pred.device)
+    ws, ws_bytes = native.workspace(rows * 4)
+    check(lib().pydtnn_hip_categorical_cross_entropy(f32(y_pred), f32(y_targ), f32(dx), f32(loss), rows, cols,
+                                                     float(eps), int(global_batch_size), ws, ws_bytes,
+                                                     stream_ptr()), "categorical_cross_entropy")
+    return loss[0], dx
+
+
 def sgd_momentum(w, dw, velocity, lr, momentum, decay=0.0, nesterov=False):
     """In place SGD step (pydtnn/backends/cpu/optimizers/sgd_cpu.py:28-41)."""
     _need_f32(w, dw, velocity)

@@ -351,6 +351,37 @@ def test_sgd_momentum(ops, oracle):
     assert_close(host(vd), v_ref, tol=1e-6, what="sgd v")
 
 
+@pytest.mark.parametrize("rows,cols", [(64, 1000), (3, 7), (1, 1), (5, 300), (2, 4097)])
+def test_softmax_forward_backward(ops, oracle, rows, cols):
+    announce("softmax", (rows, cols))
+    rng = np.random.default_rng(rows * 131 + cols)
+    x = (rng.standard_normal((rows, cols)) * 4).astype(np.float32)
+    dy = rng.standard_normal((rows, cols)).astype(np.float32)
+    y = ops.softmax(dev(x))
+    y_ref = oracle.softmax_forward(x)
+    assert_close(host(y), y_ref, tol=1e-6, what="softmax y")
+    np.testing.assert_allclose(host(y).sum(axis=1), 1.0, rtol=1e-5)
+    dx = ops.softmax_backward(dev(dy), dev(y_ref))
+    assert_close(host(dx), oracle.softmax_backward(dy, y_ref), tol=1e-5, what="softmax dx")
+
+
+@pytest.mark.parametrize("rows,cols", [(64, 1000), (3, 7), (1, 1), (5, 300)])
+def test_categorical_cross_entropy(ops, oracle, rows, cols):
+    announce("cce", (rows, cols))
+    rng = np.random.default_rng(rows * 17 + cols)
+    y_pred = oracle.softmax_forward(rng.standard_normal((rows, cols)).astype(np.float32) * 3)
+    y_targ = np.eye(cols, dtype=np.float32)[rng.integers(0, cols, rows)]
+    if rows >= 3 and cols >= 7:
+        y_pred[0, :] = 0.0                     # exercises the lower clip bound
+        y_targ[1, :] = 0.0                     # all equal: argmax is column 0
+        y_targ[2, :] = 0.0
+        y_targ[2, 3] = y_targ[2, 5] = 0.5      # tie: first maximum wins
+    loss, dx = ops.categorical_cross_entropy(dev(y_pred), dev(y_targ), 2 * rows)
+    loss_ref, dx_ref = oracle.categorical_cross_entropy(y_pred, y_targ, 2 * rows)
+    assert abs(float(loss) - float(loss_ref)) <= 1e-5 * max(1.0, abs(float(loss_ref)))
+    np.testing.assert_allclose(host(dx), dx_ref, rtol=2e-6, atol=0)
+
+
 # ------------------------------------------------------------------ host-pointer compatibility ABI
 
 def test_libconvgemm_compat_abi_runs_like_the_reference_shim(oracle):
