@@ -49,7 +49,20 @@ __global__ void __launch_bounds__(kThreads) im2col_nchw_lds_kernel(const float* 
     r1 = r1 > g.h - 1 ? g.h - 1 : r1;
     const float* plane = x + (size_t)(nn * g.c + cc) * g.h * g.w;
     const int start = r0 * g.w, end = (r1 + 1) * g.w;
-    for (int i = start + (int)threadIdx.x; i < end; i += kThreads) win[i - start] = plane[i];
+    // eight loads in flight per thread before the first LDS store
+    for (int i0 = start + (int)threadIdx.x; i0 < end; i0 += 8 * kThreads) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = i0 + u * kThreads;
+            v[u] = plane[i < end ? i : start];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = i0 + u * kThreads;
+            if (i < end) win[i - start] = v[u];
+        }
+    }
     __syncthreads();
 
     const uint32_t pp = pp_begin + threadIdx.x * 4;
@@ -190,9 +203,10 @@ __global__ void __launch_bounds__(kThreads) col2im_nchw_kernel(const float* __re
 }
 
 // ---------------------------------------------------------------- im2row NHWC
-// One block owns `rpb` consecutive pixel rows of the matrix (a contiguous run of rpb*k floats) and
-// its threads walk that run, so stores are fully coalesced; the block's first pixel is decomposed
-// once with scalar arithmetic and each element only needs multiply-high divisions.
+// One block owns `rpb`
+// consecutive pixel rows of the matrix (a contiguous run of rpb*k floats) and its threads walk that
+// run, so stores are fully coalesced; the block's first pixel is decomposed once with scalar
+// arithmetic and each element only needs multiply-high divisions.
 __global__ void __launch_bounds__(kThreads) im2row_nhwc_kernel(const float* __restrict__ x,
                                                               float* __restrict__ rows, ConvGeom g, int rpb,
                                                               FastDiv fd_k)
@@ -225,7 +239,8 @@ __global__ void __launch_bounds__(kThreads) im2row_nhwc_kernel(const float* __re
 }
 
 // ---------------------------------------------------------------- row2im NHWC (gather form)
-// grid.x * 256 threads walk one image of dx (h*w*c floats, lanes along c), grid.y walks the images.
+// grid.x * 256 threads walk one image of dx (h*w*c floats, lanes along c), grid.y walks
+// the images.
 template <bool UNIT>
 __global__ void __launch_bounds__(kThreads) row2im_nhwc_kernel(const float* __restrict__ rows,
                                                               float* __restrict__ dx, ConvGeom g, int c_exact)

@@ -83,3 +83,18 @@ small_grid = [
     D(3, 1, 10, 7, 2, 2, 3, 3, 4, 1, 2, 1, 1),
     D(2, 6, 9, 9, 5, 3, 3, 1, 1, 2, 2, 1, 2),
 ]
+
+# Channel counts from 32 up, where the NHWC gathers take their LDS-staged form: slabs that are not
+# multiples of 64, more than one slab, segments that do not divide the row, strides, dilation,
+# rectangular filters, padding larger than the filter reach, a filter wider than the image interior.
+wide_channel_grid = [
+    D(2, 32, 9, 11, 4, 3, 3, 1, 1, 1, 1, 1, 1),
+    D(1, 40, 7, 19, 3, 3, 3, 1, 1, 1, 1, 1, 1),
+    D(2, 64, 12, 17, 5, 3, 3, 1, 1, 2, 2, 1, 1),
+    D(1, 96, 10, 10, 2, 5, 3, 2, 1, 1, 1, 1, 1),
+    D(1, 130, 8, 21, 2, 3, 3, 2, 2, 1, 1, 2, 2),
+    D(2, 72, 9, 33, 2, 2, 4, 0, 3, 1, 3, 1, 1),
+    D(1, 300, 6, 6, 2, 1, 1, 0, 0, 1, 1, 1, 1),
+    D(1, 64, 5, 40, 2, 3, 7, 1, 3, 2, 1, 1, 2),
+    D(1, 48, 14, 14, 2, 3, 3, 3, 3, 2, 2, 1, 1),
+]

@@ -10,7 +10,7 @@ import pytest
 import torch
 
 from gpu_util import FP32_REL_TOL, announce, assert_close, dev, host, rel_err
-from shapes import D, alexnet_layers, small_grid, x_2x4, x_2x4_c2, x_4x4, x_4x8, x_8x8, w_1x1, w_1x2, w_2x2, w_3x3, \
+from shapes import D, alexnet_layers, small_grid, wide_channel_grid, x_2x4, x_2x4_c2, x_4x4, x_4x8, x_8x8, w_1x1, w_1x2, w_2x2, w_3x3, \
     w_c2_1234_4567
 
 pytestmark = pytest.mark.gpu
@@ -87,6 +87,23 @@ def test_im2row_row2im_nhwc_bit_exact(ops, oracle, d):
     rmat = rng.standard_normal(ref.shape).astype(np.float32)
     dx = ops.row2im_nhwc(dev(rmat), d.b, d.h, d.w, d.c, *d.geom())
     assert np.array_equal(host(dx), oracle.row2im_nhwc(rmat, d.b, d.h, d.w, d.c, *d.geom()))
+
+
+@pytest.mark.parametrize("d", wide_channel_grid, ids=repr)
+def test_nhwc_gathers_staged_form_bit_exact(ops, oracle, d):
+    announce("im2row/row2im nhwc staged", d)
+    x, _, _, _ = case(d)
+    xr = nhwc(x)
+    assert np.array_equal(host(ops.im2row_nhwc(dev(xr), *d.geom())), oracle.im2row_nhwc(xr, *d.geom()))
+    rng = np.random.default_rng(2)
+    rmat = rng.standard_normal((d.b * d.ho * d.wo, d.c * d.kh * d.kw)).astype(np.float32)
+    dx = ops.row2im_nhwc(dev(rmat), d.b, d.h, d.w, d.c, *d.geom())
+    assert np.array_equal(host(dx), oracle.row2im_nhwc(rmat, d.b, d.h, d.w, d.c, *d.geom()))
+    # the NCHW pair on the same geometry (its staged im2col has its own segmenting)
+    assert np.array_equal(host(ops.im2col_nchw(dev(x), *d.geom())), oracle.im2col_nchw(x, *d.geom()))
+    cmat = np.ascontiguousarray(rmat.T)
+    dxc = ops.col2im_nchw(dev(cmat), d.b, d.c, d.h, d.w, *d.geom())
+    assert np.array_equal(host(dxc), oracle.col2im_nchw(cmat, d.b, d.c, d.h, d.w, *d.geom()))
 
 
 def test_im2col_unaligned_column_count(ops, oracle):
