@@ -218,23 +218,34 @@ __global__ void __launch_bounds__(kThreads) im2row_nhwc_kernel(const float* __re
     const uint32_t pp0 = row0 - n0 * g.howo;
     const uint32_t count = nrows * (uint32_t)g.k;
     float* dst = rows + (long)row0 * g.k;
-    for (uint32_t e = threadIdx.x; e < count; e += kThreads) {
-        const uint32_t r = rpb > 1 ? fd_div(e, fd_k) : 0u;
-        const uint32_t col = e - r * g.k;
-        uint32_t pp = pp0 + r, nn = n0;
-        if (pp >= (uint32_t)g.howo) { pp -= g.howo; ++nn; }  // rpb <= howo: at most one wrap
-        const uint32_t yy = fd_div(pp, g.fd_wo);
-        const uint32_t xx = pp - yy * g.wo;
-        const uint32_t cc = fd_div(col, g.fd_khw);
-        const uint32_t rem = col - cc * g.khw;
-        const uint32_t ii = fd_div(rem, g.fd_kw);
-        const uint32_t jj = rem - ii * g.kw;
-        const int x_x = g.vstride * (int)yy + g.vdilation * (int)ii - g.vpadding;
-        const int x_y = g.hstride * (int)xx + g.hdilation * (int)jj - g.hpadding;
-        float val = 0.0f;
-        if ((unsigned)x_x < (unsigned)g.h && (unsigned)x_y < (unsigned)g.w)
-            val = x[((nn * g.h + x_x) * g.w + x_y) * g.c + cc];
-        dst[e] = val;
+    // four elements per trip: their loads are issued together (clamped index, then select)
+    for (uint32_t e0 = threadIdx.x; e0 < count; e0 += 4 * kThreads) {
+        float v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const uint32_t e = e0 + u * kThreads;
+            const uint32_t ec = e < count ? e : 0u;
+            const uint32_t r = rpb > 1 ? fd_div(ec, fd_k) : 0u;
+            const uint32_t col = ec - r * g.k;
+            uint32_t pp = pp0 + r, nn = n0;
+            if (pp >= (uint32_t)g.howo) { pp -= g.howo; ++nn; }  // rpb <= howo: at most one wrap
+            const uint32_t yy = fd_div(pp, g.fd_wo);
+            const uint32_t xx = pp - yy * g.wo;
+            const uint32_t cc = fd_div(col, g.fd_khw);
+            const uint32_t rem = col - cc * g.khw;
+            const uint32_t ii = fd_div(rem, g.fd_kw);
+            const uint32_t jj = rem - ii * g.kw;
+            const int x_x = g.vstride * (int)yy + g.vdilation * (int)ii - g.vpadding;
+            const int x_y = g.hstride * (int)xx + g.hdilation * (int)jj - g.hpadding;
+            const bool ok = e < count && (unsigned)x_x < (unsigned)g.h && (unsigned)x_y < (unsigned)g.w;
+            const float val = x[ok ? ((nn * g.h + x_x) * g.w + x_y) * g.c + cc : 0u];
+            v[u] = ok ? val : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const uint32_t e = e0 + u * kThreads;
+            if (e < count) dst[e] = v[u];
+        }
     }
 }
 
