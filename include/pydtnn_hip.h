@@ -188,6 +188,25 @@ int pydtnn_hip_max_pool_2d_bwd_nchw(const float *dy, const int32_t *idx_max, flo
                                     int kh, int kw, int vpadding, int hpadding, int vstride, int hstride,
                                     int vdilation, int hdilation, void *stream);
 
+/* BatchNormalization in training mode (pydtnn/backends/cpu/layers/batch_normalization_cpu.py:59-82 and
+ * :108-129; dx as pydtnn/cython_modules/bn_training_cython.pyx:236-243).  Tensors are viewed as
+ * (outer, channels, inner): NCHW = (N, C, H*W); NHWC and 2-D = (rows, C, 1).  With n = outer * inner:
+ *   forward : mu = mean(x); var = mean((x - mu)^2); std = sqrt(var + eps); xn = (x - mu) / std;
+ *             y = gamma * xn + beta; running_mean = momentum * running_mean + (1 - momentum) * mu,
+ *             running_var likewise with var.  Outputs y, xn (x-shaped) and std (channels).
+ *   backward: dgamma = sum(dy * xn); dbeta = sum(dy);
+ *             dx = (gamma / (std * n)) * (n * dy - xn * dgamma - dbeta)   (skipped when dx is NULL).
+ * Per-channel sums are taken in a fixed order (reproducible run to run).
+ * Workspace: pydtnn_hip_bn_training_workspace_bytes(channels). */
+size_t pydtnn_hip_bn_training_workspace_bytes(int channels);
+int pydtnn_hip_bn_training_fwd(const float *x, float *y, float *xn, float *std_out, const float *gamma,
+                               const float *beta, float *running_mean, float *running_var, double momentum, double eps,
+                               long outer, int channels, int inner, void *workspace, size_t workspace_bytes,
+                               void *stream);
+int pydtnn_hip_bn_training_bwd(const float *dy, const float *xn, const float *std_in, const float *gamma,
+                               float *dgamma, float *dbeta, float *dx, long outer, int channels, int inner,
+                               void *workspace, size_t workspace_bytes, void *stream);
+
 /* Softmax over the rows of a (rows, cols) matrix and its backward
  * (pydtnn/backends/cpu/activations/softmax_cpu.py:32-39):
  *   y = exp(x - max(x, axis=1)) / sum(...);   dx = y * (dy - sum(dy * y, axis=1)). */

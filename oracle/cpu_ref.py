@@ -146,6 +146,54 @@ def bn_inference_nchw(x, running_mean, inv_std, gamma, beta):
     return y
 
 
+def bn_training_forward(x, gamma, beta, running_mean, running_var, momentum=0.9, eps=1e-5, tensor_format="NHWC"):
+    """TRAIN_MODE branch of pydtnn/backends/cpu/layers/batch_normalization_cpu.py:53-82 (sync_stats off).
+    x is 2-D (rows, C) or 4-D in ``tensor_format``; the reference moves NCHW to NHWC
+    (best_transpose_0231, :54-56), flattens to (rows, C), and restores the format at the end (:101-104).
+    Returns (y, xn_2d, std, new_running_mean, new_running_var)."""
+    shape = x.shape
+    if x.ndim == 4 and tensor_format == "NCHW":
+        x = x.transpose(0, 2, 3, 1)
+    c = x.shape[-1]
+    x2 = np.ascontiguousarray(x).reshape(-1, c)
+    mu = np.mean(x2, axis=0)
+    xc = (x2 - mu)
+    var = np.mean(xc ** 2, axis=0)
+    std = np.sqrt(var + eps)
+    xn = xc / std
+    y = gamma * xn + beta
+    new_mean = momentum * running_mean + (1.0 - momentum) * mu
+    new_var = momentum * running_var + (1.0 - momentum) * var
+    if len(shape) == 4:
+        y = y.reshape(x.shape)
+        if tensor_format == "NCHW":
+            y = np.ascontiguousarray(y.transpose(0, 3, 1, 2))
+    return y, xn, std, new_mean, new_var
+
+
+def bn_training_backward(dy, xn, std, gamma, tensor_format="NHWC", need_dx=True):
+    """pydtnn/backends/cpu/layers/batch_normalization_cpu.py:108-129 with the dx formula of
+    pydtnn/cython_modules/bn_training_cython.pyx:236-243.  xn is the (rows, C) matrix kept by the forward
+    pass.  Returns (dgamma, dbeta, dx in the format of dy or None)."""
+    shape = dy.shape
+    if dy.ndim == 4 and tensor_format == "NCHW":
+        dy = dy.transpose(0, 2, 3, 1)
+    c = dy.shape[-1]
+    dy2 = np.ascontiguousarray(dy).reshape(-1, c)
+    n = dy2.shape[0]
+    dgamma = np.sum(dy2 * xn, axis=0)
+    dbeta = np.sum(dy2, axis=0)
+    dx = None
+    if need_dx:
+        nf = dy2.dtype.type(n)
+        dx = (gamma / (std * nf)) * (nf * dy2 - xn * dgamma - dbeta)
+        if len(shape) == 4:
+            dx = dx.reshape(dy.shape)
+            if tensor_format == "NCHW":
+                dx = np.ascontiguousarray(dx.transpose(0, 3, 1, 2))
+    return dgamma, dbeta, dx
+
+
 def relu(x):
     """pydtnn/cython_modules/relu_cython.pyx:25-39 -> (max(x,0), int8 mask)"""
     x = np.ascontiguousarray(x)

@@ -14,6 +14,11 @@ size_t bias_grad_workspace_floats(long, int);
 int launch_bias_grad(const float*, float*, long, int, int, float*, hipStream_t);
 int launch_splitk_reduce(const float*, float*, long, int, long, int, int, int, const ChanEpilogue&, hipStream_t);
 int launch_flip_filter(const float*, float*, int, int, int, int, int, hipStream_t);
+size_t bn_training_workspace_floats(int);
+int launch_bn_training_fwd(const float*, float*, float*, float*, const float*, const float*, float*, float*, float, float,
+                           float, long, int, int, float*, hipStream_t);
+int launch_bn_training_bwd(const float*, const float*, const float*, const float*, float*, float*, float*, long, int,
+                           int, float*, hipStream_t);
 int launch_softmax_fwd(const float*, float*, int, int, hipStream_t);
 int launch_softmax_bwd(const float*, const float*, float*, int, int, hipStream_t);
 int launch_cce(const float*, const float*, float*, float*, float*, int, int, float, float, float, hipStream_t);
@@ -678,6 +683,37 @@ int pydtnn_hip_max_pool_2d_bwd_nchw(const float* dy, const int32_t* idx_max, flo
     const int kn = 1;
     const int rc = geom_from_args(&g, GEOM_ARGS);
     return rc != PYDTNN_HIP_OK ? rc : launch_max_pool_bwd_nchw(dy, idx_max, dx, g, as_stream(stream));
+}
+
+size_t pydtnn_hip_bn_training_workspace_bytes(int channels)
+{
+    return channels > 0 ? bn_training_workspace_floats(channels) * 4 : 0;
+}
+
+int pydtnn_hip_bn_training_fwd(const float* x, float* y, float* xn, float* std_out, const float* gamma,
+                               const float* beta, float* running_mean, float* running_var, double momentum, double eps,
+                               long outer, int channels, int inner, void* workspace, size_t workspace_bytes,
+                               void* stream)
+{
+    if (!x || !y || !xn || !std_out || !gamma || !beta || !running_mean || !running_var)
+        return PYDTNN_HIP_ERR_INVALID;
+    if (!workspace || workspace_bytes < pydtnn_hip_bn_training_workspace_bytes(channels))
+        return PYDTNN_HIP_ERR_WORKSPACE;
+    // NumPy multiplies float32 arrays by the Python floats momentum and (1.0 - momentum) rounded to float32
+    return launch_bn_training_fwd(x, y, xn, std_out, gamma, beta, running_mean, running_var, (float)momentum,
+                                  (float)(1.0 - momentum), (float)eps, outer, channels, inner, (float*)workspace,
+                                  as_stream(stream));
+}
+
+int pydtnn_hip_bn_training_bwd(const float* dy, const float* xn, const float* std_in, const float* gamma,
+                               float* dgamma, float* dbeta, float* dx, long outer, int channels, int inner,
+                               void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (!dy || !xn || !std_in || !gamma || !dgamma || !dbeta) return PYDTNN_HIP_ERR_INVALID;
+    if (!workspace || workspace_bytes < pydtnn_hip_bn_training_workspace_bytes(channels))
+        return PYDTNN_HIP_ERR_WORKSPACE;
+    return launch_bn_training_bwd(dy, xn, std_in, gamma, dgamma, dbeta, dx, outer, channels, inner, (float*)workspace,
+                                  as_stream(stream));
 }
 
 int pydtnn_hip_softmax_fwd(const float* x, float* y, int rows, int cols, void* stream)

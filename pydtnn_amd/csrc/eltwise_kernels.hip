@@ -328,6 +328,165 @@ __global__ void __launch_bounds__(kThreads) sgd_momentum_kernel(float* __restric
     velocity[idx] = v;
 }
 
+// ---------------------------------------------------------------- BatchNormalization, training
+// pydtnn/backends/cpu/layers/batch_normalization_cpu.py:59-82 (forward) and :108-129 (backward), on
+// tensors viewed as (outer, channels, inner): NCHW is (N, C, H*W), NHWC and 2-D inputs are
+// (rows, C, 1), so no transposed copy is made.  Per-channel sums are taken in two deterministic
+// stages (slices of the outer axis, then a sum over slices in ascending order).
+// What is summed: MODE 0  a = x
+//                 MODE 1  a = (x - p0[ch])^2
+//                 MODE 2  a = x, b = x * q          (x = dy, q = xn)
+template <int MODE>
+__device__ __forceinline__ void bn_term(float x, float q, float p0, float* a, float* b)
+{
+    if (MODE == 0) {
+        *a += x;
+    } else if (MODE == 1) {
+        const float d = x - p0;
+        *a += d * d;
+    } else {
+        *a += x;
+        *b += x * q;
+    }
+}
+
+// NCHW: grid (C, S); slice s covers images [s*per, (s+1)*per).  partial[(which*slices + s)*c + ch]
+template <int MODE>
+__global__ void __launch_bounds__(kThreads) bn_reduce_nchw_stage1(const float* __restrict__ x,
+                                                                 const float* __restrict__ q,
+                                                                 const float* __restrict__ p0,
+                                                                 float* __restrict__ partial, int n, int c, int hw,
+                                                                 int per, int slices)
+{
+    __shared__ float red[2][kThreads / 64];
+    const int ch = blockIdx.x, s = blockIdx.y;
+    const int n0 = s * per, n1 = min(n, n0 + per);
+    const float shift = MODE == 1 ? p0[ch] : 0.0f;
+    float a = 0.0f, b = 0.0f;
+    for (int nn = n0; nn < n1; ++nn) {
+        const long base = ((long)nn * c + ch) * hw;
+        for (int i = threadIdx.x; i < hw; i += kThreads)
+            bn_term<MODE>(x[base + i], MODE == 2 ? q[base + i] : 0.0f, shift, &a, &b);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        a += __shfl_down(a, off, 64);
+        b += __shfl_down(b, off, 64);
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) { red[0][wave] = a; red[1][wave] = b; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float sa = 0.0f, sb = 0.0f;
+        for (int i = 0; i < kThreads / 64; ++i) { sa += red[0][i]; sb += red[1][i]; }
+        partial[(long)s * c + ch] = sa;
+        if (MODE == 2) partial[((long)slices + s) * c + ch] = sb;
+    }
+}
+
+// (rows, C): grid (S, ceil(C/64)); block = 64 channels x 4 row lanes.
+template <int MODE>
+__global__ void __launch_bounds__(kThreads) bn_reduce_rows_stage1(const float* __restrict__ x,
+                                                                 const float* __restrict__ q,
+                                                                 const float* __restrict__ p0,
+                                                                 float* __restrict__ partial, long rows, int c,
+                                                                 long per, int slices)
+{
+    __shared__ float red[2][4][64];
+    const int cl = threadIdx.x & 63, rl = threadIdx.x >> 6;
+    const int ch = blockIdx.y * 64 + cl;
+    const long r0 = (long)blockIdx.x * per;
+    const long r1 = r0 + per < rows ? r0 + per : rows;
+    float a = 0.0f, b = 0.0f;
+    if (ch < c) {
+        const float shift = MODE == 1 ? p0[ch] : 0.0f;
+        for (long r = r0 + rl; r < r1; r += 4)
+            bn_term<MODE>(x[r * c + ch], MODE == 2 ? q[r * c + ch] : 0.0f, shift, &a, &b);
+    }
+    red[0][rl][cl] = a;
+    red[1][rl][cl] = b;
+    __syncthreads();
+    if (rl == 0 && ch < c) {
+        partial[(long)blockIdx.x * c + ch] = (red[0][0][cl] + red[0][1][cl]) + (red[0][2][cl] + red[0][3][cl]);
+        if (MODE == 2)
+            partial[((long)slices + blockIdx.x) * c + ch] =
+                (red[1][0][cl] + red[1][1][cl]) + (red[1][2][cl] + red[1][3][cl]);
+    }
+}
+
+// Second stage of the forward statistics.  PASS 0: mu = sum / count.  PASS 1: var = sum / count,
+// std = sqrt(var + eps), running statistics updated as momentum*running + (1-momentum)*new.
+template <int PASS>
+__global__ void __launch_bounds__(kThreads) bn_stats_stage2(const float* __restrict__ partial, int c, int slices,
+                                                           float count, float* __restrict__ mu,
+                                                           float* __restrict__ std_out, float eps,
+                                                           float* __restrict__ running_mean,
+                                                           float* __restrict__ running_var, float momentum,
+                                                           float one_minus_momentum)
+{
+    const int ch = blockIdx.x * kThreads + threadIdx.x;
+    if (ch >= c) return;
+    float acc = 0.0f;
+    for (int s = 0; s < slices; ++s) acc += partial[(long)s * c + ch];
+    const float mean = acc / count;
+    if (PASS == 0) {
+        mu[ch] = mean;
+    } else {
+        std_out[ch] = sqrtf(mean + eps);
+        running_mean[ch] = __fadd_rn(__fmul_rn(momentum, running_mean[ch]), __fmul_rn(one_minus_momentum, mu[ch]));
+        running_var[ch] = __fadd_rn(__fmul_rn(momentum, running_var[ch]), __fmul_rn(one_minus_momentum, mean));
+    }
+}
+
+// Second stage of the backward sums: dbeta = sum dy, dgamma = sum dy*xn.
+__global__ void __launch_bounds__(kThreads) bn_grads_stage2(const float* __restrict__ partial, int c, int slices,
+                                                           float* __restrict__ dgamma, float* __restrict__ dbeta)
+{
+    const int ch = blockIdx.x * kThreads + threadIdx.x;
+    if (ch >= c) return;
+    float a = 0.0f, b = 0.0f;
+    for (int s = 0; s < slices; ++s) {
+        a += partial[(long)s * c + ch];
+        b += partial[((long)slices + s) * c + ch];
+    }
+    dbeta[ch] = a;
+    dgamma[ch] = b;
+}
+
+// xn = (x - mu) / std;  y = gamma * xn + beta   (two roundings in the last step, as NumPy evaluates it)
+__global__ void __launch_bounds__(kThreads) bn_train_apply_kernel(const float* __restrict__ x,
+                                                                 float* __restrict__ y, float* __restrict__ xn,
+                                                                 long total, int inner, int channels,
+                                                                 const float* __restrict__ mu,
+                                                                 const float* __restrict__ std_in,
+                                                                 const float* __restrict__ gamma,
+                                                                 const float* __restrict__ beta)
+{
+    const long idx = (long)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= total) return;
+    const int ch = (int)((idx / inner) % channels);
+    const float v = (x[idx] - mu[ch]) / std_in[ch];
+    xn[idx] = v;
+    y[idx] = __fadd_rn(__fmul_rn(gamma[ch], v), beta[ch]);
+}
+
+// dx = (gamma / (std * n)) * (n * dy - xn * dgamma - dbeta)   (bn_training_cython.pyx:236-243)
+__global__ void __launch_bounds__(kThreads) bn_train_bwd_kernel(const float* __restrict__ dy,
+                                                               const float* __restrict__ xn,
+                                                               float* __restrict__ dx, long total, int inner,
+                                                               int channels, float n,
+                                                               const float* __restrict__ std_in,
+                                                               const float* __restrict__ gamma,
+                                                               const float* __restrict__ dgamma,
+                                                               const float* __restrict__ dbeta)
+{
+    const long idx = (long)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= total) return;
+    const int ch = (int)((idx / inner) % channels);
+    const float scale = gamma[ch] / (std_in[ch] * n);
+    dx[idx] = scale * (n * dy[idx] - xn[idx] * dgamma[ch] - dbeta[ch]);
+}
+
 // ---------------------------------------------------------------- softmax and categorical cross-entropy
 // Rows of a (rows, cols) matrix, one workgroup per row.
 template <class Op>
@@ -603,5 +762,86 @@ int launch_cce(const float* y_pred, const float* y_targ, float* dx, float* loss,
     HIP_RETURN_IF_LAUNCH_FAILED();
     hipLaunchKernelGGL(cce_loss_kernel, dim3(1), dim3(64), 0, stream, row_loss, loss, rows);
     HIP_RETURN_IF_LAUNCH_FAILED();
+    return PYDTNN_HIP_OK;
+}
+
+// Slices of the outer axis for a two-stage channel reduction; at most 64.
+static int bn_slices(long outer, int inner, long* per)
+{
+    long slices;
+    if (inner > 1) {
+        slices = outer < 64 ? outer : 64;
+    } else {
+        slices = outer < 64 * 4 ? (outer + 3) / 4 : 64;
+    }
+    *per = (outer + slices - 1) / slices;
+    return (int)((outer + *per - 1) / *per);
+}
+
+template <int MODE>
+static void bn_reduce_stage1(const float* x, const float* q, const float* p0, float* partial, long outer, int channels,
+                             int inner, hipStream_t stream, int* slices_out)
+{
+    long per;
+    const int slices = bn_slices(outer, inner, &per);
+    if (inner > 1)
+        hipLaunchKernelGGL(bn_reduce_nchw_stage1<MODE>, dim3(channels, slices), dim3(kThreads), 0, stream, x, q, p0,
+                           partial, (int)outer, channels, inner, (int)per, slices);
+    else
+        hipLaunchKernelGGL(bn_reduce_rows_stage1<MODE>, dim3(slices, (channels + 63) / 64), dim3(kThreads), 0, stream,
+                           x, q, p0, partial, outer, channels, per, slices);
+    *slices_out = slices;
+}
+
+// floats: two sets of 64 partial sums per channel, then mu
+size_t bn_training_workspace_floats(int channels) { return (size_t)(2 * 64 + 1) * channels; }
+
+// Algorithmic bytes: x read three times (mean, variance, normalise), y and xn written: 20 bytes per element.
+int launch_bn_training_fwd(const float* x, float* y, float* xn, float* std_out, const float* gamma, const float* beta,
+                           float* running_mean, float* running_var, float momentum, float one_minus_momentum, float eps,
+                           long outer, int channels, int inner, float* workspace, hipStream_t stream)
+{
+    if (outer <= 0 || channels <= 0 || inner <= 0) return PYDTNN_HIP_ERR_INVALID;
+    if (inner > 1 && outer >= (1l << 31)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+    float* partial = workspace;
+    float* mu = workspace + (size_t)2 * 64 * channels;
+    const float count = (float)(outer * inner);
+    const long total = outer * channels * inner;
+    int slices = 0;
+    bn_reduce_stage1<0>(x, nullptr, nullptr, partial, outer, channels, inner, stream, &slices);
+    HIP_RETURN_IF_LAUNCH_FAILED();
+    hipLaunchKernelGGL(bn_stats_stage2<0>, dim3(blocks_for(channels)), dim3(kThreads), 0, stream, partial, channels,
+                       slices, count, mu, std_out, eps, running_mean, running_var, momentum, one_minus_momentum);
+    HIP_RETURN_IF_LAUNCH_FAILED();
+    bn_reduce_stage1<1>(x, nullptr, mu, partial, outer, channels, inner, stream, &slices);
+    HIP_RETURN_IF_LAUNCH_FAILED();
+    hipLaunchKernelGGL(bn_stats_stage2<1>, dim3(blocks_for(channels)), dim3(kThreads), 0, stream, partial, channels,
+                       slices, count, mu, std_out, eps, running_mean, running_var, momentum, one_minus_momentum);
+    HIP_RETURN_IF_LAUNCH_FAILED();
+    hipLaunchKernelGGL(bn_train_apply_kernel, dim3(blocks_for(total)), dim3(kThreads), 0, stream, x, y, xn, total,
+                       inner, channels, mu, std_out, gamma, beta);
+    HIP_RETURN_IF_LAUNCH_FAILED();
+    return PYDTNN_HIP_OK;
+}
+
+// Algorithmic bytes: dy and xn read twice, dx written: 20 bytes per element (16 without dx).
+int launch_bn_training_bwd(const float* dy, const float* xn, const float* std_in, const float* gamma, float* dgamma,
+                           float* dbeta, float* dx, long outer, int channels, int inner, float* workspace,
+                           hipStream_t stream)
+{
+    if (outer <= 0 || channels <= 0 || inner <= 0) return PYDTNN_HIP_ERR_INVALID;
+    if (inner > 1 && outer >= (1l << 31)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+    const long total = outer * channels * inner;
+    int slices = 0;
+    bn_reduce_stage1<2>(dy, xn, nullptr, workspace, outer, channels, inner, stream, &slices);
+    HIP_RETURN_IF_LAUNCH_FAILED();
+    hipLaunchKernelGGL(bn_grads_stage2, dim3(blocks_for(channels)), dim3(kThreads), 0, stream, workspace, channels,
+                       slices, dgamma, dbeta);
+    HIP_RETURN_IF_LAUNCH_FAILED();
+    if (dx) {
+        hipLaunchKernelGGL(bn_train_bwd_kernel, dim3(blocks_for(total)), dim3(kThreads), 0, stream, dy, xn, dx, total,
+                           inner, channels, (float)(outer * inner), std_in, gamma, dgamma, dbeta);
+        HIP_RETURN_IF_LAUNCH_FAILED();
+    }
     return PYDTNN_HIP_OK;
 }

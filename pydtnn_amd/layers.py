@@ -471,8 +471,8 @@ class Dropout(Layer):
 # --------------------------------------------------------------------------- BatchNormalization (inference)
 class BatchNormalization(Layer):
     """pydtnn/layers/batch_normalization.py:26-62 + the EVALUATE_MODE branch of
-    pydtnn/backends/cpu/layers/batch_normalization_cpu.py:50-52, :84-106.  Training statistics are outside
-    the conv-as-GEMM path and raise."""
+    pydtnn/backends/cpu/layers/batch_normalization_cpu.py:40-129.  ``xn`` is kept in the model's tensor
+    format (the reference keeps it as a (rows, channels) matrix); ``std`` is per channel."""
 
     def __init__(self, beta=0.0, gamma=1.0, momentum=0.9, epsilon=1e-5,
                  moving_mean_initializer="zeros", moving_variance_initializer="zeros", sync_stats=False):
@@ -517,15 +517,31 @@ class BatchNormalization(Layer):
             return ops.bn_inference_nchw(x, *bn, relu=relu)
         return ops.chan_eltwise(x, channels=x.shape[-1], inner=1, bn=bn, relu=relu)
 
+    def _view(self, t):
+        """(channels, inner) of the (outer, channels, inner) view of an activation tensor."""
+        if self.spatial and self.model.tensor_format == PYDTNN_TENSOR_FORMAT_NCHW:
+            return t.shape[1], t.shape[2] * t.shape[3]
+        return t.shape[-1], 1
+
     def forward(self, x):
         if self.model.mode == TRAIN_MODE:
-            raise NotImplementedError("BatchNormalization training is not part of the conv-as-GEMM path")
+            if self.sync_stats:
+                raise NotImplementedError("sync_stats needs more than one process")
+            channels, inner = self._view(x)
+            y, self.xn, self.std = ops.bn_training_forward(x, self.gamma, self.beta, self.running_mean,
+                                                           self.running_var, self.momentum, self.epsilon,
+                                                           channels, inner)
+            self.updated_running_var = True
+            return y
         if self.model.mode != EVALUATE_MODE:
             raise ValueError("Unexpected model mode")
         return self._apply(x, relu=False)
 
     def backward(self, dy):
-        raise NotImplementedError("BatchNormalization training is not part of the conv-as-GEMM path")
+        channels, inner = self._view(dy)
+        self.dgamma, self.dbeta, dx = ops.bn_training_backward(dy, self.xn, self.std, self.gamma, channels, inner,
+                                                               need_dx=self.need_dx)
+        return dx
 
 
 class _FromParents:

@@ -8,6 +8,7 @@ Kept from the reference: keyword flags readable as attributes (``tensor_format``
 (pydtnn/model.py:450-492, :623-644).  Datasets, MPI, checkpoints, schedulers and the CLI are not
 part of this build.
 """
+import numpy as np
 import torch
 
 from . import layers as L
@@ -179,6 +180,43 @@ class Model:
         if not self._fused:
             self.apply_layer_fusion()
         return self.evaluate_batch(x)
+
+
+    # ------------------------------------------------------------------ weights on disk (pydtnn/model.py:351-387)
+    def load_store_path(self, layers, d, mode):
+        """Walks the layers (and the paths of block layers) and moves every trainable tensor, plus the
+        running statistics of BatchNormalization, between the layers and the dictionary ``d`` under
+        the reference's key ``"{layer.id}_{canonical_name}_{variable}"``.  Arrays keep the in-memory
+        layout of the model's tensor format, as in the reference."""
+        for layer in layers:
+            name = layer.canonical_name
+            if name in ["AdditionBlock", "ConcatenationBlock"]:
+                for path in layer.paths:
+                    self.load_store_path(path, d, mode)
+                continue
+            keys = [g for g in layer.grad_vars] + \
+                   (["running_var", "running_mean"] if name == "BatchNormalization" else [])
+            if name == "BatchNormalization":
+                layer.updated_running_var = True
+            for key in keys:
+                base = f"{layer.id}_{name}_{key}"
+                if mode == "load":
+                    if base not in d:
+                        print(f"Could not find '{base}' for layer '{name}' in file!")
+                        continue
+                    ary = np.ascontiguousarray(d[base], dtype=np.float32)
+                    setattr(layer, key, torch.from_numpy(ary).cuda())
+                elif mode == "store":
+                    d[base] = getattr(layer, key).detach().cpu().numpy()
+
+    def load_weights_and_bias(self, filename):
+        d = np.load(filename)
+        self.load_store_path(self.layers, d, "load")
+
+    def store_weights_and_bias(self, filename):
+        d = {}
+        self.load_store_path(self.layers, d, "store")
+        np.savez_compressed(filename, **d)
 
 
 # --------------------------------------------------------------------------- loss and optimizer

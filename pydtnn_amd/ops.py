@@ -207,6 +207,35 @@ def max_pool_2d_bwd_nchw(dy, idx_max, n, c, h, w, kh, kw, vpadding, hpadding, vs
     return dx
 
 
+def bn_training_forward(x, gamma, beta, running_mean, running_var, momentum, eps, channels, inner):
+    """pydtnn/backends/cpu/layers/batch_normalization_cpu.py:59-82 on x viewed as (outer, channels, inner).
+    Updates running_mean / running_var in place; returns (y, xn, std)."""
+    _need_f32(x, gamma, beta, running_mean, running_var)
+    x = x.contiguous()
+    outer = x.numel() // (channels * inner)
+    y, xn = torch.empty_like(x), torch.empty_like(x)
+    std = torch.empty((channels,), dtype=x.dtype, device=x.device)
+    ws, ws_bytes = native.workspace(lib().pydtnn_hip_bn_training_workspace_bytes(channels))
+    check(lib().pydtnn_hip_bn_training_fwd(f32(x), f32(y), f32(xn), f32(std), f32(gamma), f32(beta), f32(running_mean),
+                                           f32(running_var), float(momentum), float(eps), outer, channels, inner, ws,
+                                           ws_bytes, stream_ptr()), "bn_training_fwd")
+    return y, xn, std
+
+
+def bn_training_backward(dy, xn, std, gamma, channels, inner, need_dx=True):
+    """batch_normalization_cpu.py:108-129 -> (dgamma, dbeta, dx or None)"""
+    _need_f32(dy, xn, std, gamma)
+    dy = dy.contiguous()
+    outer = dy.numel() // (channels * inner)
+    dgamma = torch.empty((channels,), dtype=dy.dtype, device=dy.device)
+    dbeta = torch.empty_like(dgamma)
+    dx = torch.empty_like(dy) if need_dx else None
+    ws, ws_bytes = native.workspace(lib().pydtnn_hip_bn_training_workspace_bytes(channels))
+    check(lib().pydtnn_hip_bn_training_bwd(f32(dy), f32(xn), f32(std), f32(gamma), f32(dgamma), f32(dbeta), f32(dx),
+                                           outer, channels, inner, ws, ws_bytes, stream_ptr()), "bn_training_bwd")
+    return dgamma, dbeta, dx
+
+
 def softmax(x):
     """pydtnn/backends/cpu/activations/softmax_cpu.py:32-35 on a (batch, classes) matrix."""
     _need_f32(x)

@@ -368,6 +368,40 @@ def test_sgd_momentum(ops, oracle):
     assert_close(host(vd), v_ref, tol=1e-6, what="sgd v")
 
 
+@pytest.mark.parametrize("fmt,shape", [("NCHW", (8, 6, 5, 7)), ("NCHW", (70, 3, 4, 4)), ("NHWC", (8, 5, 7, 6)),
+                                       ("NHWC", (3, 9, 9, 130)), ("2D", (64, 10)), ("2D", (300, 70)), ("2D", (2, 3))])
+def test_bn_training_forward_backward(ops, oracle, fmt, shape):
+    announce("bn training", (fmt, shape))
+    rng = np.random.default_rng(sum(shape))
+    c = shape[1] if fmt == "NCHW" else shape[-1]
+    inner = shape[2] * shape[3] if fmt == "NCHW" else 1
+    x = (rng.standard_normal(shape) * 2 + 1).astype(np.float32)
+    dy = rng.standard_normal(shape).astype(np.float32)
+    gamma, beta = rng.uniform(0.5, 1.5, c).astype(np.float32), rng.standard_normal(c).astype(np.float32)
+    rm, rv = rng.standard_normal(c).astype(np.float32), rng.uniform(0.5, 2, c).astype(np.float32)
+    y_ref, xn_ref, std_ref, rm_ref, rv_ref = oracle.bn_training_forward(x, gamma, beta, rm, rv, 0.9, 1e-5,
+                                                                        tensor_format=fmt)
+    rmd, rvd = dev(rm), dev(rv)
+    y, xn, std = ops.bn_training_forward(dev(x), dev(gamma), dev(beta), rmd, rvd, 0.9, 1e-5, c, inner)
+    assert_close(host(y), y_ref, tol=1e-5, what="bn y")
+    assert_close(host(std), std_ref, tol=1e-5, what="bn std")
+    assert_close(host(rmd), rm_ref, tol=1e-5, what="bn running mean")
+    assert_close(host(rvd), rv_ref, tol=1e-5, what="bn running var")
+    xn_in_format = host(xn).transpose(0, 2, 3, 1).reshape(-1, c) if fmt == "NCHW" else host(xn).reshape(-1, c)
+    assert_close(xn_in_format, xn_ref, tol=1e-5, what="bn xn")
+    # backward from the oracle's own xn / std so that only this kernel's arithmetic is compared
+    xn_dev = xn_ref.reshape((shape[0], shape[2], shape[3], c)).transpose(0, 3, 1, 2) if fmt == "NCHW" \
+        else xn_ref.reshape(shape)
+    dgamma_ref, dbeta_ref, dx_ref = oracle.bn_training_backward(dy, xn_ref, std_ref, gamma, tensor_format=fmt)
+    dgamma, dbeta, dx = ops.bn_training_backward(dev(dy), dev(np.ascontiguousarray(xn_dev)), dev(std_ref),
+                                                 dev(gamma), c, inner)
+    assert_close(host(dgamma), dgamma_ref, tol=1e-5, what="bn dgamma")
+    assert_close(host(dbeta), dbeta_ref, tol=1e-5, what="bn dbeta")
+    assert_close(host(dx), dx_ref, tol=2e-5, what="bn dx")
+    assert ops.bn_training_backward(dev(dy), dev(np.ascontiguousarray(xn_dev)), dev(std_ref), dev(gamma), c, inner,
+                                    need_dx=False)[2] is None
+
+
 @pytest.mark.parametrize("rows,cols", [(64, 1000), (3, 7), (1, 1), (5, 300), (2, 4097)])
 def test_softmax_forward_backward(ops, oracle, rows, cols):
     announce("softmax", (rows, cols))

@@ -330,3 +330,85 @@ def test_small_vgg_training_step_matches_the_oracle_chain(pd, oracle):
             w_new, _ = oracle.sgd_update(w.copy(), dw, np.zeros_like(w), np.float32(0.01), np.float32(0.9))
             assert_close(host(l.weights), w_new, tol=1e-5, what=f"{l} updated weights")
             dcur = dx
+
+
+# ------------------------------------------------------------------ BatchNormalization in training mode
+
+@pytest.mark.parametrize("fmt", ["NCHW", "NHWC"])
+def test_batch_normalization_training_layer(pd, oracle, fmt):
+    """Forward / backward of the layer in TRAIN_MODE against the restated reference branch, then an
+    EVALUATE_MODE forward that must use the running statistics the training step has just updated
+    (pydtnn/backends/cpu/layers/batch_normalization_cpu.py:59-82, :92-96, :108-129)."""
+    announce("bn layer training", fmt)
+    rng = np.random.default_rng(5)
+    n, c, h, w = 6, 10, 7, 9
+    shape = (n, c, h, w) if fmt == "NCHW" else (n, h, w, c)
+    x = (rng.standard_normal(shape) * 3 - 1).astype(np.float32)
+    dy = rng.standard_normal(shape).astype(np.float32)
+    model = pd.Model(tensor_format=fmt, batch_size=n)
+    model.mode = pd.TRAIN_MODE
+    bn = pd.BatchNormalization(moving_variance_initializer="ones")
+    bn.set_model(model)
+    bn.initialize(prev_shape=shape[1:])
+    bn.gamma = dev(rng.uniform(0.5, 1.5, c).astype(np.float32))
+    bn.beta = dev(rng.standard_normal(c).astype(np.float32))
+    gamma, beta = host(bn.gamma), host(bn.beta)
+    rm0, rv0 = host(bn.running_mean).copy(), host(bn.running_var).copy()
+    y = bn.forward(dev(x))
+    dx = bn.backward(dev(dy))
+    y_ref, xn_ref, std_ref, rm_ref, rv_ref = oracle.bn_training_forward(x, gamma, beta, rm0, rv0, bn.momentum,
+                                                                        bn.epsilon, tensor_format=fmt)
+    dgamma_ref, dbeta_ref, dx_ref = oracle.bn_training_backward(dy, xn_ref, std_ref, gamma, tensor_format=fmt)
+    assert_close(host(y), y_ref, tol=1e-5, what="y")
+    assert_close(host(dx), dx_ref, tol=5e-5, what="dx")
+    assert_close(host(bn.dgamma), dgamma_ref, tol=1e-5, what="dgamma")
+    assert_close(host(bn.dbeta), dbeta_ref, tol=1e-5, what="dbeta")
+    assert_close(host(bn.running_mean), rm_ref, tol=1e-5, what="running mean")
+    assert_close(host(bn.running_var), rv_ref, tol=1e-5, what="running var")
+    model.mode = pd.EVALUATE_MODE
+    y_eval = bn.forward(dev(x))
+    inv_std = (1.0 / np.sqrt(rv_ref + np.float32(bn.epsilon))).astype(np.float32)
+    if fmt == "NCHW":
+        ref = oracle.bn_inference_nchw(x, rm_ref.astype(np.float32), inv_std, gamma, beta)
+    else:
+        ref = oracle.bn_inference(x.reshape(-1, c), rm_ref.astype(np.float32), inv_std, gamma, beta).reshape(shape)
+    assert_close(host(y_eval), ref, tol=1e-5, what="y in evaluate mode")
+
+
+def test_store_and_load_weights_use_the_reference_key_names(pd, tmp_path):
+    """pydtnn/model.py:351-387: ``{id}_{Name}_{variable}`` keys, BatchNormalization adds its running statistics."""
+    announce("weights file")
+    def build():
+        model = pd.Model(tensor_format="NHWC", batch_size=2)
+        model.add(pd.Input(shape=(8, 8, 3)))
+        model.add(pd.Conv2D(nfilters=4, filter_shape=(3, 3), padding=1))
+        model.add(pd.BatchNormalization())
+        model.add(pd.Relu())
+        model.add(pd.AdditionBlock([pd.Conv2D(nfilters=4, filter_shape=(1, 1))], []))
+        model.add(pd.Flatten())
+        model.add(pd.FC(shape=(5,)))
+        return model
+    np.random.seed(1)
+    a = build()
+    a.layers[2].running_mean = dev(np.arange(4, dtype=np.float32))
+    path = str(tmp_path / "weights.npz")
+    a.store_weights_and_bias(path)
+    stored = np.load(path)
+    names = sorted(stored.files)
+    convs = [l for l in a.get_all_layers() if l.canonical_name == "Conv2D"]
+    bn = a.layers[2]
+    assert f"{convs[0].id}_Conv2D_weights" in names and f"{convs[0].id}_Conv2D_biases" in names
+    assert f"{convs[1].id}_Conv2D_weights" in names                      # inside the AdditionBlock's path
+    for key in ("beta", "gamma", "running_mean", "running_var"):
+        assert f"{bn.id}_BatchNormalization_{key}" in names
+    assert stored[f"{convs[0].id}_Conv2D_weights"].shape == (3, 3, 3, 4)  # NHWC layout (ci, kh, kw, co) as in memory
+    np.random.seed(2)
+    b = build()
+    assert not np.array_equal(host(b.layers[1].weights), host(a.layers[1].weights))
+    b.load_weights_and_bias(path)
+    for la, lb in zip(a.get_all_layers(), b.get_all_layers()):
+        for key in list(la.grad_vars) + (["running_mean", "running_var"] if la.canonical_name == "BatchNormalization" else []):
+            assert np.array_equal(host(getattr(la, key)), host(getattr(lb, key))), (la, key)
+    assert b.layers[2].updated_running_var
+    x = dev(np.random.default_rng(0).standard_normal((2, 8, 8, 3)).astype(np.float32))
+    assert np.array_equal(host(a.evaluate_batch(x)), host(b.evaluate_batch(x)))

@@ -357,6 +357,41 @@ def test_fc_against_torch_autograd(oracle):
     np.testing.assert_allclose(dx, xt.grad.numpy(), rtol=1e-12, atol=1e-12)
 
 
+@pytest.mark.parametrize("fmt", ["NCHW", "NHWC", "2D"])
+def test_bn_training_against_torch_batch_norm_and_autograd(oracle, fmt):
+    """Pins the TRAIN_MODE restatement with an independent library in fp64: torch's batch_norm in training
+    mode uses the same biased variance for normalisation (its running_var is the unbiased one, so the running
+    variance is checked against the closed form instead) and autograd supplies dx, dgamma, dbeta."""
+    rng = np.random.default_rng(21)
+    c = 5
+    shape = {"NCHW": (4, c, 3, 6), "NHWC": (4, 3, 6, c), "2D": (9, c)}[fmt]
+    x = rng.standard_normal(shape) * 2 + 1
+    dy = rng.standard_normal(shape)
+    gamma, beta = rng.uniform(0.5, 1.5, c), rng.standard_normal(c)
+    rm, rv = rng.standard_normal(c), rng.uniform(0.5, 2, c)
+    y, xn, std, new_rm, new_rv = oracle.bn_training_forward(x, gamma, beta, rm, rv, 0.9, 1e-5, tensor_format=fmt)
+    to_nc = {"NCHW": lambda a: a, "NHWC": lambda a: a.transpose(0, 3, 1, 2), "2D": lambda a: a}[fmt]
+    from_nc = {"NCHW": lambda a: a, "NHWC": lambda a: a.transpose(0, 2, 3, 1), "2D": lambda a: a}[fmt]
+    xt = torch.from_numpy(np.ascontiguousarray(to_nc(x))).requires_grad_(True)
+    gt, bt = torch.from_numpy(gamma).requires_grad_(True), torch.from_numpy(beta).requires_grad_(True)
+    rmt = torch.from_numpy(rm.copy())
+    yt = F.batch_norm(xt, rmt, torch.from_numpy(rv.copy()), gt, bt, training=True, momentum=0.1, eps=1e-5)
+    np.testing.assert_allclose(y, from_nc(yt.detach().numpy()), rtol=1e-10, atol=1e-10)
+    np.testing.assert_allclose(new_rm, rmt.numpy(), rtol=1e-12)                 # same update rule for the mean
+    x2 = np.ascontiguousarray(from_nc(to_nc(x)) if fmt != "NCHW" else x.transpose(0, 2, 3, 1)).reshape(-1, c)
+    var = ((x2 - x2.mean(0)) ** 2).mean(0)
+    np.testing.assert_allclose(new_rv, 0.9 * rv + 0.1 * var, rtol=1e-12)        # biased variance, closed form
+    np.testing.assert_allclose(std, np.sqrt(var + 1e-5), rtol=1e-12)
+    np.testing.assert_allclose(xn.mean(0), 0, atol=1e-12)
+    np.testing.assert_allclose((xn ** 2).mean(0), var / (var + 1e-5), rtol=1e-10)
+    yt.backward(torch.from_numpy(np.ascontiguousarray(to_nc(dy))))
+    dgamma, dbeta, dx = oracle.bn_training_backward(dy, xn, std, gamma, tensor_format=fmt)
+    np.testing.assert_allclose(dgamma, gt.grad.numpy(), rtol=1e-10, atol=1e-10)
+    np.testing.assert_allclose(dbeta, bt.grad.numpy(), rtol=1e-10, atol=1e-10)
+    np.testing.assert_allclose(dx, from_nc(xt.grad.numpy()), rtol=1e-9, atol=1e-10)
+    assert oracle.bn_training_backward(dy, xn, std, gamma, tensor_format=fmt, need_dx=False)[2] is None
+
+
 def test_softmax_cce_gradient_is_p_minus_t_over_batch(oracle):
     rng = np.random.default_rng(13)
     z = rng.standard_normal((6, 10))
