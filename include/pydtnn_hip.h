@@ -188,6 +188,14 @@ int pydtnn_hip_max_pool_2d_bwd_nchw(const float *dy, const int32_t *idx_max, flo
                                     int kh, int kw, int vpadding, int hpadding, int vstride, int hstride,
                                     int vdilation, int hdilation, void *stream);
 
+/* MaxPool2D, NHWC (pydtnn/cython_modules/max_pool_2d_nhwc_cython.pyx:25-52, :140-166); idx_max is int32 (b,ho,wo,c). */
+int pydtnn_hip_max_pool_2d_fwd_nhwc(const float *x, float *y, int32_t *idx_max, int b, int h, int w, int c, int kh,
+                                    int kw, int vpadding, int hpadding, int vstride, int hstride, int vdilation,
+                                    int hdilation, void *stream);
+int pydtnn_hip_max_pool_2d_bwd_nhwc(const float *dy, const int32_t *idx_max, float *dx, int b, int h, int w, int c,
+                                    int kh, int kw, int vpadding, int hpadding, int vstride, int hstride,
+                                    int vdilation, int hdilation, void *stream);
+
 /* BatchNormalization in training mode (pydtnn/backends/cpu/layers/batch_normalization_cpu.py:59-82 and
  * :108-129; dx as pydtnn/cython_modules/bn_training_cython.pyx:236-243).  Tensors are viewed as
  * (outer, channels, inner): NCHW = (N, C, H*W); NHWC and 2-D = (rows, C, 1).  With n = outer * inner:

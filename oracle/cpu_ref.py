@@ -234,6 +234,29 @@ def max_pool_2d_bwd_nchw(dy, idx_max, n, c, h, w, kh, kw, vpadding, hpadding, vs
     return dx
 
 
+def max_pool_2d_fwd_nhwc(x, kh, kw, vpadding, hpadding, vstride, hstride, vdilation=1, hdilation=1):
+    """pydtnn/cython_modules/max_pool_2d_nhwc_cython.pyx:25-52"""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    n, h, w, c = x.shape
+    hh, ww = out_hw(h, w, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
+    y = np.zeros((n, hh, ww, c), dtype=np.float32)
+    idx = np.zeros((n, hh, ww, c), dtype=np.int32)
+    lib().oracle_max_pool_2d_fwd_nhwc_f32(_p(x), _p(y), _p(idx), n, h, w, c, kh, kw, vpadding, hpadding,
+                                          vstride, hstride, vdilation, hdilation)
+    return y, idx
+
+
+def max_pool_2d_bwd_nhwc(dy, idx_max, n, h, w, c, kh, kw, vpadding, hpadding, vstride, hstride,
+                         vdilation=1, hdilation=1):
+    """pydtnn/cython_modules/max_pool_2d_nhwc_cython.pyx:140-166"""
+    dy = np.ascontiguousarray(dy, dtype=np.float32)
+    idx_max = np.ascontiguousarray(idx_max, dtype=np.int32)
+    dx = np.zeros((n, h, w, c), dtype=np.float32)
+    lib().oracle_max_pool_2d_bwd_nhwc_f32(_p(dy), _p(idx_max), _p(dx), n, h, w, c, kh, kw, vpadding, hpadding,
+                                          vstride, hstride, vdilation, hdilation)
+    return dx
+
+
 # --------------------------------------------------------------------------- conv layers (i2c)
 
 class ConvParams:

@@ -329,3 +329,62 @@ void oracle_max_pool_2d_bwd_nchw_f32(const float *dy, const int32_t *idx_max, fl
                         dx[IDX4(nn, cc, x_x, x_y, c, h, w)] += dy[IDX4(nn, cc, xx, yy, c, hh, ww)];
                 }
 }
+
+/* ---------------------------------------------------------------------------
+ * MaxPool2D NHWC forward / backward.
+ * pydtnn/cython_modules/max_pool_2d_nhwc_cython.pyx:86-110 and :194-212: the
+ * same rules as the NCHW pair (first maximum, index ii*kw + jj, decoded as
+ * ii = idx / kh, jj = idx % kw), loop order n, output row, output column, c.
+ * ------------------------------------------------------------------------- */
+#define IDX_NHWC(n_, y_, x_, c_, H, W, C) ((((long)(n_) * (H) + (y_)) * (W) + (x_)) * (C) + (c_))
+
+void oracle_max_pool_2d_fwd_nhwc_f32(const float *x, float *y, int32_t *idx_max,
+                                     int n, int h, int w, int c, int kh, int kw,
+                                     int vpadding, int hpadding, int vstride, int hstride,
+                                     int vdilation, int hdilation)
+{
+    const int hh = out_dim(h, vpadding, vdilation, kh, vstride);
+    const int ww = out_dim(w, hpadding, hdilation, kw, hstride);
+    #pragma omp parallel for
+    for (int nn = 0; nn < n; nn++)
+        for (int xx = 0; xx < hh; xx++)
+            for (int yy = 0; yy < ww; yy++)
+                for (int cc = 0; cc < c; cc++) {
+                    float maxval = -FLT_MAX;
+                    int idx_maxval = 0;
+                    for (int ii = 0; ii < kh; ii++) {
+                        const int x_x = vstride * xx + vdilation * ii - vpadding;
+                        if (0 <= x_x && x_x < h)
+                            for (int jj = 0; jj < kw; jj++) {
+                                const int x_y = hstride * yy + hdilation * jj - hpadding;
+                                if (0 <= x_y && x_y < w) {
+                                    const float val = x[IDX_NHWC(nn, x_x, x_y, cc, h, w, c)];
+                                    if (val > maxval) { maxval = val; idx_maxval = ii * kw + jj; }
+                                }
+                            }
+                    }
+                    y[IDX_NHWC(nn, xx, yy, cc, hh, ww, c)] = maxval;
+                    idx_max[IDX_NHWC(nn, xx, yy, cc, hh, ww, c)] = idx_maxval;
+                }
+}
+
+void oracle_max_pool_2d_bwd_nhwc_f32(const float *dy, const int32_t *idx_max, float *dx,
+                                     int n, int h, int w, int c, int kh, int kw,
+                                     int vpadding, int hpadding, int vstride, int hstride,
+                                     int vdilation, int hdilation)
+{
+    const int hh = out_dim(h, vpadding, vdilation, kh, vstride);
+    const int ww = out_dim(w, hpadding, hdilation, kw, hstride);
+    #pragma omp parallel for
+    for (int nn = 0; nn < n; nn++)
+        for (int xx = 0; xx < hh; xx++)
+            for (int yy = 0; yy < ww; yy++)
+                for (int cc = 0; cc < c; cc++) {
+                    const int idx_maxval = idx_max[IDX_NHWC(nn, xx, yy, cc, hh, ww, c)];
+                    const int ii = idx_maxval / kh, jj = idx_maxval % kw;
+                    const int x_x = vstride * xx + vdilation * ii - vpadding;
+                    const int x_y = hstride * yy + hdilation * jj - hpadding;
+                    if (0 <= x_x && x_x < h && 0 <= x_y && x_y < w)
+                        dx[IDX_NHWC(nn, x_x, x_y, cc, h, w, c)] += dy[IDX_NHWC(nn, xx, yy, cc, hh, ww, c)];
+                }
+}

@@ -24,6 +24,8 @@ int launch_softmax_bwd(const float*, const float*, float*, int, int, hipStream_t
 int launch_cce(const float*, const float*, float*, float*, float*, int, int, float, float, float, hipStream_t);
 int launch_max_pool_fwd_nchw(const float*, float*, int32_t*, const ConvGeom&, hipStream_t);
 int launch_max_pool_bwd_nchw(const float*, const int32_t*, float*, const ConvGeom&, hipStream_t);
+int launch_max_pool_fwd_nhwc(const float*, float*, int32_t*, const ConvGeom&, hipStream_t);
+int launch_max_pool_bwd_nhwc(const float*, const int32_t*, float*, const ConvGeom&, hipStream_t);
 int launch_sgd_momentum(float*, const float*, float*, long, float, float, float, int, hipStream_t);
 
 namespace {
@@ -683,6 +685,28 @@ int pydtnn_hip_max_pool_2d_bwd_nchw(const float* dy, const int32_t* idx_max, flo
     const int kn = 1;
     const int rc = geom_from_args(&g, GEOM_ARGS);
     return rc != PYDTNN_HIP_OK ? rc : launch_max_pool_bwd_nchw(dy, idx_max, dx, g, as_stream(stream));
+}
+
+int pydtnn_hip_max_pool_2d_fwd_nhwc(const float* x, float* y, int32_t* idx_max, int b, int h, int w, int c, int kh,
+                                    int kw, int vpadding, int hpadding, int vstride, int hstride, int vdilation,
+                                    int hdilation, void* stream)
+{
+    if (!x || !y || !idx_max) return PYDTNN_HIP_ERR_INVALID;
+    ConvGeom g;
+    const int kn = 1;
+    const int rc = geom_from_args(&g, GEOM_ARGS);
+    return rc != PYDTNN_HIP_OK ? rc : launch_max_pool_fwd_nhwc(x, y, idx_max, g, as_stream(stream));
+}
+
+int pydtnn_hip_max_pool_2d_bwd_nhwc(const float* dy, const int32_t* idx_max, float* dx, int b, int h, int w, int c,
+                                    int kh, int kw, int vpadding, int hpadding, int vstride, int hstride,
+                                    int vdilation, int hdilation, void* stream)
+{
+    if (!dy || !dx || !idx_max) return PYDTNN_HIP_ERR_INVALID;
+    ConvGeom g;
+    const int kn = 1;
+    const int rc = geom_from_args(&g, GEOM_ARGS);
+    return rc != PYDTNN_HIP_OK ? rc : launch_max_pool_bwd_nhwc(dy, idx_max, dx, g, as_stream(stream));
 }
 
 size_t pydtnn_hip_bn_training_workspace_bytes(int channels)

@@ -312,6 +312,77 @@ __global__ void __launch_bounds__(kThreads) max_pool_bwd_nchw_kernel(const float
     }
 }
 
+// ---------------------------------------------------------------- MaxPool2D NHWC
+// pydtnn/cython_modules/max_pool_2d_nhwc_cython.pyx:86-110 and :194-212: the rules of the NCHW pair.
+// grid.x * 256 threads walk the (pixel, channel) elements of one image, lanes along c; grid.y walks the images.
+__global__ void __launch_bounds__(kThreads) max_pool_fwd_nhwc_kernel(const float* __restrict__ x,
+                                                                    float* __restrict__ y,
+                                                                    int32_t* __restrict__ idx_max, ConvGeom g,
+                                                                    int c_exact)
+{
+    const uint32_t per_image = (uint32_t)(g.howo * g.c);
+    const uint32_t e = blockIdx.x * kThreads + threadIdx.x;
+    if (e >= per_image) return;
+    const uint32_t pix = fd_div_checked(e, g.fd_c, c_exact);
+    const uint32_t cc = e - pix * g.c;
+    const int oy = (int)fd_div(pix, g.fd_wo);
+    const int ox = (int)pix - oy * g.wo;
+    const int y0 = g.vstride * oy - g.vpadding, x0 = g.hstride * ox - g.hpadding;
+    for (uint32_t nn = blockIdx.y; nn < (uint32_t)g.n; nn += gridDim.y) {
+        const float* src = x + (size_t)nn * g.h * g.w * g.c + cc;
+        float maxval = -3.402823466e+38f;
+        int best = 0;
+        for (int ii = 0; ii < g.kh; ++ii) {
+            const int x_x = y0 + g.vdilation * ii;
+            if ((unsigned)x_x >= (unsigned)g.h) continue;
+            for (int jj = 0; jj < g.kw; ++jj) {
+                const int x_y = x0 + g.hdilation * jj;
+                if ((unsigned)x_y >= (unsigned)g.w) continue;
+                const float val = src[(size_t)(x_x * g.w + x_y) * g.c];
+                if (val > maxval) { maxval = val; best = ii * g.kw + jj; }
+            }
+        }
+        y[(size_t)nn * per_image + e] = maxval;
+        idx_max[(size_t)nn * per_image + e] = best;
+    }
+}
+
+// Gather form of the backward scatter: windows visited in ascending (oy, ox), i.e. descending taps.
+__global__ void __launch_bounds__(kThreads) max_pool_bwd_nhwc_kernel(const float* __restrict__ dy,
+                                                                    const int32_t* __restrict__ idx_max,
+                                                                    float* __restrict__ dx, ConvGeom g, int c_exact)
+{
+    const uint32_t per_image = (uint32_t)(g.h * g.w * g.c);
+    const uint32_t e = blockIdx.x * kThreads + threadIdx.x;
+    if (e >= per_image) return;
+    const uint32_t pix = fd_div_checked(e, g.fd_c, c_exact);
+    const uint32_t cc = e - pix * g.c;
+    const int hh = (int)fd_div(pix, g.fd_w);
+    const int ww = (int)pix - hh * g.w;
+    for (uint32_t nn = blockIdx.y; nn < (uint32_t)g.n; nn += gridDim.y) {
+        const size_t base = (size_t)nn * g.howo * g.c + cc;
+        float acc = 0.0f;
+        for (int ii = g.kh - 1; ii >= 0; --ii) {
+            const int ty = hh + g.vpadding - g.vdilation * ii;
+            if (ty < 0) continue;
+            const int oy = (int)fd_div((uint32_t)ty, g.fd_vs);
+            if (oy * g.vstride != ty || oy >= g.ho) continue;
+            for (int jj = g.kw - 1; jj >= 0; --jj) {
+                const int tx = ww + g.hpadding - g.hdilation * jj;
+                if (tx < 0) continue;
+                const int ox = (int)fd_div((uint32_t)tx, g.fd_hs);
+                if (ox * g.hstride != tx || ox >= g.wo) continue;
+                const size_t at = base + (size_t)(oy * g.wo + ox) * g.c;
+                const uint32_t rec = (uint32_t)idx_max[at];
+                const uint32_t ri = fd_div(rec, g.fd_kh);
+                const uint32_t rj = rec - fd_div(rec, g.fd_kw) * g.kw;
+                if ((int)ri == ii && (int)rj == jj) acc += dy[at];
+            }
+        }
+        dx[(size_t)nn * per_image + e] = acc;
+    }
+}
+
 // ---------------------------------------------------------------- SGD with momentum
 // pydtnn/backends/cpu/optimizers/sgd_cpu.py:28-41
 __global__ void __launch_bounds__(kThreads) sgd_momentum_kernel(float* __restrict__ w, const float* __restrict__ dw,
@@ -723,6 +794,29 @@ int launch_max_pool_bwd_nchw(const float* dy, const int32_t* idx_max, float* dx,
         hipLaunchKernelGGL(max_pool_bwd_nchw_kernel<true>, grid, dim3(kThreads), 0, stream, dy, idx_max, dx, g);
     else
         hipLaunchKernelGGL(max_pool_bwd_nchw_kernel<false>, grid, dim3(kThreads), 0, stream, dy, idx_max, dx, g);
+    HIP_RETURN_IF_LAUNCH_FAILED();
+    return PYDTNN_HIP_OK;
+}
+
+int launch_max_pool_fwd_nhwc(const float* x, float* y, int32_t* idx_max, const ConvGeom& g, hipStream_t stream)
+{
+    const long per_image = (long)g.howo * g.c;
+    if (per_image >= (1l << 31) - kThreads) return PYDTNN_HIP_ERR_UNSUPPORTED;
+    const int c_exact = (unsigned long)(per_image + kThreads) * (unsigned long)g.c < (1ul << 32);
+    dim3 grid(blocks_for(per_image), (unsigned)(g.n < 65535 ? g.n : 65535));
+    hipLaunchKernelGGL(max_pool_fwd_nhwc_kernel, grid, dim3(kThreads), 0, stream, x, y, idx_max, g, c_exact);
+    HIP_RETURN_IF_LAUNCH_FAILED();
+    return PYDTNN_HIP_OK;
+}
+
+int launch_max_pool_bwd_nhwc(const float* dy, const int32_t* idx_max, float* dx, const ConvGeom& g,
+                             hipStream_t stream)
+{
+    const long per_image = (long)g.h * g.w * g.c;
+    if (per_image >= (1l << 31) - kThreads) return PYDTNN_HIP_ERR_UNSUPPORTED;
+    const int c_exact = (unsigned long)(per_image + kThreads) * (unsigned long)g.c < (1ul << 32);
+    dim3 grid(blocks_for(per_image), (unsigned)(g.n < 65535 ? g.n : 65535));
+    hipLaunchKernelGGL(max_pool_bwd_nhwc_kernel, grid, dim3(kThreads), 0, stream, dy, idx_max, dx, g, c_exact);
     HIP_RETURN_IF_LAUNCH_FAILED();
     return PYDTNN_HIP_OK;
 }

@@ -411,22 +411,24 @@ class MaxPool2D(Layer):
         assert self.ho > 0 and self.wo > 0, "Output dimensions must be greater than 0"
         self.shape = encode_tensor((self.ho, self.wo, self.co), self.model.tensor_format)
         self.n = int(np.prod(self.shape))
-        if self.model.tensor_format != PYDTNN_TENSOR_FORMAT_NCHW:
-            raise NotImplementedError("MaxPool2D is implemented for the NCHW tensor format only")
 
     def _geom(self):
         return (self.kh, self.kw, self.vpadding, self.hpadding, self.vstride, self.hstride,
                 self.vdilation, self.hdilation)
 
     def forward(self, x):
-        y, idx_max = ops.max_pool_2d_fwd_nchw(x, *self._geom())
+        nchw = self.model.tensor_format == PYDTNN_TENSOR_FORMAT_NCHW
+        y, idx_max = (ops.max_pool_2d_fwd_nchw if nchw else ops.max_pool_2d_fwd_nhwc)(x, *self._geom())
         if self.model.mode == TRAIN_MODE:
             self.idx_max = idx_max
         return y
 
     def backward(self, dy):
         if self.need_dx:
-            return ops.max_pool_2d_bwd_nchw(dy, self.idx_max, dy.shape[0], self.ci, self.hi, self.wi, *self._geom())
+            if self.model.tensor_format == PYDTNN_TENSOR_FORMAT_NCHW:
+                return ops.max_pool_2d_bwd_nchw(dy, self.idx_max, dy.shape[0], self.ci, self.hi, self.wi,
+                                                *self._geom())
+            return ops.max_pool_2d_bwd_nhwc(dy, self.idx_max, dy.shape[0], self.hi, self.wi, self.ci, *self._geom())
 
 
 class Flatten(Layer):

@@ -207,6 +207,29 @@ def max_pool_2d_bwd_nchw(dy, idx_max, n, c, h, w, kh, kw, vpadding, hpadding, vs
     return dx
 
 
+def max_pool_2d_fwd_nhwc(x, kh, kw, vpadding, hpadding, vstride, hstride, vdilation=1, hdilation=1):
+    """pydtnn/cython_modules/max_pool_2d_nhwc_cython.pyx:25-52 -> (y, idx_max int32)"""
+    _need_f32(x)
+    n, h, w, c = x.shape
+    hh, ww = _out_hw(h, w, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
+    y = torch.empty((n, hh, ww, c), dtype=x.dtype, device=x.device)
+    idx = torch.empty((n, hh, ww, c), dtype=torch.int32, device=x.device)
+    check(lib().pydtnn_hip_max_pool_2d_fwd_nhwc(f32(x), f32(y), ptr(idx), n, h, w, c, kh, kw, vpadding, hpadding,
+                                                vstride, hstride, vdilation, hdilation, stream_ptr()), "max_pool_fwd")
+    return y, idx
+
+
+def max_pool_2d_bwd_nhwc(dy, idx_max, n, h, w, c, kh, kw, vpadding, hpadding, vstride, hstride,
+                         vdilation=1, hdilation=1):
+    """pydtnn/cython_modules/max_pool_2d_nhwc_cython.pyx:140-166"""
+    _need_f32(dy)
+    dx = torch.empty((n, h, w, c), dtype=dy.dtype, device=dy.device)
+    check(lib().pydtnn_hip_max_pool_2d_bwd_nhwc(f32(dy), ptr(idx_max), f32(dx), n, h, w, c, kh, kw, vpadding,
+                                                hpadding, vstride, hstride, vdilation, hdilation, stream_ptr()),
+          "max_pool_bwd")
+    return dx
+
+
 def bn_training_forward(x, gamma, beta, running_mean, running_var, momentum, eps, channels, inner):
     """pydtnn/backends/cpu/layers/batch_normalization_cpu.py:59-82 on x viewed as (outer, channels, inner).
     Updates running_mean / running_var in place; returns (y, xn, std)."""

@@ -368,6 +368,23 @@ def test_sgd_momentum(ops, oracle):
     assert_close(host(vd), v_ref, tol=1e-6, what="sgd v")
 
 
+def test_maxpool_nhwc_matches_oracle(ops, oracle):
+    rng = np.random.default_rng(12)
+    for (shape, kh, kw, p, s, dil) in [((2, 8, 10, 3), 2, 2, 0, 2, 1), ((2, 9, 9, 70), 3, 3, 1, 2, 1),
+                                       ((1, 7, 11, 5), 3, 2, 1, 1, 1), ((1, 9, 9, 2), 2, 2, 1, 1, 2)]:
+        announce("maxpool nhwc", shape, kh, kw, p, s, dil)
+        x = rng.standard_normal(shape).astype(np.float32)
+        x[0, :2, :2, 0] = 1.5  # ties: the first tap must win
+        g = (kh, kw, p, p, s, s, dil, dil)
+        y, idx = ops.max_pool_2d_fwd_nhwc(dev(x), *g)
+        y_ref, idx_ref = oracle.max_pool_2d_fwd_nhwc(x, *g)
+        assert np.array_equal(host(y), y_ref) and np.array_equal(host(idx), idx_ref)
+        dy = rng.standard_normal(y_ref.shape).astype(np.float32)
+        dx = ops.max_pool_2d_bwd_nhwc(dev(dy), idx, *shape, *g)
+        dx_ref = oracle.max_pool_2d_bwd_nhwc(dy, idx_ref, *shape, *g)
+        assert np.array_equal(host(dx), dx_ref)
+
+
 @pytest.mark.parametrize("fmt,shape", [("NCHW", (8, 6, 5, 7)), ("NCHW", (70, 3, 4, 4)), ("NHWC", (8, 5, 7, 6)),
                                        ("NHWC", (3, 9, 9, 130)), ("2D", (64, 10)), ("2D", (300, 70)), ("2D", (2, 3))])
 def test_bn_training_forward_backward(ops, oracle, fmt, shape):

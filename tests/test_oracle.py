@@ -428,6 +428,26 @@ def test_maxpool_against_torch_and_tie_rule(oracle):
     assert idx1.item() == 0 and y1.item() == 3.0
 
 
+def test_maxpool_nhwc_is_the_nchw_pool_in_the_other_layout(oracle):
+    """The NHWC pair follows the same rules, so it must equal the (torch-pinned) NCHW pair on the transposed
+    tensor, including rectangular windows, padding, dilation and the reference's idx // kh, idx % kw decode."""
+    rng = np.random.default_rng(15)
+    for (n, c, h, w, kh, kw, pv, ph, sv, sh, dv, dh) in [(2, 3, 8, 10, 2, 2, 0, 0, 2, 2, 1, 1),
+                                                          (2, 4, 9, 9, 3, 3, 1, 1, 2, 2, 1, 1),
+                                                          (1, 5, 7, 11, 3, 2, 1, 0, 1, 2, 1, 1),
+                                                          (1, 2, 9, 9, 2, 2, 1, 1, 1, 1, 2, 2)]:
+        x = rng.standard_normal((n, c, h, w)).astype(np.float32)
+        x[0, 0, :3, :3] = 0.75
+        g = (kh, kw, pv, ph, sv, sh, dv, dh)
+        y, idx = oracle.max_pool_2d_fwd_nchw(x, *g)
+        yh, idxh = oracle.max_pool_2d_fwd_nhwc(np.ascontiguousarray(x.transpose(0, 2, 3, 1)), *g)
+        assert np.array_equal(yh, y.transpose(0, 2, 3, 1)) and np.array_equal(idxh, idx.transpose(0, 2, 3, 1))
+        dy = rng.standard_normal(y.shape).astype(np.float32)
+        dx = oracle.max_pool_2d_bwd_nchw(dy, idx, n, c, h, w, *g)
+        dxh = oracle.max_pool_2d_bwd_nhwc(np.ascontiguousarray(dy.transpose(0, 2, 3, 1)), idxh, n, h, w, c, *g)
+        assert np.array_equal(dxh, dx.transpose(0, 2, 3, 1))
+
+
 # ------------------------------------------------------------------ larger library cross-check
 
 @pytest.mark.parametrize("layer", [0, 1, 4, 7], ids=lambda i: f"alexnet{i}")
