@@ -35,27 +35,44 @@ using namespace gemm;
 typedef Tile<128, 128, 2, 2> T128x128;
 typedef Tile<64, 256, 1, 4> T64x256;
 typedef Tile<256, 64, 4, 1> T256x64;
+typedef Tile<64, 64, 2, 2> T64x64;
 
-enum TileSel { SEL_128x128, SEL_64x256, SEL_256x64 };
+enum TileSel { SEL_128x128, SEL_64x256, SEL_256x64, SEL_64x64, SEL_COUNT };
 
-inline TileSel pick_tile(long m, long n)
-{
-    if (m <= 64) return SEL_64x256;
-    if (n <= 64) return SEL_256x64;
-    return SEL_128x128;
-}
+struct TileShape {
+    long bm, bn;
+    double efficiency;  // matrix-core rate of the shape relative to 128x128 (fewer MFMAs per load and barrier)
+};
+constexpr TileShape kTileShapes[SEL_COUNT] = {{128, 128, 1.0}, {64, 256, 0.93}, {256, 64, 0.93}, {64, 64, 0.6}};
 
 inline long tiles_of(TileSel sel, long m, long n)
 {
-    const long bm = sel == SEL_64x256 ? 64 : sel == SEL_256x64 ? 256 : 128;
-    const long bn = sel == SEL_64x256 ? 256 : sel == SEL_256x64 ? 64 : 128;
-    return ((m + bm - 1) / bm) * ((n + bn - 1) / bn);
+    const TileShape& t = kTileShapes[sel];
+    return ((m + t.bm - 1) / t.bm) * ((n + t.bn - 1) / t.bn);
+}
+
+// The shape that computes the fewest padded products, weighted by what the shape achieves.  A
+// reduction of a step or two is all set-up (per-row tap masks, prologue): then the small tile, which
+// has a quarter of the rows per thread and fills the chip with more workgroups, unless the
+// problem already makes plenty of large ones.
+inline TileSel pick_tile(long m, long n, long k = 1l << 30)
+{
+    if (k <= 2 * BK && tiles_of(SEL_128x128, m, n) < 2048) return SEL_64x64;
+    TileSel best = SEL_128x128;
+    double best_cost = 0.0;
+    for (int s = 0; s < SEL_COUNT; ++s) {
+        const TileShape& t = kTileShapes[s];
+        const double cost = (double)tiles_of((TileSel)s, m, n) * (double)(t.bm * t.bn) / t.efficiency;
+        if (s == 0 || cost < best_cost) { best = (TileSel)s; best_cost = cost; }
+    }
+    return best;
 }
 
 #define WITH_TILE(sel, ...)                                                 \
     switch (sel) {                                                          \
         case SEL_64x256: { typedef T64x256 T; __VA_ARGS__; } break;         \
         case SEL_256x64: { typedef T256x64 T; __VA_ARGS__; } break;         \
+        case SEL_64x64: { typedef T64x64 T; __VA_ARGS__; } break;           \
         default: { typedef T128x128 T; __VA_ARGS__; } break;                \
     }
 
@@ -184,7 +201,7 @@ template <bool WIDE>
 int conv_fwd_nchw_t(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan, float* ws,
                     size_t ws_bytes, hipStream_t stream)
 {
-    const TileSel sel = pick_tile(g.kn, g.p);
+    const TileSel sel = pick_tile(g.kn, g.p, g.k);
     int rc = PYDTNN_HIP_OK;
     WITH_TILE(sel, {
         if (!span_ok_k(T::BM, g.k, 0, 0)) return PYDTNN_HIP_ERR_UNSUPPORTED;
@@ -209,7 +226,7 @@ template <bool WIDE>
 int conv_fwd_nhwc_t(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan, float* ws,
                     size_t ws_bytes, hipStream_t stream)
 {
-    const TileSel sel = pick_tile(g.p, g.kn);
+    const TileSel sel = pick_tile(g.p, g.kn, g.k);
     int rc = PYDTNN_HIP_OK;
     WITH_TILE(sel, {
         Im2rowNhwcK<T::BM, WIDE> al;
@@ -591,7 +608,7 @@ int pydtnn_hip_conv_i2c_forward(int nhwc, int b, int c, int h, int w, int kn, in
     const ChanEpilogue chan = make_chan(bias_vector, nullptr, nullptr, nullptr, nullptr, 0);
     const hipStream_t st = as_stream(stream);
     if (!nhwc) {
-        const TileSel sel = pick_tile(g.kn, g.p);
+        const TileSel sel = pick_tile(g.kn, g.p, g.k);
         WITH_TILE(sel, {
             if (!span_ok_mn(g.p)) return PYDTNN_HIP_ERR_UNSUPPORTED;
             rc = launch<T>(plain_k<T::BM, false>(weights, (long)g.kn * g.k, g.k, 0, g.kn, 0),
@@ -599,7 +616,7 @@ int pydtnn_hip_conv_i2c_forward(int nhwc, int b, int c, int h, int w, int kn, in
                            epi_nchw(y, g.kn, g.howo, g.p, chan), g.kn, g.p, no_split(g.k), 1, st);
         })
     } else {
-        const TileSel sel = pick_tile(g.p, g.kn);
+        const TileSel sel = pick_tile(g.p, g.kn, g.k);
         WITH_TILE(sel, {
             rc = launch<T>(plain_k<T::BM, false>(mat, g.p * g.k, g.k, 0, g.p, 0),
                            plain_mn<T::BN>(weights, (long)g.k * g.kn, g.kn, 0, g.kn),

@@ -973,20 +973,26 @@ __global__ void __launch_bounds__(kThreads) streamk_fixup_kernel(EP ep, int tile
     for (int q = 0; q < 4; ++q) ep.store(col, m0 + wm0 + i * 32 + 8 * ((v0 + q) / 4) + 4 * frag_k + ((v0 + q) % 4), acc[q]);
 }
 
-// Workgroups of gemm_streamk_kernel<T, ...> the device holds at once.
+// Workgroups of gemm_streamk_kernel<T, ...> the device holds at once, and its compute units.
+struct Residency {
+    int workgroups;
+    int cus;
+};
+
 template <class T, class AL, class BL, class EP>
-inline int resident_workgroups()
+inline Residency resident_workgroups()
 {
-    static int cached = 0;
-    if (cached == 0) {
+    static Residency cached = {0, 0};
+    if (cached.workgroups == 0) {
         int dev = 0, cus = 0, per_cu = 0;
         if (hipGetDevice(&dev) != hipSuccess ||
             hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
             hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_streamk_kernel<T, AL, BL, EP>, kThreads, 0) !=
                 hipSuccess ||
             cus <= 0 || per_cu <= 0)
-            return 0;
-        cached = cus * per_cu;
+            return cached;
+        cached.workgroups = cus * per_cu;
+        cached.cus = cus;
     }
     return cached;
 }
@@ -1002,10 +1008,18 @@ inline int launch_balanced(const AL& al, const BL& bl, const EP& ep, long m, lon
     const long tiles_m = (m + T::BM - 1) / T::BM, tiles_n = (n + T::BN - 1) / T::BN;
     const long tiles = tiles_m * tiles_n;
     if (tiles >= (1l << 31)) return PYDTNN_HIP_ERR_UNSUPPORTED;
-    const int resident = resident_workgroups<T, AL, BL, EP>();
+    const Residency res = resident_workgroups<T, AL, BL, EP>();
+    const int resident = res.workgroups;
     const int units = (k + 2 * BK - 1) / (2 * BK);
     bool balanced = resident > 0 && partial && partial_bytes >= streamk_workspace_bytes(resident, T::BM, T::BN) &&
-                    tiles % resident != 0 && tiles < 16l * resident && units >= 8;
+                    tiles % resident != 0 && units >= 8;
+    if (balanced) {
+        // A plain grid keeps every compute unit busy for ceil(tiles / CUs) tile times; balancing is
+        // worth its partial-tile traffic only when more than a twentieth of that is idle.
+        const double per_cu = (double)tiles / res.cus;
+        const double rounds = (double)((tiles + res.cus - 1) / res.cus);
+        balanced = per_cu / rounds < 0.95;
+    }
     if (!balanced) return launch<T>(al, bl, ep, m, n, no_split(k), 1, stream);
     StreamK sk;
     sk.tiles = (int)tiles;
