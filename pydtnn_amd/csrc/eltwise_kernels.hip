@@ -119,7 +119,9 @@ __device__ __forceinline__ float block_sum(float v)
     return s;  // valid on thread 0
 }
 
-// NCHW: grid (C, S); slice s covers images [s*per, (s+1)*per).
+// NCHW: grid (C, S); slice s covers images [s*per, (s+1)*per).  VEC4: planes are read 16 bytes per lane
+// (hw % 4 == 0 and a 16-byte aligned tensor).
+template <bool VEC4>
 __global__ void __launch_bounds__(kThreads) bias_grad_nchw_stage1(const float* __restrict__ dy,
                                                                  float* __restrict__ partial, int n, int c,
                                                                  int hw, int per)
@@ -129,7 +131,17 @@ __global__ void __launch_bounds__(kThreads) bias_grad_nchw_stage1(const float* _
     float acc = 0.0f;
     for (int nn = n0; nn < n1; ++nn) {
         const float* plane = dy + ((long)nn * c + ch) * hw;
-        for (int i = threadIdx.x; i < hw; i += kThreads) acc += plane[i];
+        if (VEC4) {
+            const float4* p4 = reinterpret_cast<const float4*>(plane);
+            float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+            for (int i = threadIdx.x; i < hw / 4; i += kThreads) {
+                const float4 v = p4[i];
+                a0 += v.x; a1 += v.y; a2 += v.z; a3 += v.w;
+            }
+            acc += (a0 + a1) + (a2 + a3);
+        } else {
+            for (int i = threadIdx.x; i < hw; i += kThreads) acc += plane[i];
+        }
     }
     const float tot = block_sum(acc);
     if (threadIdx.x == 0) partial[(long)s * c + ch] = tot;
@@ -254,11 +266,44 @@ __global__ void __launch_bounds__(kThreads) max_pool_fwd_nchw_kernel(const float
     }
 }
 
+// Backward when square windows tile the plane exactly (kh == kw == both strides, no padding or
+// dilation, h == ho*kh, w == wo*kw): one thread owns one window, reads its index and gradient once
+// and writes the window's kh x kw elements of dx (the decoded element gets 0 + dy, the others 0).
+// The decode is the reference's own (ii = idx / kh, jj = idx % kw, max_pool_2d_nchw_cython.pyx:204-205).
+template <int KW>
+__global__ void __launch_bounds__(kThreads) max_pool_bwd_windows_nchw_kernel(const float* __restrict__ dy,
+                                                                            const int32_t* __restrict__ idx_max,
+                                                                            float* __restrict__ dx, ConvGeom g)
+{
+    const uint32_t win = blockIdx.x * kThreads + threadIdx.x;
+    if (win >= (uint32_t)g.howo) return;
+    const int oy = (int)fd_div(win, g.fd_wo);
+    const int ox = (int)win - oy * g.wo;
+    const uint32_t planes = (uint32_t)(g.n * g.c);
+    const int kw = KW > 0 ? KW : g.kw;
+    for (uint32_t plane = blockIdx.y; plane < planes; plane += gridDim.y) {
+        const uint32_t rec = (uint32_t)idx_max[(size_t)plane * g.howo + win];
+        const float grad = 0.0f + dy[(size_t)plane * g.howo + win];
+        const int ri = (int)fd_div(rec, g.fd_kh);
+        const int rj = (int)(rec - fd_div(rec, g.fd_kw) * g.kw);
+        float* dst = dx + (size_t)plane * g.h * g.w + (size_t)(oy * g.kh) * g.w + ox * kw;
+        for (int ii = 0; ii < g.kh; ++ii) {
+            if (KW == 2) {
+                *reinterpret_cast<float2*>(dst) =
+                    make_float2(ii == ri && rj == 0 ? grad : 0.0f, ii == ri && rj == 1 ? grad : 0.0f);
+            } else {
+                for (int jj = 0; jj < kw; ++jj) dst[jj] = ii == ri && jj == rj ? grad : 0.0f;
+            }
+            dst += g.w;
+        }
+    }
+}
+
 // Backward in gather form: one thread per dx element sums dy of every window whose recorded
 // maximum decodes to this element.  The decode is the reference's own
 // (ii = idx / kh, jj = idx % kw, max_pool_2d_nchw_cython.pyx:204-205).  Windows are visited in
 // ascending (oy, ox), the order of the reference's scatter loop.
-// TILED: windows do not overlap and have no padding or dilation (kh == vstride, kw == hstride),
+// TILED: square windows that do not overlap and have no padding or dilation (kh == kw == both strides),
 // so each element lies in at most one window and the tap loops collapse to one lookup.
 template <bool TILED>
 __global__ void __launch_bounds__(kThreads) max_pool_bwd_nchw_kernel(const float* __restrict__ dy,
@@ -292,7 +337,8 @@ __global__ void __launch_bounds__(kThreads) max_pool_bwd_nchw_kernel(const float
         const float* gy = dy + (long)plane * g.howo;
         const int32_t* gi = idx_max + (long)plane * g.howo;
         float acc = 0.0f;
-        for (int ii = g.kh - 1; ii >= 0; --ii) {
+        // decoded rows run up to (kh*kw - 1) / kh, which exceeds kh - 1 when kw > kh
+        for (int ii = (g.khw - 1) / g.kh; ii >= 0; --ii) {
             const int ty = hh + g.vpadding - g.vdilation * ii;
             if (ty < 0) continue;
             const int oy = (int)fd_div((uint32_t)ty, g.fd_vs);
@@ -362,7 +408,8 @@ __global__ void __launch_bounds__(kThreads) max_pool_bwd_nhwc_kernel(const float
     for (uint32_t nn = blockIdx.y; nn < (uint32_t)g.n; nn += gridDim.y) {
         const size_t base = (size_t)nn * g.howo * g.c + cc;
         float acc = 0.0f;
-        for (int ii = g.kh - 1; ii >= 0; --ii) {
+        // decoded rows run up to (kh*kw - 1) / kh, which exceeds kh - 1 when kw > kh
+        for (int ii = (g.khw - 1) / g.kh; ii >= 0; --ii) {
             const int ty = hh + g.vpadding - g.vdilation * ii;
             if (ty < 0) continue;
             const int oy = (int)fd_div((uint32_t)ty, g.fd_vs);
@@ -734,8 +781,12 @@ int launch_bias_grad(const float* dy, float* db, long outer, int channels, int i
         slices = n < 64 ? n : 64;
         const int per = (n + slices - 1) / slices;
         slices = (n + per - 1) / per;
-        hipLaunchKernelGGL(bias_grad_nchw_stage1, dim3(channels, slices), dim3(kThreads), 0, stream, dy, workspace, n,
-                           channels, inner, per);
+        if (inner % 4 == 0 && (reinterpret_cast<uintptr_t>(dy) & 15) == 0)
+            hipLaunchKernelGGL(bias_grad_nchw_stage1<true>, dim3(channels, slices), dim3(kThreads), 0, stream, dy,
+                               workspace, n, channels, inner, per);
+        else
+            hipLaunchKernelGGL(bias_grad_nchw_stage1<false>, dim3(channels, slices), dim3(kThreads), 0, stream, dy,
+                               workspace, n, channels, inner, per);
     } else {
         slices = outer < 64 * 4 ? (int)((outer + 3) / 4) : 64;
         const long per = (outer + slices - 1) / slices;
@@ -788,9 +839,19 @@ int launch_max_pool_bwd_nchw(const float* dy, const int32_t* idx_max, float* dx,
 {
     const long planes = (long)g.n * g.c;
     dim3 grid(blocks_for((long)g.h * g.w), (unsigned)(planes < 65535 ? planes : 65535));
-    const bool tiled = g.kh == g.vstride && g.kw == g.hstride && g.vpadding == 0 && g.hpadding == 0 &&
-                       g.vdilation == 1 && g.hdilation == 1;
-    if (tiled)
+    // square windows only: with kh != kw the reference's decode can leave the window it came from and land
+    // in a neighbour's, which only the general gather follows
+    const bool tiled = g.kh == g.kw && g.kh == g.vstride && g.kw == g.hstride && g.vpadding == 0 &&
+                       g.hpadding == 0 && g.vdilation == 1 && g.hdilation == 1;
+    if (tiled && g.h == g.ho * g.kh && g.w == g.wo * g.kw) {
+        dim3 wgrid(blocks_for(g.howo), (unsigned)(planes < 65535 ? planes : 65535));
+        if (g.kw == 2 && (reinterpret_cast<uintptr_t>(dx) & 7) == 0)
+            hipLaunchKernelGGL(max_pool_bwd_windows_nchw_kernel<2>, wgrid, dim3(kThreads), 0, stream, dy, idx_max, dx,
+                               g);
+        else
+            hipLaunchKernelGGL(max_pool_bwd_windows_nchw_kernel<0>, wgrid, dim3(kThreads), 0, stream, dy, idx_max, dx,
+                               g);
+    } else if (tiled)
         hipLaunchKernelGGL(max_pool_bwd_nchw_kernel<true>, grid, dim3(kThreads), 0, stream, dy, idx_max, dx, g);
     else
         hipLaunchKernelGGL(max_pool_bwd_nchw_kernel<false>, grid, dim3(kThreads), 0, stream, dy, idx_max, dx, g);

@@ -345,7 +345,8 @@ def test_bias_grad(ops):
 
 def test_maxpool_matches_oracle(ops, oracle):
     rng = np.random.default_rng(10)
-    for (shape, k, s, p) in [((2, 3, 8, 10), 2, 2, 0), ((2, 4, 9, 9), 3, 2, 1), ((1, 2, 7, 7), 3, 1, 1)]:
+    for (shape, k, s, p) in [((2, 3, 8, 10), 2, 2, 0), ((2, 4, 9, 9), 3, 2, 1), ((1, 2, 7, 7), 3, 1, 1),
+                             ((2, 3, 9, 11), 2, 2, 0), ((1, 2, 9, 12), 3, 3, 0), ((3, 5, 14, 14), 2, 2, 0)]:
         announce("maxpool", shape, k, s, p)
         x = rng.standard_normal(shape).astype(np.float32)
         x[0, 0, :2, :2] = 1.5  # ties: the first tap must win
@@ -368,10 +369,27 @@ def test_sgd_momentum(ops, oracle):
     assert_close(host(vd), v_ref, tol=1e-6, what="sgd v")
 
 
+def test_maxpool_rectangular_windows_keep_the_reference_decode(ops, oracle):
+    """kh != kw: the reference decodes the stored index as (idx // kh, idx % kw), which differs from how it
+    was encoded (ii*kw + jj); the backward kernels must reproduce that, also when windows tile the plane."""
+    rng = np.random.default_rng(13)
+    for (shape, kh, kw, sv, sh) in [((2, 3, 8, 12), 2, 3, 2, 3), ((1, 2, 9, 8), 3, 2, 3, 2), ((1, 2, 7, 9), 2, 3, 1, 1)]:
+        announce("maxpool rect", shape, kh, kw, sv, sh)
+        x = rng.standard_normal(shape).astype(np.float32)
+        g = (kh, kw, 0, 0, sv, sh)
+        y, idx = ops.max_pool_2d_fwd_nchw(dev(x), *g)
+        y_ref, idx_ref = oracle.max_pool_2d_fwd_nchw(x, *g)
+        assert np.array_equal(host(y), y_ref) and np.array_equal(host(idx), idx_ref)
+        dy = rng.standard_normal(y_ref.shape).astype(np.float32)
+        dx = ops.max_pool_2d_bwd_nchw(dev(dy), idx, *shape, *g)
+        assert_close(host(dx), oracle.max_pool_2d_bwd_nchw(dy, idx_ref, *shape, *g), tol=1e-6, what="maxpool bwd")
+
+
 def test_maxpool_nhwc_matches_oracle(ops, oracle):
     rng = np.random.default_rng(12)
     for (shape, kh, kw, p, s, dil) in [((2, 8, 10, 3), 2, 2, 0, 2, 1), ((2, 9, 9, 70), 3, 3, 1, 2, 1),
-                                       ((1, 7, 11, 5), 3, 2, 1, 1, 1), ((1, 9, 9, 2), 2, 2, 1, 1, 2)]:
+                                       ((1, 7, 11, 5), 3, 2, 1, 1, 1), ((1, 9, 9, 2), 2, 2, 1, 1, 2),
+                                       ((2, 8, 12, 4), 2, 3, 0, 1, 1), ((1, 8, 12, 3), 2, 3, 1, 2, 1)]:
         announce("maxpool nhwc", shape, kh, kw, p, s, dil)
         x = rng.standard_normal(shape).astype(np.float32)
         x[0, :2, :2, 0] = 1.5  # ties: the first tap must win
