@@ -109,24 +109,40 @@ __device__ __forceinline__ uint32_t lds_addr(const float* p)
     return (uint32_t)(uintptr_t)((__attribute__((address_space(3))) const float*)p);
 }
 
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+
 template <int OFF>
-__device__ __forceinline__ float lds_read(uint32_t addr)
+__device__ __forceinline__ floatx2 lds_read2(uint32_t addr)
 {
-    static_assert(OFF >= 0 && OFF < 65536, "ds_read_b32 takes a 16-bit byte offset");
-    float v;
-    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+    static_assert(OFF >= 0 && OFF < 65536 && OFF % 8 == 0, "ds_read_b64 takes a 16-bit byte offset");
+    floatx2 v;
+    asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
     return v;
 }
 
 // Waits for every outstanding LDS read; the registers are passed through so that their uses cannot be
 // scheduled above the wait.
 template <int N>
-__device__ __forceinline__ void lds_wait(float (&a)[N])
+__device__ __forceinline__ void lds_wait(floatx2 (&a)[N])
 {
     asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]));
 #pragma unroll
     for (int i = 1; i < N; ++i) asm volatile("" : "+v"(a[i]));
 }
+
+// LDS tile layout.  Reduction rows k and k+2 of the same column sit next to each other, so that one
+// 64-bit read serves two consecutive MFMA k-steps (lane (r, h) needs k = 2J + h for step J):
+//   float index of (k, mn) = ((k >> 2) * 2 + (k & 1)) * kRowPitch + mn * 2 + ((k >> 1) & 1)
+// with kRowPitch = 2 * (BMN + kPad) floats; the tile takes BK * (BMN + kPad) floats as before.
+template <int BMN>
+struct LdsTile {
+    static constexpr int kRowPitch = 2 * (BMN + kPad);
+    static constexpr int kFloats = BK * (BMN + kPad);
+    static __device__ __forceinline__ int index(int k, int mn)
+    {
+        return ((k >> 2) * 2 + (k & 1)) * kRowPitch + mn * 2 + ((k >> 1) & 1);
+    }
+};
 
 // Tap masks for the padding test.  Bit t of the returned word is 1 when tap t must read as zero.
 // Narrow form (kh*kw <= 31): one word over the combined tap index i*kw + j.  Wide form: one word over
@@ -160,11 +176,27 @@ struct MapMN {
     static constexpr int NLD = BK / kRowsPerPass;
     static __device__ __forceinline__ int mn(int tid) { return tid % BMN; }
     static __device__ __forceinline__ int krow(int tid) { return uniform(tid / BMN); }
+    // This thread's rows are k0 + e * kRowsPerPass.  With one or two rows per pass it holds both rows
+    // of every (k, k+2) pair and writes them with one 64-bit store; with four (BMN = 64) it does not.
     static __device__ __forceinline__ void store(float* lds, const float (&r)[NLD], int tid)
     {
         const int m = tid % BMN, k0 = tid / BMN;
+        float* base = lds + LdsTile<BMN>::index(k0, m);
+        constexpr int P = LdsTile<BMN>::kRowPitch;
+        if constexpr (kRowsPerPass == 2) {
 #pragma unroll
-        for (int e = 0; e < NLD; ++e) lds[(k0 + e * kRowsPerPass) * (BMN + kPad) + m] = r[e];
+            for (int e = 0; e < NLD; e += 2)  // k = k0 + 2e and k + 2
+                *reinterpret_cast<floatx2*>(base + (e >> 1) * 2 * P) = floatx2{r[e], r[e + 1]};
+        } else if constexpr (kRowsPerPass == 1) {
+#pragma unroll
+            for (int e = 0; e < NLD; ++e)  // k = e (k0 = 0); pairs (e, e + 2) for e % 4 in {0, 1}
+                if ((e & 2) == 0)
+                    *reinterpret_cast<floatx2*>(base + ((e >> 2) * 2 + (e & 1)) * P) = floatx2{r[e], r[e + 2]};
+        } else {
+            static_assert(kRowsPerPass == 4, "tile extents are 64, 128 or 256");
+#pragma unroll
+            for (int e = 0; e < NLD; ++e) base[e * 2 * P] = r[e];  // k = k0 + 4e
+        }
     }
 };
 
@@ -178,8 +210,9 @@ struct MapK {
     static __device__ __forceinline__ void store(float* lds, const float (&r)[NLD], int tid)
     {
         const int k = tid % BK, m0 = tid / BK;
+        float* base = lds + LdsTile<BMN>::index(k, m0);
 #pragma unroll
-        for (int e = 0; e < NLD; ++e) lds[k * (BMN + kPad) + m0 + e * kMnPerPass] = r[e];
+        for (int e = 0; e < NLD; ++e) base[e * kMnPerPass * 2] = r[e];
     }
 };
 
@@ -646,41 +679,45 @@ __device__ __forceinline__ void load_all(const L& l, const typename L::State& s,
     }
 }
 
-// MFMA operands of k-step J out of LDS buffer BUF: lane (r, h) of a wavefront holds A[m = 32*i + r][k = 2*J + h]
-// and B[k = 2*J + h][n = 32*j + r].  `a_base` / `b_base` are the LDS byte addresses of this lane's element of
-// buffer 0 at J = 0, i = j = 0; everything else is an immediate offset.
-template <class T, int BUF, int J>
-__device__ __forceinline__ void request_operands(uint32_t a_base, uint32_t b_base, float (&af)[T::TM], float (&bf)[T::TN])
+// MFMA operands of the k-steps 2P and 2P+1 out of LDS buffer BUF: lane (r, h) of a wavefront gets
+// A[m = 32*i + r][k = 4P + h] and [k = 4P + 2 + h] in one 64-bit read, likewise B.  `a_base` / `b_base` are the
+// LDS byte addresses of this lane's pair of buffer 0 at P = 0, i = j = 0; everything else is an immediate offset.
+template <class T, int BUF, int P>
+__device__ __forceinline__ void request_operands(uint32_t a_base, uint32_t b_base, floatx2 (&af)[T::TM],
+                                                 floatx2 (&bf)[T::TN])
 {
-    constexpr int a_off = (BUF * BK * (T::BM + kPad) + 2 * J * (T::BM + kPad)) * 4;
-    constexpr int b_off = (BUF * BK * (T::BN + kPad) + 2 * J * (T::BN + kPad)) * 4;
-    if constexpr (T::TM >= 1) af[0] = lds_read<a_off>(a_base);
-    if constexpr (T::TM >= 2) af[1] = lds_read<a_off + 128>(a_base);
-    if constexpr (T::TM >= 3) af[2] = lds_read<a_off + 256>(a_base);
-    if constexpr (T::TM >= 4) af[3] = lds_read<a_off + 384>(a_base);
-    if constexpr (T::TN >= 1) bf[0] = lds_read<b_off>(b_base);
-    if constexpr (T::TN >= 2) bf[1] = lds_read<b_off + 128>(b_base);
-    if constexpr (T::TN >= 3) bf[2] = lds_read<b_off + 256>(b_base);
-    if constexpr (T::TN >= 4) bf[3] = lds_read<b_off + 384>(b_base);
+    constexpr int a_off = (BUF * LdsTile<T::BM>::kFloats + 2 * P * LdsTile<T::BM>::kRowPitch) * 4;
+    constexpr int b_off = (BUF * LdsTile<T::BN>::kFloats + 2 * P * LdsTile<T::BN>::kRowPitch) * 4;
+    if constexpr (T::TM >= 1) af[0] = lds_read2<a_off>(a_base);
+    if constexpr (T::TM >= 2) af[1] = lds_read2<a_off + 256>(a_base);
+    if constexpr (T::TM >= 3) af[2] = lds_read2<a_off + 512>(a_base);
+    if constexpr (T::TM >= 4) af[3] = lds_read2<a_off + 768>(a_base);
+    if constexpr (T::TN >= 1) bf[0] = lds_read2<b_off>(b_base);
+    if constexpr (T::TN >= 2) bf[1] = lds_read2<b_off + 256>(b_base);
+    if constexpr (T::TN >= 3) bf[2] = lds_read2<b_off + 512>(b_base);
+    if constexpr (T::TN >= 4) bf[3] = lds_read2<b_off + 768>(b_base);
     static_assert(T::TM <= 4 && T::TN <= 4, "operand fetch is written for up to 4 blocks per axis");
 }
 
-// One MFMA group (k-step J of the LDS tile) and everything scheduled around it: wait for its operands,
-// start the first MFMA, request the next group's operands, issue this group's share of the global loads,
-// then the remaining MFMAs.
+// One MFMA group (k-step J of the LDS tile) and everything scheduled around it: an even group waits for
+// the operand pair it shares with the next group, starts the first MFMA and requests the following pair;
+// every group issues its share of the global loads, then the remaining MFMAs.
 template <class T, int BUF, int J, class AL, class BL>
 __device__ __forceinline__ void mfma_groups(const AL& al, const BL& bl, const typename AL::State& as,
                                             const typename BL::State& bs, const typename AL::Iter& ai,
                                             const typename BL::Iter& bi, float (&ra)[AL::NLD], float (&rb)[BL::NLD],
                                             uint32_t a_base, uint32_t b_base, floatx16 (&acc)[T::TM][T::TN],
-                                            float (&af)[2][T::TM], float (&bf)[2][T::TN], int knext, int kend)
+                                            floatx2 (&af)[2][T::TM], floatx2 (&bf)[2][T::TN], int knext, int kend)
 {
     constexpr int G = BK / 2;
     if constexpr (J < G) {
-        lds_wait(af[J & 1]);
-        lds_wait(bf[J & 1]);
-        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[J & 1][0], bf[J & 1][0], acc[0][0], 0, 0, 0);
-        if constexpr (J + 1 < G) request_operands<T, BUF, J + 1>(a_base, b_base, af[(J + 1) & 1], bf[(J + 1) & 1]);
+        constexpr int P = J / 2, S = P & 1, H = J & 1;
+        if constexpr (H == 0) {
+            lds_wait(af[S]);
+            lds_wait(bf[S]);
+        }
+        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[S][0][H], bf[S][0][H], acc[0][0], 0, 0, 0);
+        if constexpr (H == 0 && J + 2 < G) request_operands<T, BUF, P + 1>(a_base, b_base, af[S ^ 1], bf[S ^ 1]);
         group_load<J, 0, AL>(al, as, ai, ra, knext, kend);
         group_load<J, 0, BL>(bl, bs, bi, rb, knext, kend);
 #pragma unroll
@@ -688,7 +725,7 @@ __device__ __forceinline__ void mfma_groups(const AL& al, const BL& bl, const ty
 #pragma unroll
             for (int j = 0; j < T::TN; ++j)
                 if (i + j > 0)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[J & 1][i], bf[J & 1][j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[S][i][H], bf[S][j][H], acc[i][j], 0, 0, 0);
         // keep this group's LDS fetches, global loads and MFMAs together: the instruction scheduler
         // must not sink the loads to the end of the step
         __builtin_amdgcn_sched_barrier(0);
@@ -705,7 +742,7 @@ __device__ __forceinline__ void step(const AL& al, const BL& bl, const typename 
 {
     typename AL::Iter ai;
     typename BL::Iter bi;
-    float af[2][T::TM], bf[2][T::TN];
+    floatx2 af[2][T::TM], bf[2][T::TN];
     request_operands<T, BUF, 0>(a_base, b_base, af[0], bf[0]);
     al.begin(as, ai, knext, kend);
     bl.begin(bs, bi, knext, kend);
@@ -798,15 +835,15 @@ __device__ __forceinline__ void operand_bases(const float* As0, const float* Bs0
     const int wave = tid >> 6, lane = tid & 63;
     const int wm0 = (wave % T::WGM) * T::WM, wn0 = (wave / T::WGM) * T::WN;
     const int frag_r = lane & 31, frag_k = lane >> 5;
-    *a_base = lds_addr(&As0[frag_k * (T::BM + kPad) + wm0 + frag_r]);
-    *b_base = lds_addr(&Bs0[frag_k * (T::BN + kPad) + wn0 + frag_r]);
+    *a_base = lds_addr(&As0[LdsTile<T::BM>::index(frag_k, wm0 + frag_r)]);
+    *b_base = lds_addr(&Bs0[LdsTile<T::BN>::index(frag_k, wn0 + frag_r)]);
 }
 
 template <class T, class AL, class BL, class EP>
 __global__ void __launch_bounds__(kThreads) gemm_kernel(AL al, BL bl, EP ep, int tiles_m, SplitInfo si)
 {
-    __shared__ float As[2][BK * (T::BM + kPad)];
-    __shared__ float Bs[2][BK * (T::BN + kPad)];
+    __shared__ __align__(16) float As[2][BK * (T::BM + kPad)];
+    __shared__ __align__(16) float Bs[2][BK * (T::BN + kPad)];
 
     const int tid = threadIdx.x;
     const int tile = xcd_remap(blockIdx.x, gridDim.x);
@@ -870,8 +907,8 @@ __host__ __device__ inline long sk_first_unit(int g, long total_units, int sk_bl
 template <class T, class AL, class BL, class EP>
 __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))) gemm_streamk_kernel(AL al, BL bl, EP ep, int tiles_m, StreamK sk)
 {
-    __shared__ float As[2][BK * (T::BM + kPad)];
-    __shared__ float Bs[2][BK * (T::BN + kPad)];
+    __shared__ __align__(16) float As[2][BK * (T::BM + kPad)];
+    __shared__ __align__(16) float Bs[2][BK * (T::BN + kPad)];
 
     const int tid = threadIdx.x;
     const int g = xcd_remap(blockIdx.x, gridDim.x);
