@@ -28,13 +28,13 @@
 //   * wave-uniform index arithmetic (tap decomposition of a reduction index) is done on the scalar ALU;
 //   * the padding test of an element is one bit-field extract from a per-thread tap mask that is
 //     computed once per tile, and invalid elements get their offset's top bit set with one more op;
-//   * MFMA operands are fetched from LDS with ds_read_b32 and 16-bit immediate offsets from one base
+//   * MFMA operands are fetched from LDS with ds_read_b64 and 16-bit immediate offsets from one base
 //     register per operand (explicit instructions: the compiler would re-add a base per k-step).
 //
-// LDS tiles are kept as [k][m] and [k][n] with rows padded by 4 floats, so that an MFMA operand
-// fetch - lane l reads element (row l%32, k l/32) - is a conflict-free read of 32 consecutive
-// floats per half-wave, and stores from loaders whose lanes run along k (row stride = 4 banks)
-// spread over all banks.
+// LDS tiles are k-major ([k][m] and [k][n], rows padded by 4 floats) with reduction rows k and k+2 of a
+// column interleaved, so that an MFMA operand fetch - lane l needs element (row l%32, k = 2J + l/32) for
+// k-step J - is one conflict-free 64-bit read per two k-steps, stores from loaders whose lanes run
+// along k spread over all banks, and loaders whose lanes run along m / n store two rows at once.
 #pragma once
 #include "common.h"
 
