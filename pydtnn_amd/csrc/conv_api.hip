@@ -79,9 +79,10 @@ inline TileSel pick_tile(long m, long n, long k = 1l << 30)
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 inline long round_up(long v, long m) { return (v + m - 1) / m * m; }
 
-// Target number of workgroups for a launch that has to be split along the reduction axis:
-// four per CU on a 256-CU part.
-constexpr long kTargetBlocks = 1024;
+// Target number of workgroups for a launch that has to be split along the reduction axis: what the
+// chip holds at once (three per CU on a 256-CU part).  A few more would run as a second, nearly
+// empty round, so the split rounds down.
+constexpr long kTargetBlocks = 768;
 constexpr long kMinChunk = 256;
 constexpr size_t kMaxPartialBytes = (size_t)768 << 20;
 
@@ -90,21 +91,26 @@ struct SplitPlan {
     int splits;
 };
 
-// Reduction over `images` segments of `seg` elements (pixels of one image).
+// Reduction over `images` segments of `seg` elements (pixels of one image): equal chunks of the whole
+// run of images where the index arithmetic allows it, else groups of whole images.
 SplitPlan plan_pixel_split(long tiles, int images, int seg, long out_elems)
 {
     const long total = (long)images * seg;
-    long want = tiles >= kTargetBlocks ? 1 : (kTargetBlocks + tiles - 1) / tiles;
+    long want = tiles >= kTargetBlocks ? 1 : kTargetBlocks / tiles;
     const long max_by_ws = (long)(kMaxPartialBytes / ((size_t)out_elems * 4));
     if (want > max_by_ws) want = max_by_ws < 1 ? 1 : max_by_ws;
     long chunk = round_up((total + want - 1) / want, BK);
     if (chunk < kMinChunk) chunk = kMinChunk;
     SplitPlan p;
-    if (chunk >= seg) {
+    // FastDiv by seg must stay exact for every reduction index of a group
+    const long ips_cap = (((1l << 32) - 1) / seg - 256) / seg;
+    if (images <= ips_cap) {
+        const int cpg = (int)((total + chunk - 1) / chunk);
+        p.si = make_split(seg, images, images, cpg, (int)chunk);
+        p.splits = cpg;
+    } else if (chunk >= seg) {
         long ips = chunk / seg;
         if (ips > images) ips = images;
-        // FastDiv by seg must stay exact for every reduction index of a group
-        const long ips_cap = (((1l << 32) - 1) / seg - 256) / seg;
         if (ips > ips_cap) ips = ips_cap < 1 ? 1 : ips_cap;
         p.si = make_split(seg, images, (int)ips, 1, (int)(ips * seg));
         p.splits = (int)((images + ips - 1) / ips);
