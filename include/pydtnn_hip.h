@@ -40,6 +40,12 @@ extern "C" {
 int pydtnn_hip_version(void);
 /* Human-readable text for a status code (static storage). */
 const char *pydtnn_hip_status_string(int status);
+/* One launch addresses a tensor with 32-bit byte offsets: at most 2^29 floats.  The implicit
+ * convolution entry points (sconvGemm*, *_back) run a larger batch as consecutive groups of whole
+ * images, each below that limit; the filter gradient is summed over the groups in order.  For tests
+ * only: lowers the limit (1 .. 2^29 floats) so that small tensors take that route; returns the
+ * previous value.  Process-wide, not synchronised with running calls. */
+long pydtnn_hip_debug_set_tensor_floats_limit(long floats);
 
 /* ------------------------------------------------------------------------------------------
  * Explicit im2col / col2im.  Replace the Cython modules

@@ -12,7 +12,7 @@ int launch_relu_fwd(const float*, float*, int8_t*, long, hipStream_t);
 int launch_relu_bwd(const float*, const int8_t*, float*, long, hipStream_t);
 size_t bias_grad_workspace_floats(long, int);
 int launch_bias_grad(const float*, float*, long, int, int, float*, hipStream_t);
-int launch_splitk_reduce(const float*, float*, long, int, long, int, int, int, const ChanEpilogue&, hipStream_t);
+int launch_splitk_reduce(const float*, float*, long, int, long, int, int, int, const ChanEpilogue&, int, hipStream_t);
 int launch_flip_filter(const float*, float*, int, int, int, int, int, hipStream_t);
 size_t bn_training_workspace_floats(int);
 int launch_bn_training_fwd(const float*, float*, float*, float*, const float*, const float*, float*, float*, float, float,
@@ -102,19 +102,22 @@ SplitPlan plan_pixel_split(long tiles, int images, int seg, long out_elems)
     long chunk = round_up((total + want - 1) / want, BK);
     if (chunk < kMinChunk) chunk = kMinChunk;
     SplitPlan p;
-    // FastDiv by seg must stay exact for every reduction index of a group
+    // A group of several images finds the image of a reduction index with a multiply-high division by
+    // seg, exact while (ips*seg + 256) * seg < 2^32; a group of one image needs no division
+    // (group_div below).
     const long ips_cap = (((1l << 32) - 1) / seg - 256) / seg;
     if (images <= ips_cap) {
         const int cpg = (int)((total + chunk - 1) / chunk);
         p.si = make_split(seg, images, images, cpg, (int)chunk);
         p.splits = cpg;
-    } else if (chunk >= seg) {
+    } else if (chunk >= seg && ips_cap >= 2) {
         long ips = chunk / seg;
         if (ips > images) ips = images;
-        if (ips > ips_cap) ips = ips_cap < 1 ? 1 : ips_cap;
+        if (ips > ips_cap) ips = ips_cap;
         p.si = make_split(seg, images, (int)ips, 1, (int)(ips * seg));
         p.splits = (int)((images + ips - 1) / ips);
     } else {
+        if (chunk > seg) chunk = seg;
         int cpg = (int)((seg + chunk - 1) / chunk);
         chunk = round_up((seg + cpg - 1) / cpg, BK);
         cpg = (int)((seg + chunk - 1) / chunk);
@@ -122,6 +125,15 @@ SplitPlan plan_pixel_split(long tiles, int images, int seg, long out_elems)
         p.splits = images * cpg;
     }
     return p;
+}
+
+// Divider that maps a reduction index of a group to its image: a real one for groups of several
+// images, "always image 0" for groups of one (exact for any image size).
+inline FastDiv group_div(int seg, int ips)
+{
+    if (ips > 1) return make_fastdiv((uint32_t)seg);
+    FastDiv f = {0u, (uint32_t)seg, 0u};
+    return f;
 }
 
 // Plain GEMM: one segment of length k.
@@ -263,7 +275,7 @@ SplitPlan plan_dw(const ConvGeom& g, int nhwc)
 }
 
 int conv_dw_nchw(const ConvGeom& g, const float* dy, const float* x, const float* cols, float* dw, float* ws,
-                 size_t ws_bytes, hipStream_t stream)
+                 size_t ws_bytes, hipStream_t stream, int accumulate = 0)
 {
     const SplitPlan sp = plan_dw(g, 0);
     const long out_elems = (long)g.kn * g.k;
@@ -275,24 +287,27 @@ int conv_dw_nchw(const ConvGeom& g, const float* dy, const float* x, const float
         const long dy_img = (long)g.kn * g.howo;
         if (!span_ok_k(T::BM, g.howo, sp.si.ips, dy_img)) return PYDTNN_HIP_ERR_UNSUPPORTED;
         auto al = plain_k<T::BM, true>(dy, g.p * g.kn, g.howo, dy_img, g.kn, g.howo);
+        al.fd_seg = group_div(g.howo, sp.si.ips);
         const EpiPlain ep = epi_plain(ws, g.k, out_elems, g.kn, g.k, no_epilogue());
         if (cols) {
             // B(k = (image, pixel), n = row of cols) = cols[n][image*howo + pixel]
             if (!span_ok_k(T::BN, g.p, sp.si.ips, g.howo)) return PYDTNN_HIP_ERR_UNSUPPORTED;
             auto bl = plain_k<T::BN, true>(cols, (long)g.k * g.p, g.p, g.howo, g.k, g.howo);
+            bl.fd_seg = group_div(g.howo, sp.si.ips);
             rc = launch<T>(al, bl, ep, g.kn, g.k, sp.si, sp.splits, stream);
         } else {
             Im2colNchwK<T::BN> bl;
             bl.x = x; bl.g = g;
+            bl.g.fd_howo = group_div(g.howo, sp.si.ips);
             rc = launch<T>(al, bl, ep, g.kn, g.k, sp.si, sp.splits, stream);
         }
     })
     if (rc != PYDTNN_HIP_OK) return rc;
-    return launch_splitk_reduce(ws, dw, g.kn, g.k, out_elems, sp.splits, 0, 0, no_epilogue(), stream);
+    return launch_splitk_reduce(ws, dw, g.kn, g.k, out_elems, sp.splits, 0, 0, no_epilogue(), accumulate, stream);
 }
 
 int conv_dw_nhwc(const ConvGeom& g, const float* dy, const float* x, const float* rows, float* dw, float* ws,
-                 size_t ws_bytes, hipStream_t stream)
+                 size_t ws_bytes, hipStream_t stream, int accumulate = 0)
 {
     const SplitPlan sp = plan_dw(g, 1);
     const long out_elems = (long)g.kn * g.k;
@@ -310,13 +325,15 @@ int conv_dw_nhwc(const ConvGeom& g, const float* dy, const float* x, const float
         } else {
             Im2rowNhwcMN<T::BM> al;
             al.x = x; al.g = g;
+            al.g.fd_howo = group_div(g.howo, sp.si.ips);
             rc = launch<T>(al, bl, ep, g.k, g.kn, sp.si, sp.splits, stream);
         }
     })
     if (rc != PYDTNN_HIP_OK) return rc;
     // implicit rows come out in (i, j, c) order; materialised x_rows already has the (c, i, j) order
     const int perm_c = rows ? 0 : g.c;
-    return launch_splitk_reduce(ws, dw, g.k, g.kn, out_elems, sp.splits, perm_c, g.khw, no_epilogue(), stream);
+    return launch_splitk_reduce(ws, dw, g.k, g.kn, out_elems, sp.splits, perm_c, g.khw, no_epilogue(), accumulate,
+                                stream);
 }
 
 // ---------------------------------------------------------------- input gradient
@@ -396,7 +413,7 @@ int geom_from_args(ConvGeom* g, long b, long c, long h, long w, long kn, long kh
 
 int sconv_gemm(int nhwc, char trans, const ConvGeom& g, const float* in1, const float* x, float* out,
                const float* bias, const float* mean, const float* inv_std, const float* gamma, const float* beta,
-               bool relu, void* ws, size_t ws_bytes, hipStream_t stream)
+               bool relu, void* ws, size_t ws_bytes, hipStream_t stream, int accumulate = 0)
 {
     if (!in1 || !x || !out) return PYDTNN_HIP_ERR_INVALID;
     if (trans == 'N') {
@@ -407,15 +424,98 @@ int sconv_gemm(int nhwc, char trans, const ConvGeom& g, const float* in1, const 
     }
     if (trans == 'Y') {
         if (bias || mean || inv_std || gamma || beta || relu) return PYDTNN_HIP_ERR_INVALID;
-        return nhwc ? conv_dw_nhwc(g, in1, x, nullptr, out, (float*)ws, ws_bytes, stream)
-                    : conv_dw_nchw(g, in1, x, nullptr, out, (float*)ws, ws_bytes, stream);
+        return nhwc ? conv_dw_nhwc(g, in1, x, nullptr, out, (float*)ws, ws_bytes, stream, accumulate)
+                    : conv_dw_nchw(g, in1, x, nullptr, out, (float*)ws, ws_bytes, stream, accumulate);
     }
     return PYDTNN_HIP_ERR_INVALID;
+}
+
+#define GEOM_ARGS b, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation
+
+// ---------------------------------------------------------------- batches beyond the addressing limit
+// One launch addresses every tensor through 32-bit byte offsets (fewer than 2^29 floats per tensor).
+// Larger batches are run as consecutive groups of whole images: forward and dX are independent per
+// image; the filter gradient of the second and later groups is added to the first's (in that order).
+long g_tensor_floats_limit = 1l << 29;
+
+struct ImageGroups {
+    long per_image_in, per_image_out;  // floats of x and of y per image
+    long images;                       // images per launch
+};
+
+inline int plan_image_groups(ImageGroups* ig, long b, long c, long h, long w, long kn, long kh, long kw, long vpadding,
+                             long hpadding, long vstride, long hstride, long vdilation, long hdilation)
+{
+    if (b <= 0 || c <= 0 || h <= 0 || w <= 0 || kn <= 0 || kh <= 0 || kw <= 0 || vstride <= 0 || hstride <= 0 ||
+        vdilation <= 0 || hdilation <= 0 || h >= (1l << 20) || w >= (1l << 20) || c >= (1l << 24) || kn >= (1l << 24))
+        return PYDTNN_HIP_ERR_INVALID;
+    const long ho = (h + 2 * vpadding - vdilation * (kh - 1) - 1) / vstride + 1;
+    const long wo = (w + 2 * hpadding - hdilation * (kw - 1) - 1) / hstride + 1;
+    if (ho <= 0 || wo <= 0) return PYDTNN_HIP_ERR_INVALID;
+    ig->per_image_in = c * h * w;
+    ig->per_image_out = kn * ho * wo;
+    const long largest = ig->per_image_in > ig->per_image_out ? ig->per_image_in : ig->per_image_out;
+    long images = (g_tensor_floats_limit - 1) / largest;
+    if (images < 1) images = 1;  // a single image beyond the limit is refused by make_conv_geom
+    ig->images = images < b ? images : b;
+    return PYDTNN_HIP_OK;
+}
+
+int sconv_gemm_batched(int nhwc, char trans, long b, long c, long h, long w, long kn, long kh, long kw, long vpadding,
+                       long hpadding, long vstride, long hstride, long vdilation, long hdilation, const float* in1,
+                       const float* x, float* out, const float* bias, const float* mean, const float* inv_std,
+                       const float* gamma, const float* beta, bool relu, void* ws, size_t ws_bytes, hipStream_t stream)
+{
+    if (!in1 || !x || !out) return PYDTNN_HIP_ERR_INVALID;
+    ImageGroups ig;
+    int rc = plan_image_groups(&ig, GEOM_ARGS);
+    if (rc != PYDTNN_HIP_OK) return rc;
+    for (long n0 = 0; n0 < b; n0 += ig.images) {
+        ConvGeom g;
+        const long nb = b - n0 < ig.images ? b - n0 : ig.images;
+        rc = geom_from_args(&g, nb, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation);
+        if (rc != PYDTNN_HIP_OK) return rc;
+        const float* xg = x + n0 * ig.per_image_in;
+        if (trans == 'Y')  // in1 = dy, out = dw
+            rc = sconv_gemm(nhwc, trans, g, in1 + n0 * ig.per_image_out, xg, out, bias, mean, inv_std, gamma, beta,
+                            relu, ws, ws_bytes, stream, n0 > 0);
+        else               // in1 = weights, out = y
+            rc = sconv_gemm(nhwc, trans, g, in1, xg, out + n0 * ig.per_image_out, bias, mean, inv_std, gamma, beta,
+                            relu, ws, ws_bytes, stream);
+        if (rc != PYDTNN_HIP_OK) return rc;
+    }
+    return PYDTNN_HIP_OK;
+}
+
+int conv_dx_batched(int nhwc, long b, long c, long h, long w, long kn, long kh, long kw, long vpadding, long hpadding,
+                    long vstride, long hstride, long vdilation, long hdilation, const float* weights, const float* dy,
+                    float* dx, float* ws, size_t ws_bytes, hipStream_t stream)
+{
+    if (!weights || !dy || !dx) return PYDTNN_HIP_ERR_INVALID;
+    ImageGroups ig;
+    int rc = plan_image_groups(&ig, GEOM_ARGS);
+    if (rc != PYDTNN_HIP_OK) return rc;
+    for (long n0 = 0; n0 < b; n0 += ig.images) {
+        ConvGeom g;
+        const long nb = b - n0 < ig.images ? b - n0 : ig.images;
+        rc = geom_from_args(&g, nb, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation);
+        if (rc != PYDTNN_HIP_OK) return rc;
+        rc = conv_dx(g, nhwc, weights, dy + n0 * ig.per_image_out, dx + n0 * ig.per_image_in, ws, ws_bytes, stream);
+        if (rc != PYDTNN_HIP_OK) return rc;
+    }
+    return PYDTNN_HIP_OK;
 }
 
 }  // namespace
 
 extern "C" {
+
+long pydtnn_hip_debug_set_tensor_floats_limit(long floats)
+{
+    const long before = g_tensor_floats_limit;
+    if (floats > 0 && floats <= (1l << 29)) g_tensor_floats_limit = floats;
+    return before;
+}
 
 int pydtnn_hip_version(void) { return 10000 * 0 + 100 * 1 + 0; }
 
@@ -431,7 +531,6 @@ const char* pydtnn_hip_status_string(int status)
     }
 }
 
-#define GEOM_ARGS b, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation
 
 int pydtnn_hip_im2col_nchw(const float* x, float* cols, int b, int c, int h, int w, int kh, int kw, int vpadding,
                            int hpadding, int vstride, int hstride, int vdilation, int hdilation, void* stream)
@@ -527,7 +626,7 @@ int pydtnn_hip_sgemm(int transa, int transb, long m, long n, long k, const float
     })
     if (rc != PYDTNN_HIP_OK || sp.splits == 1) return rc;
     if (ldc != n) return PYDTNN_HIP_ERR_UNSUPPORTED;  // the split reduction writes a dense C
-    return launch_splitk_reduce((const float*)workspace, c, m, (int)n, m * n, sp.splits, 0, 0, chan, st);
+    return launch_splitk_reduce((const float*)workspace, c, m, (int)n, m * n, sp.splits, 0, 0, chan, 0, st);
 }
 
 // ---------------------------------------------------------------- convolution
@@ -535,8 +634,14 @@ size_t pydtnn_hip_conv_workspace_bytes(int op, int nhwc, int b, int c, int h, in
                                        int vpadding, int hpadding, int vstride, int hstride, int vdilation,
                                        int hdilation)
 {
+    // the implicit routes run a large batch as groups of images: their workspace is that of one group
     ConvGeom g;
-    if (geom_from_args(&g, GEOM_ARGS) != PYDTNN_HIP_OK) return 0;
+    ImageGroups ig;
+    long nb = b;
+    if (op != PYDTNN_HIP_OP_DX_I2C && plan_image_groups(&ig, GEOM_ARGS) == PYDTNN_HIP_OK) nb = ig.images;
+    if (geom_from_args(&g, nb, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation) !=
+        PYDTNN_HIP_OK)
+        return 0;
     switch (op) {
         case PYDTNN_HIP_OP_DW: return (size_t)plan_dw(g, nhwc).splits * g.kn * g.k * 4;
         case PYDTNN_HIP_OP_FWD: return kBalanceBytes;  // optional: a smaller or absent workspace only costs speed
@@ -556,11 +661,8 @@ int pydtnn_hip_sconvGemmNCHW(char trans, unsigned b, unsigned c, unsigned h, uns
                              const float* bn_gamma, const float* bn_beta, bool relu, void* workspace,
                              size_t workspace_bytes, void* stream)
 {
-    ConvGeom g;
-    const int rc = geom_from_args(&g, GEOM_ARGS);
-    if (rc != PYDTNN_HIP_OK) return rc;
-    return sconv_gemm(0, trans, g, in1, x, out, bias_vector, bn_running_mean, bn_inv_std, bn_gamma, bn_beta, relu,
-                      workspace, workspace_bytes, as_stream(stream));
+    return sconv_gemm_batched(0, trans, GEOM_ARGS, in1, x, out, bias_vector, bn_running_mean, bn_inv_std, bn_gamma,
+                              bn_beta, relu, workspace, workspace_bytes, as_stream(stream));
 }
 
 int pydtnn_hip_sconvGemmNHWC(char trans, unsigned b, unsigned h, unsigned w, unsigned c, unsigned kn, unsigned kh,
@@ -570,11 +672,8 @@ int pydtnn_hip_sconvGemmNHWC(char trans, unsigned b, unsigned h, unsigned w, uns
                              const float* bn_gamma, const float* bn_beta, bool relu, void* workspace,
                              size_t workspace_bytes, void* stream)
 {
-    ConvGeom g;
-    const int rc = geom_from_args(&g, GEOM_ARGS);
-    if (rc != PYDTNN_HIP_OK) return rc;
-    return sconv_gemm(1, trans, g, in1, x, out, bias_vector, bn_running_mean, bn_inv_std, bn_gamma, bn_beta, relu,
-                      workspace, workspace_bytes, as_stream(stream));
+    return sconv_gemm_batched(1, trans, GEOM_ARGS, in1, x, out, bias_vector, bn_running_mean, bn_inv_std, bn_gamma,
+                              bn_beta, relu, workspace, workspace_bytes, as_stream(stream));
 }
 
 int pydtnn_hip_sconvGemmNCHW_back(unsigned b, unsigned c, unsigned h, unsigned w, unsigned kn, unsigned kh,
@@ -582,11 +681,7 @@ int pydtnn_hip_sconvGemmNCHW_back(unsigned b, unsigned c, unsigned h, unsigned w
                                   unsigned hpadding, unsigned vdilation, unsigned hdilation, const float* weights,
                                   const float* dy, float* dx, void* workspace, size_t workspace_bytes, void* stream)
 {
-    if (!weights || !dy || !dx) return PYDTNN_HIP_ERR_INVALID;
-    ConvGeom g;
-    const int rc = geom_from_args(&g, GEOM_ARGS);
-    if (rc != PYDTNN_HIP_OK) return rc;
-    return conv_dx(g, 0, weights, dy, dx, (float*)workspace, workspace_bytes, as_stream(stream));
+    return conv_dx_batched(0, GEOM_ARGS, weights, dy, dx, (float*)workspace, workspace_bytes, as_stream(stream));
 }
 
 int pydtnn_hip_sconvGemmNHWC_back(unsigned b, unsigned h, unsigned w, unsigned c, unsigned kn, unsigned kh,
@@ -594,11 +689,7 @@ int pydtnn_hip_sconvGemmNHWC_back(unsigned b, unsigned h, unsigned w, unsigned c
                                   unsigned hpadding, unsigned vdilation, unsigned hdilation, const float* weights,
                                   const float* dy, float* dx, void* workspace, size_t workspace_bytes, void* stream)
 {
-    if (!weights || !dy || !dx) return PYDTNN_HIP_ERR_INVALID;
-    ConvGeom g;
-    const int rc = geom_from_args(&g, GEOM_ARGS);
-    if (rc != PYDTNN_HIP_OK) return rc;
-    return conv_dx(g, 1, weights, dy, dx, (float*)workspace, workspace_bytes, as_stream(stream));
+    return conv_dx_batched(1, GEOM_ARGS, weights, dy, dx, (float*)workspace, workspace_bytes, as_stream(stream));
 }
 
 // ---------------------------------------------------------------- explicit (i2c) GEMM steps

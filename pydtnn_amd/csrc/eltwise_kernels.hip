@@ -176,13 +176,14 @@ __global__ void __launch_bounds__(kThreads) bias_grad_stage2(const float* __rest
 }
 
 // ---------------------------------------------------------------- split-K reduction
-// out[map(r, col)] = epilogue(col, sum_s partial[s*stride + r*ncols + col]).
+// out[map(r, col)] = epilogue(col, sum_s partial[s*stride + r*ncols + col]), or with `accumulate` that value
+// added to what out already holds (a filter gradient built up over several launches).
 // perm_c > 0 re-orders rows from the kernels' internal (i, j, c) order to the reference's
 // (c, i, j) weight rows: r = ij*perm_c + c  ->  c*khw + ij.
 __global__ void __launch_bounds__(kThreads) splitk_reduce_kernel(const float* __restrict__ partial,
                                                                 float* __restrict__ out, long total, long stride,
                                                                 int slices, int ncols, int perm_c, int khw,
-                                                                ChanEpilogue epi)
+                                                                ChanEpilogue epi, int accumulate)
 {
     const long idx = (long)blockIdx.x * kThreads + threadIdx.x;
     if (idx >= total) return;
@@ -195,7 +196,8 @@ __global__ void __launch_bounds__(kThreads) splitk_reduce_kernel(const float* __
         const long cc = r - ij * perm_c;
         r = cc * khw + ij;
     }
-    out[r * ncols + col] = chan_epilogue_apply(epi, col, acc);
+    const float v = chan_epilogue_apply(epi, col, acc);
+    out[r * ncols + col] = accumulate ? out[r * ncols + col] + v : v;
 }
 
 // ---------------------------------------------------------------- filter re-layouts for dX
@@ -802,12 +804,12 @@ int launch_bias_grad(const float* dy, float* db, long outer, int channels, int i
 }
 
 int launch_splitk_reduce(const float* partial, float* out, long rows, int ncols, long stride, int slices, int perm_c,
-                         int khw, const ChanEpilogue& epi, hipStream_t stream)
+                         int khw, const ChanEpilogue& epi, int accumulate, hipStream_t stream)
 {
     const long total = rows * ncols;
     if (total <= 0 || slices <= 0) return PYDTNN_HIP_ERR_INVALID;
     hipLaunchKernelGGL(splitk_reduce_kernel, dim3(blocks_for(total)), dim3(kThreads), 0, stream, partial, out, total,
-                       stride, slices, ncols, perm_c, khw, epi);
+                       stride, slices, ncols, perm_c, khw, epi, accumulate);
     HIP_RETURN_IF_LAUNCH_FAILED();
     return PYDTNN_HIP_OK;
 }

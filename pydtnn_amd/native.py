@@ -25,6 +25,7 @@ _geom13_u = [_c.c_uint] * 13
 SIGNATURES = {
     "pydtnn_hip_version": (_c.c_int, []),
     "pydtnn_hip_status_string": (_c.c_char_p, [_c.c_int]),
+    "pydtnn_hip_debug_set_tensor_floats_limit": (_c.c_long, [_c.c_long]),
     "pydtnn_hip_im2col_nchw": (_c.c_int, [_f32p, _f32p] + [_c.c_int] * 12 + [_vp]),
     "pydtnn_hip_col2im_nchw": (_c.c_int, [_f32p, _f32p] + [_c.c_int] * 12 + [_vp]),
     "pydtnn_hip_im2row_nhwc": (_c.c_int, [_f32p, _f32p] + [_c.c_int] * 12 + [_vp]),

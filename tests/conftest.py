@@ -21,3 +21,18 @@ def oracle():
         subprocess.check_call(["make", "-C", os.path.join(ROOT, "oracle")])
     from oracle import cpu_ref
     return cpu_ref
+
+
+@pytest.fixture(scope="session")
+def hand_cases():
+    """Committed known answers for the literal arrays of the reference's convolution tests
+    (tests/golden/reference_hand_cases.json, written by tests/golden/make_hand_cases.py)."""
+    import json
+    import numpy as np
+    with open(os.path.join(ROOT, "tests", "golden", "reference_hand_cases.json")) as f:
+        data = json.load(f)
+    for case in data["cases"]:
+        for key in ("x", "w", "y", "bias_matrix", "y_plus_bias_matrix"):
+            if key in case:
+                case[key] = np.array(case[key], dtype=np.float32)
+    return data["cases"]

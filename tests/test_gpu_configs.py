@@ -108,6 +108,59 @@ def test_cfg2_full_size_sampled_direct_convolution(pd):
         rel_err(y2 - b[None, :, None, None], 2 * (y - b[None, :, None, None])) < 1e-6
 
 
+# ------------------------------------------------------------------ tensors beyond 2^29 floats
+
+def test_tensors_beyond_the_per_launch_limit(pd):
+    """x, y, dy and dx of 40 x 64 x 460 x 460 = 541.7 M floats each (2.17 GB) exceed what one launch can address, so
+    the entry points run the batch as groups of images.  Checked by sampled direct convolution in float64."""
+    announce("beyond 2^29 floats")
+    n, c, hw, kn = 40, 64, 460, 64
+    assert n * c * hw * hw > 2 ** 29
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    xd = torch.randn((n, c, hw, hw), device="cuda", generator=gen)
+    dyd = torch.randn((n, kn, hw, hw), device="cuda", generator=gen)
+    w = (np.random.default_rng(4).standard_normal((kn, c, 3, 3)) * np.sqrt(2.0 / (c * 9))).astype(np.float32)
+    wd = dev(w)
+    cg = pd.ConvGemm()
+    y = host(cg.conv_gemm_nchw(wd, xd, vpadding=1, hpadding=1))
+    dwd = torch.empty_like(wd)
+    cg.conv_gemm_nchw(dyd, xd, biases=dwd, trans=True, vpadding=1, hpadding=1)
+    dxd = torch.empty_like(xd)
+    cg.deconv_gemm_nchw(wd, dyd, dxd, vpadding=1, hpadding=1)
+    x, dy, dw = host(xd), host(dyd), host(dwd)
+    del xd, dyd
+    rng = np.random.default_rng(5)
+    s = 1500
+    ni, oy, ox = rng.integers(0, n, s), rng.integers(0, hw, s), rng.integers(0, hw, s)
+    ni[:8] = n - 1                     # the last image group
+    co, cc = rng.integers(0, kn, s), rng.integers(0, c, s)
+
+    def taps(t, ch_axis_len, flip):
+        """(s, channels, 9) patches of t around (oy, ox), zero outside the image; flip mirrors the taps."""
+        out = np.zeros((s, ch_axis_len, 9))
+        for i in range(3):
+            for j in range(3):
+                yy, xx = (oy + 1 - i, ox + 1 - j) if flip else (oy + i - 1, ox + j - 1)
+                ok = (yy >= 0) & (yy < hw) & (xx >= 0) & (xx < hw)
+                out[ok, :, i * 3 + j] = t[ni[ok], :, yy[ok], xx[ok]]
+        return out
+
+    ref_y = np.einsum("sck,sck->s", taps(x, c, False), w[co].reshape(s, c, 9).astype(np.float64))
+    assert np.max(np.abs(y[ni, co, oy, ox] - ref_y)) / np.abs(y).max() <= FP32_REL_TOL
+    del y
+    dx = host(dxd)
+    del dxd
+    ref_dx = np.einsum("sok,sok->s", taps(dy, kn, True), w[:, cc].transpose(1, 0, 2, 3).reshape(s, kn, 9).astype(np.float64))
+    assert np.max(np.abs(dx[ni, cc, oy, ox] - ref_dx)) / np.abs(dx).max() <= FP32_REL_TOL
+    del dx
+    for _ in range(6):
+        o, ci, i, j = rng.integers(0, kn), rng.integers(0, c), rng.integers(0, 3), rng.integers(0, 3)
+        ys, ye = max(0, 1 - i), min(hw, hw + 1 - i)        # output rows whose tap (i, j) lies inside the image
+        xs, xe = max(0, 1 - j), min(hw, hw + 1 - j)
+        ref = np.sum(dy[:, o, ys:ye, xs:xe].astype(np.float64) * x[:, ci, ys + i - 1:ye + i - 1, xs + j - 1:xe + j - 1])
+        assert abs(dw[o, ci, i, j] - ref) / np.abs(dw).max() <= FP32_REL_TOL
+
+
 # ------------------------------------------------------------------ VGG16, layer by layer
 
 def test_vgg16_step_layer_by_layer_against_oracle(pd, oracle):

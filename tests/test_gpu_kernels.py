@@ -468,6 +468,83 @@ def test_categorical_cross_entropy(ops, oracle, rows, cols):
     np.testing.assert_allclose(host(dx), dx_ref, rtol=2e-6, atol=0)
 
 
+# ------------------------------------------------------------------ images of more than 2^16 pixels
+
+@pytest.mark.parametrize("fmt", ["NCHW", "NHWC"])
+def test_images_larger_than_65536_pixels(oracle, fmt):
+    """300 x 300 output pixels per image: a reduction index of the filter gradient no longer fits the
+    multiply-high division by the image size, so the split must keep one image per group."""
+    from pydtnn_amd.conv_gemm import ConvGemm
+    d = D(3, 6, 300, 300, 8, 3, 3, 1, 1, 1, 1)
+    announce("large images", fmt, d)
+    x, w, b, dy = case(d)
+    cg = ConvGemm()
+    p = oracle.ConvParams(*d.geom())
+    kw = dict(vpadding=1, hpadding=1)
+    if fmt == "NCHW":
+        y = cg.conv_gemm_nchw(dev(w), dev(x), biases_vector=dev(b), **kw)
+        dw = torch.empty_like(dev(w))
+        cg.conv_gemm_nchw(dev(dy), dev(x), biases=dw, trans=True, **kw)
+        dx = torch.empty_like(dev(x))
+        cg.deconv_gemm_nchw(dev(w), dev(dy), dx, **kw)
+        y_ref, cols = oracle.conv2d_forward_nchw_i2c(x, w, b, p)
+        dw_ref, _, dx_ref = oracle.conv2d_backward_nchw_i2c(dy, cols, w, x.shape, p)
+    else:
+        xr, wr, dyr = nhwc(x), w_nhwc(w), nhwc(dy)
+        y = cg.conv_gemm_nhwc(dev(wr), dev(xr), biases_vector=dev(b), **kw)
+        dw = torch.empty_like(dev(wr))
+        cg.conv_gemm_nhwc(dev(dyr), dev(xr), biases=dw, trans=True, **kw)
+        dx = torch.empty_like(dev(xr))
+        cg.deconv_gemm_nhwc(dev(wr), dev(dyr), dx, **kw)
+        y_ref, rows = oracle.conv2d_forward_nhwc_i2c(xr, wr, b, p)
+        dw_ref, _, dx_ref = oracle.conv2d_backward_nhwc_i2c(dyr, rows, wr, xr.shape, p)
+    assert_close(host(y), y_ref, what="y")
+    assert_close(host(dw), dw_ref, what="dw")
+    assert_close(host(dx), dx_ref, what="dx")
+
+
+# ------------------------------------------------------------------ batches run as groups of images
+
+@pytest.mark.parametrize("d", [D(7, 5, 12, 11, 6, 3, 3, 1, 1, 2, 1), D(8, 4, 9, 10, 8, 3, 3, 1, 1, 1, 1)], ids=repr)
+@pytest.mark.parametrize("fmt", ["NCHW", "NHWC"])
+def test_large_batches_run_as_image_groups(oracle, fmt, d):
+    """With the per-launch tensor limit lowered, forward / dW / dX of a batch run as groups of 3 images (3, 3, 1
+    or 3, 3, 2); results must equal the oracle's (dW is summed over the groups)."""
+    from pydtnn_amd import native
+    from pydtnn_amd.conv_gemm import ConvGemm
+    announce("image groups", fmt, d)
+    x, w, b, dy = case(d)
+    per_image = max(d.c * d.h * d.w, d.kn * d.ho * d.wo)
+    lib = native.lib()
+    before = lib.pydtnn_hip_debug_set_tensor_floats_limit(3 * per_image + 1)
+    try:
+        cg = ConvGemm()
+        p = oracle.ConvParams(*d.geom())
+        kw = dict(vpadding=d.vpadding, hpadding=d.hpadding, vstride=d.vstride, hstride=d.hstride)
+        if fmt == "NCHW":
+            y = cg.conv_gemm_nchw(dev(w), dev(x), biases_vector=dev(b), **kw)
+            dw = torch.empty_like(dev(w))
+            cg.conv_gemm_nchw(dev(dy), dev(x), biases=dw, trans=True, **kw)
+            dx = torch.empty_like(dev(x))
+            cg.deconv_gemm_nchw(dev(w), dev(dy), dx, **kw)
+            y_ref, cols = oracle.conv2d_forward_nchw_i2c(x, w, b, p)
+            dw_ref, _, dx_ref = oracle.conv2d_backward_nchw_i2c(dy, cols, w, x.shape, p)
+        else:
+            xr, wr, dyr = nhwc(x), w_nhwc(w), nhwc(dy)
+            y = cg.conv_gemm_nhwc(dev(wr), dev(xr), biases_vector=dev(b), **kw)
+            dw = torch.empty_like(dev(wr))
+            cg.conv_gemm_nhwc(dev(dyr), dev(xr), biases=dw, trans=True, **kw)
+            dx = torch.empty_like(dev(xr))
+            cg.deconv_gemm_nhwc(dev(wr), dev(dyr), dx, **kw)
+            y_ref, rows = oracle.conv2d_forward_nhwc_i2c(xr, wr, b, p)
+            dw_ref, _, dx_ref = oracle.conv2d_backward_nhwc_i2c(dyr, rows, wr, xr.shape, p)
+        assert_close(host(y), y_ref, what="y")
+        assert_close(host(dw), dw_ref, what="dw")
+        assert_close(host(dx), dx_ref, what="dx")
+    finally:
+        lib.pydtnn_hip_debug_set_tensor_floats_limit(before)
+
+
 # ------------------------------------------------------------------ host-pointer compatibility ABI
 
 def test_libconvgemm_compat_abi_runs_like_the_reference_shim(oracle):

@@ -412,3 +412,27 @@ def test_store_and_load_weights_use_the_reference_key_names(pd, tmp_path):
     assert b.layers[2].updated_running_var
     x = dev(np.random.default_rng(0).standard_normal((2, 8, 8, 3)).astype(np.float32))
     assert np.array_equal(host(a.evaluate_batch(x)), host(b.evaluate_batch(x)))
+
+
+# ------------------------------------------------------------------ committed known answers
+
+@pytest.mark.parametrize("variant", ["i2c", "cg"])
+@pytest.mark.parametrize("fmt", ["NCHW", "NHWC"])
+def test_committed_hand_cases_through_the_layer(pd, hand_cases, fmt, variant):
+    """Every conv variant against tests/golden/reference_hand_cases.json: small integers, so the GPU result
+    must be exact."""
+    for case in hand_cases:
+        announce("hand case", fmt, variant, case["name"])
+        x, w = case["x"], case["w"]
+        d = D(x.shape[0], x.shape[1], x.shape[2], x.shape[3], w.shape[0], w.shape[2], w.shape[3],
+              case["vpadding"], case["hpadding"], case["vstride"], case["hstride"], case["vdilation"],
+              case["hdilation"])
+        model, layer = make_conv(pd, d, fmt, variant, use_bias=False)
+        model.mode = pd.EVALUATE_MODE
+        if fmt == "NCHW":
+            layer.weights = dev(w)
+            y = host(layer.forward(dev(x)))
+        else:
+            layer.weights = dev(np.ascontiguousarray(w.transpose(1, 2, 3, 0)))
+            y = host(layer.forward(dev(nhwc(x)))).transpose(0, 3, 1, 2)
+        assert np.array_equal(y, case["y"]), (case["name"], y, case["y"])

@@ -179,6 +179,23 @@ def test_known_answers_from_reference_hand_arrays(oracle):
     assert y2.ravel()[0] == 1 + 4 + 48 + 128 + 512 + 1280 + 12288 + 28672
 
 
+def test_committed_hand_cases(oracle, hand_cases):
+    """The oracle's forward routes (NCHW and NHWC) against the committed known answers."""
+    assert len(hand_cases) == 10
+    for case in hand_cases:
+        x, w = case["x"], case["w"]
+        p = oracle.ConvParams(w.shape[2], w.shape[3], case["vpadding"], case["hpadding"], case["vstride"],
+                              case["hstride"], case["vdilation"], case["hdilation"])
+        zero = np.zeros(w.shape[0], np.float32)
+        y, _ = oracle.conv2d_forward_nchw_i2c(x, w, zero, p)
+        assert np.array_equal(y, case["y"]), case["name"]
+        yh, _ = oracle.conv2d_forward_nhwc_i2c(np.ascontiguousarray(x.transpose(0, 2, 3, 1)),
+                                               np.ascontiguousarray(w.transpose(1, 2, 3, 0)), zero, p)
+        assert np.array_equal(yh.transpose(0, 3, 1, 2), case["y"]), case["name"]
+        if "bias_matrix" in case:
+            assert np.array_equal(y + case["bias_matrix"], case["y_plus_bias_matrix"])
+
+
 def test_default_D_ones_interior_and_border(oracle):
     """ones(1,1,128,100) (*) ones(16x10), pad 1: 160 inside, fewer by the clipped taps at the border."""
     d = D()
