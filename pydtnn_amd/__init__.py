@@ -9,6 +9,8 @@ from .layers import (EVALUATE_MODE, TRAIN_MODE, UNSPECIFIED_MODE, AdditionBlock,
                      BatchNormalizationRelu, Conv2D, Conv2DBatchNormalization, Conv2DBatchNormalizationRelu,
                      Conv2DRelu, Dropout, FC, Flatten, Input, Layer, MaxPool2D, Relu, Softmax)
 from .model import SGD, CategoricalCrossEntropy, Model
+from . import tracers
+from .best_of import BestOf
 from .conv_gemm import ConvGemm
 from .utils import (PYDTNN_TENSOR_FORMAT_NCHW, PYDTNN_TENSOR_FORMAT_NHWC, decode_tensor, encode_tensor, to_device,
                     to_host)

@@ -14,6 +14,8 @@ import numpy as np
 import torch
 
 from . import ops
+from .best_of import BestOf
+from . import tracers as ev
 from .conv_gemm import ConvGemm
 from .utils import PYDTNN_TENSOR_FORMAT_NCHW, decode_tensor, encode_tensor
 
@@ -89,6 +91,26 @@ class Layer:
     @property
     def canonical_name(self):
         return type(self).__name__
+
+    @property
+    def _id_prefix(self):
+        """pydtnn/layers/layer_and_activation_base.py:46-60: the id padded to the width of the model's last id."""
+        model = getattr(self, "model", None)
+        if self.id is None or model is None:
+            return ""
+        try:
+            last = model.layers[-1]
+        except IndexError:
+            width = 1
+        else:
+            last_id = last.children[-1].id if len(last.children) else last.id
+            width = len(str(last_id))
+        return "{:0{width}d}_".format(self.id, width=width)
+
+    @property
+    def canonical_name_with_id(self):
+        """pydtnn/layers/layer.py:32-34"""
+        return f"{self._id_prefix}{self.canonical_name}"
 
     def __repr__(self):
         return f"{self.id if self.id is not None else '?'}_{type(self).__name__}"
@@ -240,6 +262,22 @@ class Conv2D(Layer):
         if self.model.enable_conv_gemm:
             self.cg = ConvGemm(dtype=self.model.dtype, debug=self.debug, parent_layer=self)
         variant = "cg" if self.model.enable_conv_gemm else "i2c"  # conv_2d_cpu.py:89, :139-140
+        if getattr(self.model, "enable_best_of", False):
+            # conv_2d_cpu.py:95-130: the explicit and the implicit route race per problem size, forward alone
+            # in EVALUATE_MODE and as a forward + backward pipeline in TRAIN_MODE
+            variant = "best_of"
+            if self.cg is None:
+                self.cg = ConvGemm(dtype=self.model.dtype, debug=self.debug, parent_layer=self)
+            pairs = [(v, self._get_class_forward_and_backward(v)) for v in ("i2c", "cg")]
+
+            def problem_size(*args):
+                return tuple(list(args[0].shape) + list(args[0].weights.shape))
+
+            self._best_fw = BestOf(name="Conv2D only forward", alternatives=[(v, fb[0]) for v, fb in pairs],
+                                   get_problem_size=problem_size)
+            self._best_fw_bw_pipeline = BestOf(name="Conv2D forward backward",
+                                               alternatives=[(v, list(fb)) for v, fb in pairs],
+                                               get_problem_size=problem_size)
         forward, backward = self._get_forward_and_backward(variant)
         setattr(self, "forward", forward)
         setattr(self, "backward", backward)
@@ -248,6 +286,32 @@ class Conv2D(Layer):
         tensor_format = "nchw" if self.model.tensor_format == PYDTNN_TENSOR_FORMAT_NCHW else "nhwc"
         return (getattr(self, f"_forward_{tensor_format}_{variant}"),
                 getattr(self, f"_backward_{tensor_format}_{variant}"))
+
+    def _get_class_forward_and_backward(self, variant):
+        """Unbound functions, called as f(layer, x) (conv_2d_cpu.py:165-181)."""
+        tensor_format = "nchw" if self.model.tensor_format == PYDTNN_TENSOR_FORMAT_NCHW else "nhwc"
+        return (getattr(type(self), f"_forward_{tensor_format}_{variant}"),
+                getattr(type(self), f"_backward_{tensor_format}_{variant}"))
+
+    def _fw_bw_best_of(self, stage, x_or_y):
+        """conv_2d_cpu.py:251-259"""
+        if self.model.mode == TRAIN_MODE:
+            return self._best_fw_bw_pipeline(stage, self, x_or_y)
+        if self.model.mode == EVALUATE_MODE:
+            return self._best_fw(self, x_or_y)
+        raise RuntimeError("Conv2D BestOf variant requires Model.mode to be set to EVALUATE_MODE or TRAIN_MODE")
+
+    def _forward_nchw_best_of(self, x):
+        return self._fw_bw_best_of(0, x)
+
+    def _forward_nhwc_best_of(self, x):
+        return self._fw_bw_best_of(0, x)
+
+    def _backward_nchw_best_of(self, dy):
+        return self._fw_bw_best_of(1, dy)
+
+    def _backward_nhwc_best_of(self, dy):
+        return self._fw_bw_best_of(1, dy)
 
     def _geom(self):
         return (self.kh, self.kw, self.vpadding, self.hpadding, self.vstride, self.hstride,
@@ -261,64 +325,102 @@ class Conv2D(Layer):
         return dict(vpadding=self.vpadding, hpadding=self.hpadding, vstride=self.vstride, hstride=self.hstride,
                     vdilation=self.vdilation, hdilation=self.hdilation)
 
+    def _op(self, kind):
+        """Opens the operation event `kind` of this layer (closed by _end)."""
+        self.model.tracer.emit_event(ev.PYDTNN_OPS_EVENT, self.id * ev.PYDTNN_OPS_EVENTS + kind)
+
+    def _end(self):
+        self.model.tracer.emit_event(ev.PYDTNN_OPS_EVENT, 0)
+
     # ---------------------------------------------------------------- i2c, NHWC (conv_2d_cpu.py:183-209, :363-397)
     def _forward_nhwc_i2c(self, x):
+        self._op(ev.PYDTNN_OPS_FORWARD_IM2COL)
         x_rows = ops.im2row_nhwc(x, *self._geom())
+        self._end()
         if self.model.mode == TRAIN_MODE:
             self.x_rows = x_rows
         y = torch.empty((x.shape[0], self.ho, self.wo, self.co), dtype=x.dtype, device=x.device)
         # matmul + add_nhwc_cython fused: the bias is added in the GEMM's store
+        self._op(ev.PYDTNN_OPS_FORWARD_MATMUL)
         ops.conv_i2c_forward(True, self._geom13(x.shape[0]), self.weights, x_rows, y,
                              self.biases if self.use_bias else None)
+        self._end()
         return y
 
     def _backward_nhwc_i2c(self, dy):
         b = dy.shape[0]
         self.dw = torch.empty_like(self.weights)
+        self._op(ev.PYDTNN_OPS_COMP_DW_MATMUL)
         ops.conv_i2c_dw(True, self._geom13(b), dy, self.x_rows, self.dw)
+        self._end()
         if self.use_bias:
+            self._op(ev.PYDTNN_OPS_BACKWARD_SUM_BIASES)
             self.db = ops.bias_grad(dy, self.co, 1)
+            self._end()
         if self.need_dx:
             dx = torch.empty((b, self.hi, self.wi, self.ci), dtype=dy.dtype, device=dy.device)
-            return ops.conv_i2c_dx(True, self._geom13(b), self.weights, dy, dx)
+            self._op(ev.PYDTNN_OPS_COMP_DX_MATMUL)  # the GEMM and row2im of the explicit route
+            ops.conv_i2c_dx(True, self._geom13(b), self.weights, dy, dx)
+            self._end()
+            return dx
 
     # ---------------------------------------------------------------- i2c, NCHW (conv_2d_cpu.py:264-291, :447-481)
     def _forward_nchw_i2c(self, x):
+        self._op(ev.PYDTNN_OPS_FORWARD_IM2COL)
         x_cols = ops.im2col_nchw(x, *self._geom())
+        self._end()
         if self.model.mode == TRAIN_MODE:
             self.x_cols = x_cols
         y = torch.empty((x.shape[0], self.co, self.ho, self.wo), dtype=x.dtype, device=x.device)
         # matmul + add_nchw_cython + best_transpose_1023 fused into the GEMM's store
+        self._op(ev.PYDTNN_OPS_FORWARD_MATMUL)
         ops.conv_i2c_forward(False, self._geom13(x.shape[0]), self.weights, x_cols, y,
                              self.biases if self.use_bias else None)
+        self._end()
         return y
 
     def _backward_nchw_i2c(self, dy):
         b = dy.shape[0]
         self.dw = torch.empty_like(self.weights)
+        self._op(ev.PYDTNN_OPS_COMP_DW_MATMUL)
         ops.conv_i2c_dw(False, self._geom13(b), dy, self.x_cols, self.dw)
+        self._end()
         if self.use_bias:
+            self._op(ev.PYDTNN_OPS_BACKWARD_SUM_BIASES)
             self.db = ops.bias_grad(dy, self.co, self.ho * self.wo)
+            self._end()
         if self.need_dx:
             dx = torch.empty((b, self.ci, self.hi, self.wi), dtype=dy.dtype, device=dy.device)
-            return ops.conv_i2c_dx(False, self._geom13(b), self.weights, dy, dx)
+            self._op(ev.PYDTNN_OPS_COMP_DX_MATMUL)  # the GEMM and col2im of the explicit route
+            ops.conv_i2c_dx(False, self._geom13(b), self.weights, dy, dx)
+            self._end()
+            return dx
 
     # ---------------------------------------------------------------- cg, NHWC (conv_2d_cpu.py:211-227, :399-427)
     def _forward_nhwc_cg(self, x):
         if self.model.mode == TRAIN_MODE:
             self.cg_x = x
         biases_vector = self.biases if self.use_bias else None
-        return self.cg.conv_gemm_nhwc(self.weights, x, biases_vector=biases_vector, **self._cg_kwargs())
+        self._op(ev.PYDTNN_OPS_FORWARD_CONVGEMM)
+        y = self.cg.conv_gemm_nhwc(self.weights, x, biases_vector=biases_vector, **self._cg_kwargs())
+        self._end()
+        return y
 
     def _backward_nhwc_cg(self, dy):
         res = torch.empty(self.weights.shape, dtype=dy.dtype, device=dy.device)
+        self._op(ev.PYDTNN_OPS_BACKWARD_CONVGEMM)
         self.cg.conv_gemm_nhwc(dy, self.cg_x, biases=res, trans=True, **self._cg_kwargs())
+        self._end()
         self.dw = res
         if self.use_bias:
+            self._op(ev.PYDTNN_OPS_BACKWARD_SUM_BIASES)
             self.db = ops.bias_grad(dy, self.co, 1)
+            self._end()
         if self.need_dx:
             dx = torch.empty((dy.shape[0], self.hi, self.wi, self.ci), dtype=dy.dtype, device=dy.device)
+            self._op(ev.PYDTNN_OPS_BACKWARD_DECONV_GEMM)
             self.cg.deconv_gemm_nhwc(self.weights, dy, dx, **self._cg_kwargs())
+            self._end()
             return dx
 
     # ---------------------------------------------------------------- cg, NCHW (conv_2d_cpu.py:293-308, :483-510)
@@ -326,18 +428,26 @@ class Conv2D(Layer):
         if self.model.mode == TRAIN_MODE:
             self.cg_x = x
         biases_vector = self.biases if self.use_bias else None
-        return self.cg.conv_gemm_nchw(self.weights, x, biases=None, biases_vector=biases_vector,
-                                      **self._cg_kwargs())
+        self._op(ev.PYDTNN_OPS_FORWARD_CONVGEMM)
+        y = self.cg.conv_gemm_nchw(self.weights, x, biases=None, biases_vector=biases_vector, **self._cg_kwargs())
+        self._end()
+        return y
 
     def _backward_nchw_cg(self, dy):
         res = torch.empty(self.weights.shape, dtype=dy.dtype, device=dy.device)
+        self._op(ev.PYDTNN_OPS_BACKWARD_CONVGEMM)
         self.cg.conv_gemm_nchw(dy, self.cg_x, biases=res, trans=True, **self._cg_kwargs())
+        self._end()
         self.dw = res
         if self.use_bias:
+            self._op(ev.PYDTNN_OPS_BACKWARD_SUM_BIASES)
             self.db = ops.bias_grad(dy, self.co, self.ho * self.wo)
+            self._end()
         if self.need_dx:
             dx = torch.empty((dy.shape[0], self.ci, self.hi, self.wi), dtype=dy.dtype, device=dy.device)
+            self._op(ev.PYDTNN_OPS_BACKWARD_DECONV_GEMM)
             self.cg.deconv_gemm_nchw(self.weights, dy, dx, **self._cg_kwargs())
+            self._end()
             return dx
 
 

@@ -13,6 +13,9 @@ import torch
 
 from . import layers as L
 from . import ops
+from .best_of import BestOf
+from .tracers import (PYDTNN_MDL_BACKWARD, PYDTNN_MDL_EVENT, PYDTNN_MDL_EVENTS, PYDTNN_MDL_FORWARD,
+                      PYDTNN_MDL_UPDATE_DW, NullTracer)
 from .layers import EVALUATE_MODE, TRAIN_MODE, UNSPECIFIED_MODE
 from .utils import PYDTNN_TENSOR_FORMAT_NCHW, PYDTNN_TENSOR_FORMAT_NHWC
 
@@ -22,16 +25,6 @@ def _layer_id_generator():
     while True:
         yield current_layer_id
         current_layer_id += 1
-
-
-class _NullTracer:
-    """Same call surface as pydtnn/tracers/tracer.py:72-90 with tracing disabled (rocprofv3 is the tracer here)."""
-
-    def emit_event(self, evt_type, evt_val):
-        pass
-
-    def emit_nevent(self, evt_types, evt_vals):
-        pass
 
 
 _DEFAULTS = dict(
@@ -61,7 +54,7 @@ class Model:
         if dtype != torch.float32:
             raise ValueError("only float32 models run on the MI355X kernels")
         self.dtype = dtype
-        self.tracer = _NullTracer()
+        self.tracer = NullTracer()
         self.layers = []
         self.layer_id = _layer_id_generator()
         self.matmul = ops.matmul
@@ -73,6 +66,8 @@ class Model:
         self.tensor_format = PYDTNN_TENSOR_FORMAT_NHWC if fmt == "NHWC" else PYDTNN_TENSOR_FORMAT_NCHW
         self.batch_size = self.kwargs["batch_size"]
         self._fused = False
+        # pydtnn/model.py:216-218: without the flag every BestOf just calls its first alternative
+        BestOf.use_always_the_first_alternative(not self.kwargs["enable_best_of"])
 
     def __getattr__(self, item):
         try:
@@ -158,22 +153,37 @@ class Model:
         self.mode = TRAIN_MODE
         if global_batch_size is None:
             global_batch_size = x.shape[0]
+        emit = self.tracer.emit_event
         for i in range(1, len(self.layers)):
+            emit(PYDTNN_MDL_EVENT, self.layers[i].id * PYDTNN_MDL_EVENTS + PYDTNN_MDL_FORWARD)
             x = self.layers[i].forward(x)
+            emit(PYDTNN_MDL_EVENT, 0)
         loss, dx = loss_func(x, y_targ, global_batch_size)
         for i in range(len(self.layers) - 1, 0, -1):
+            emit(PYDTNN_MDL_EVENT, self.layers[i].id * PYDTNN_MDL_EVENTS + PYDTNN_MDL_BACKWARD)
             dx = self.layers[i].backward(dx)
+            emit(PYDTNN_MDL_EVENT, 0)
         for i in range(len(self.layers) - 1, 0, -1):
             self.layers[i].reduce_weights_sync()
+            emit(PYDTNN_MDL_EVENT, self.layers[i].id * PYDTNN_MDL_EVENTS + PYDTNN_MDL_UPDATE_DW)
             self.layers[i].update_weights(optimizer)
+            emit(PYDTNN_MDL_EVENT, 0)
         return loss
 
     def evaluate_batch(self, x):
         """Forward pass of pydtnn/model.py:623-644."""
         self.mode = EVALUATE_MODE
+        emit = self.tracer.emit_event
         for i in range(1, len(self.layers)):
+            emit(PYDTNN_MDL_EVENT, self.layers[i].id * PYDTNN_MDL_EVENTS + PYDTNN_MDL_FORWARD)
             x = self.layers[i].forward(x)
+            emit(PYDTNN_MDL_EVENT, 0)
         return x
+
+    def set_tracer(self, tracer):
+        """Installs a tracer (pydtnn_amd.tracers) and names its events after this model's layers."""
+        self.tracer = tracer
+        tracer.define_event_types(self)
 
     def evaluate_dataset_batch(self, x):
         """pydtnn/model.py:653-667: the fusion pass runs once, on the first evaluation."""

@@ -436,3 +436,91 @@ def test_committed_hand_cases_through_the_layer(pd, hand_cases, fmt, variant):
             layer.weights = dev(np.ascontiguousarray(w.transpose(1, 2, 3, 0)))
             y = host(layer.forward(dev(nhwc(x)))).transpose(0, 3, 1, 2)
         assert np.array_equal(y, case["y"]), (case["name"], y, case["y"])
+
+
+# ------------------------------------------------------------------ BestOf variant
+
+@pytest.mark.parametrize("fmt", ["NCHW", "NHWC"])
+def test_best_of_variant_races_the_two_routes_and_keeps_the_numbers(pd, oracle, fmt):
+    """enable_best_of: Conv2D.forward / backward go through BestOf (pydtnn/backends/cpu/layers/conv_2d_cpu.py:95-130,
+    :251-262); whichever route is being tried, y / dw / dx must match the oracle, and after the rounds one route
+    is chosen for the layer's problem size."""
+    announce("best_of", fmt)
+    d = D(4, 6, 14, 13, 10, 3, 3, 1, 1, 1, 1)
+    x, w, b, dy = (None,) * 4
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((d.b, d.c, d.h, d.w)).astype(np.float32)
+    w = (rng.standard_normal((d.kn, d.c, 3, 3)) * 0.2).astype(np.float32)
+    b = rng.standard_normal(d.kn).astype(np.float32)
+    dy = rng.standard_normal((d.b, d.kn, d.ho, d.wo)).astype(np.float32)
+    model = pd.Model(tensor_format=fmt, batch_size=d.b, enable_best_of=True)
+    try:
+        model.mode = pd.TRAIN_MODE
+        layer = pd.Conv2D(nfilters=d.kn, filter_shape=(3, 3), padding=1)
+        layer.set_model(model)
+        layer.initialize(prev_shape=(d.c, d.h, d.w) if fmt == "NCHW" else (d.h, d.w, d.c))
+        assert layer.forward.__name__ == f"_forward_{fmt.lower()}_best_of"
+        p = oracle.ConvParams(3, 3, 1, 1)
+        if fmt == "NCHW":
+            xin, win, dyin = x, w, dy
+            y_ref, cols = oracle.conv2d_forward_nchw_i2c(x, w, b, p)
+            dw_ref, db_ref, dx_ref = oracle.conv2d_backward_nchw_i2c(dy, cols, w, x.shape, p)
+        else:
+            xin, win, dyin = nhwc(x), np.ascontiguousarray(w.transpose(1, 2, 3, 0)), nhwc(dy)
+            y_ref, rows = oracle.conv2d_forward_nhwc_i2c(xin, win, b, p)
+            dw_ref, db_ref, dx_ref = oracle.conv2d_backward_nhwc_i2c(dyin, rows, win, xin.shape, p)
+        layer.weights, layer.biases = dev(win), dev(b)
+        pipeline = layer._best_fw_bw_pipeline
+        for step in range(pipeline.total_rounds * 2 + 2):
+            y = layer.forward(dev(xin))
+            dx = layer.backward(dev(dyin))
+            assert_close(host(y), y_ref, what=f"y step {step}")
+            assert_close(host(layer.dw), dw_ref, what=f"dw step {step}")
+            assert_close(host(dx), dx_ref, what=f"dx step {step}")
+        assert pipeline.best_method_has_been_found(layer, None)
+        assert list(pipeline.best_name.values())[0] in ("i2c", "cg")
+        model.mode = pd.EVALUATE_MODE
+        for _ in range(layer._best_fw.total_rounds * 2 + 1):
+            assert_close(host(layer.forward(dev(xin))), y_ref, what="y eval")
+        assert layer._best_fw.best_method_has_been_found(layer, None)
+    finally:
+        pd.BestOf.use_always_the_first_alternative(True)
+
+
+# ------------------------------------------------------------------ tracers on a real model
+
+def test_tracers_see_layers_and_operations_of_a_training_step(pd, tmp_path):
+    """SimpleTracer on a small model: one Model event per layer and direction, the convolution's operation
+    events inside them; RoctxTracer pushes and pops the same regions without error."""
+    announce("tracers")
+    t = pd.tracers
+    model = pd.Model(tensor_format="NCHW", batch_size=2)
+    model.add(pd.Input(shape=(8, 8, 3)))                      # (h, w, c), encoded into the model's format
+    model.add(pd.Conv2D(nfilters=4, filter_shape=(3, 3), padding=1, activation="relu"))
+    model.add(pd.Conv2D(nfilters=4, filter_shape=(3, 3), padding=1))
+    model.add(pd.Flatten())
+    model.add(pd.FC(shape=(5,), activation="softmax"))
+    tracer = t.SimpleTracer(True, str(tmp_path / "trace.csv"))
+    model.set_tracer(tracer)
+    x = dev(np.random.default_rng(0).standard_normal((2, 3, 8, 8)).astype(np.float32))
+    y = dev(np.eye(5, dtype=np.float32)[[1, 3]])
+    for _ in range(2):
+        model.train_batch(x, y, pd.CategoricalCrossEntropy(), pd.SGD(0.01, 0.9))
+    assert not tracer.pending_events
+    conv2 = model.layers[3]
+    assert conv2.canonical_name == "Conv2D" and conv2.need_dx
+    mdl, ops_ = tracer.events[t.PYDTNN_MDL_EVENT], tracer.events[t.PYDTNN_OPS_EVENT]
+    for layer in model.layers[1:]:
+        assert mdl[layer.id * t.PYDTNN_MDL_EVENTS + t.PYDTNN_MDL_FORWARD][0] == 2
+        assert mdl[layer.id * t.PYDTNN_MDL_EVENTS + t.PYDTNN_MDL_BACKWARD][0] == 2
+    for kind in (t.PYDTNN_OPS_FORWARD_CONVGEMM, t.PYDTNN_OPS_BACKWARD_CONVGEMM, t.PYDTNN_OPS_BACKWARD_SUM_BIASES,
+                 t.PYDTNN_OPS_BACKWARD_DECONV_GEMM):
+        assert ops_[conv2.id * t.PYDTNN_OPS_EVENTS + kind][0] == 2
+    first = model.layers[1]                                   # no dx for the first layer
+    assert first.id * t.PYDTNN_OPS_EVENTS + t.PYDTNN_OPS_BACKWARD_DECONV_GEMM not in ops_
+    tracer.write_output()
+    text = (tmp_path / "trace.csv").read_text()
+    assert f"{conv2.canonical_name_with_id}_forward" in text and "_Conv2D_backward_convgemm" in text
+    model.set_tracer(t.RoctxTracer(True))
+    model.train_batch(x, y, pd.CategoricalCrossEntropy(), pd.SGD(0.01, 0.9))
+    assert not model.tracer._open
