@@ -178,7 +178,9 @@ struct MapMN {
     static __device__ __forceinline__ int krow(int tid) { return uniform(tid / BMN); }
     // This thread's rows are k0 + e * kRowsPerPass.  With one or two rows per pass it holds both rows
     // of every (k, k+2) pair and writes them with one 64-bit store; with four (BMN = 64) it does not.
-    static __device__ __forceinline__ void store(float* lds, const float (&r)[NLD], int tid)
+    // Stores the elements e with e*PARTS/NLD == PART (a pair goes with its first element).
+    template <int PART, int PARTS>
+    static __device__ __forceinline__ void store_part(float* lds, const float (&r)[NLD], int tid)
     {
         const int m = tid % BMN, k0 = tid / BMN;
         float* base = lds + LdsTile<BMN>::index(k0, m);
@@ -186,17 +188,23 @@ struct MapMN {
         if constexpr (kRowsPerPass == 2) {
 #pragma unroll
             for (int e = 0; e < NLD; e += 2)  // k = k0 + 2e and k + 2
-                *reinterpret_cast<floatx2*>(base + (e >> 1) * 2 * P) = floatx2{r[e], r[e + 1]};
+                if (e * PARTS / NLD == PART)
+                    *reinterpret_cast<floatx2*>(base + (e >> 1) * 2 * P) = floatx2{r[e], r[e + 1]};
         } else if constexpr (kRowsPerPass == 1) {
 #pragma unroll
             for (int e = 0; e < NLD; ++e)  // k = e (k0 = 0); pairs (e, e + 2) for e % 4 in {0, 1}
-                if ((e & 2) == 0)
+                if ((e & 2) == 0 && e * PARTS / NLD == PART)
                     *reinterpret_cast<floatx2*>(base + ((e >> 2) * 2 + (e & 1)) * P) = floatx2{r[e], r[e + 2]};
         } else {
             static_assert(kRowsPerPass == 4, "tile extents are 64, 128 or 256");
 #pragma unroll
-            for (int e = 0; e < NLD; ++e) base[e * 2 * P] = r[e];  // k = k0 + 4e
+            for (int e = 0; e < NLD; ++e)
+                if (e * PARTS / NLD == PART) base[e * 2 * P] = r[e];  // k = k0 + 4e
         }
+    }
+    static __device__ __forceinline__ void store(float* lds, const float (&r)[NLD], int tid)
+    {
+        store_part<0, 1>(lds, r, tid);
     }
 };
 
@@ -207,12 +215,18 @@ struct MapK {
     static constexpr int NLD = BMN / kMnPerPass;
     static __device__ __forceinline__ int kk(int tid) { return tid % BK; }
     static __device__ __forceinline__ int mn(int tid, int e) { return tid / BK + e * kMnPerPass; }
-    static __device__ __forceinline__ void store(float* lds, const float (&r)[NLD], int tid)
+    template <int PART, int PARTS>
+    static __device__ __forceinline__ void store_part(float* lds, const float (&r)[NLD], int tid)
     {
         const int k = tid % BK, m0 = tid / BK;
         float* base = lds + LdsTile<BMN>::index(k, m0);
 #pragma unroll
-        for (int e = 0; e < NLD; ++e) base[e * kMnPerPass * 2] = r[e];
+        for (int e = 0; e < NLD; ++e)
+            if (e * PARTS / NLD == PART) base[e * kMnPerPass * 2] = r[e];
+    }
+    static __device__ __forceinline__ void store(float* lds, const float (&r)[NLD], int tid)
+    {
+        store_part<0, 1>(lds, r, tid);
     }
 };
 
@@ -279,6 +293,11 @@ struct PlainK {
         return buf_load(s.rsrc, s.rowoff[E] + it.voff, it.soff);
     }
     __device__ __forceinline__ void store(float* lds, const float (&r)[NLD], int tid) const { Map::store(lds, r, tid); }
+    template <int PART, int PARTS>
+    __device__ __forceinline__ void store_part(float* lds, const float (&r)[NLD], int tid) const
+    {
+        Map::template store_part<PART, PARTS>(lds, r, tid);
+    }
 };
 
 // elem(mn, k) = base[image*image_stride + k*ld + mn]   (mn contiguous).  The descriptor is re-based to
@@ -321,6 +340,11 @@ struct PlainMN {
         return buf_load(it.rsrc, s.voff + (uint32_t)(E * Map::kRowsPerPass) * (uint32_t)ld * 4u, 0);
     }
     __device__ __forceinline__ void store(float* lds, const float (&r)[NLD], int tid) const { Map::store(lds, r, tid); }
+    template <int PART, int PARTS>
+    __device__ __forceinline__ void store_part(float* lds, const float (&r)[NLD], int tid) const
+    {
+        Map::template store_part<PART, PARTS>(lds, r, tid);
+    }
 };
 
 // ---------------------------------------------------------------- implicit im2col, NCHW
@@ -388,6 +412,11 @@ struct Im2colNchwMN {
         return buf_load(s.rsrc, ((s.inv0 << (31u - bit)) & kOob) | s.base, off);
     }
     __device__ __forceinline__ void store(float* lds, const float (&r)[NLD], int tid) const { Map::store(lds, r, tid); }
+    template <int PART, int PARTS>
+    __device__ __forceinline__ void store_part(float* lds, const float (&r)[NLD], int tid) const
+    {
+        Map::template store_part<PART, PARTS>(lds, r, tid);
+    }
 };
 
 // dW view of the same matrix: B(k = (image, pixel), n = (c,i,j)).  Lanes run along the pixel (reduction)
@@ -441,6 +470,11 @@ struct Im2colNchwK {
         return buf_load(s.rsrc, ok ? (uint32_t)(it.base + s.coff[E]) * 4u : kOob, 0);
     }
     __device__ __forceinline__ void store(float* lds, const float (&r)[NLD], int tid) const { Map::store(lds, r, tid); }
+    template <int PART, int PARTS>
+    __device__ __forceinline__ void store_part(float* lds, const float (&r)[NLD], int tid) const
+    {
+        Map::template store_part<PART, PARTS>(lds, r, tid);
+    }
 };
 
 // ---------------------------------------------------------------- implicit im2row, NHWC
@@ -507,6 +541,11 @@ struct Im2rowNhwcK {
         return buf_load(s.rsrc, guarded_offset(invalid, s.base[E] + it.koff), 0);
     }
     __device__ __forceinline__ void store(float* lds, const float (&r)[NLD], int tid) const { Map::store(lds, r, tid); }
+    template <int PART, int PARTS>
+    __device__ __forceinline__ void store_part(float* lds, const float (&r)[NLD], int tid) const
+    {
+        Map::template store_part<PART, PARTS>(lds, r, tid);
+    }
 };
 
 // Filter in NHWC layout (c, kh, kw, kn) read as B(k in (i,j,c) order, n = filter).
@@ -540,6 +579,11 @@ struct FilterNhwcMN {
         return buf_load(s.rsrc, s.voff + rowoff, 0);
     }
     __device__ __forceinline__ void store(float* lds, const float (&r)[NLD], int tid) const { Map::store(lds, r, tid); }
+    template <int PART, int PARTS>
+    __device__ __forceinline__ void store_part(float* lds, const float (&r)[NLD], int tid) const
+    {
+        Map::template store_part<PART, PARTS>(lds, r, tid);
+    }
 };
 
 // dW view in NHWC: A(m = (i,j,c), k = (image, pixel)).  Lanes run along m (consecutive channels);
@@ -587,6 +631,11 @@ struct Im2rowNhwcMN {
         return buf_load(s.rsrc, ok ? (uint32_t)(pix * g.c + s.moff) * 4u : kOob, 0);
     }
     __device__ __forceinline__ void store(float* lds, const float (&r)[NLD], int tid) const { Map::store(lds, r, tid); }
+    template <int PART, int PARTS>
+    __device__ __forceinline__ void store_part(float* lds, const float (&r)[NLD], int tid) const
+    {
+        Map::template store_part<PART, PARTS>(lds, r, tid);
+    }
 };
 
 // ---------------------------------------------------------------- epilogues
@@ -699,13 +748,32 @@ __device__ __forceinline__ void request_operands(uint32_t a_base, uint32_t b_bas
     static_assert(T::TM <= 4 && T::TN <= 4, "operand fetch is written for up to 4 blocks per axis");
 }
 
+// Everything a step needs besides the accumulators: the register set that receives the loads of the
+// tile two steps ahead, and the register set (filled one step earlier) that this step stores into the
+// LDS buffer it does not read.
+template <class AL, class BL>
+struct StepRegs {
+    float (&ra)[AL::NLD];
+    float (&rb)[BL::NLD];
+    const float (&sa)[AL::NLD];
+    const float (&sb)[BL::NLD];
+    float* a_store;
+    float* b_store;
+    int tid;
+};
+
+// The LDS stores of a step are spread over its last kStoreGroups MFMA groups.
+constexpr int kStoreGroups = 4;
+
 // One MFMA group (k-step J of the LDS tile) and everything scheduled around it: an even group waits for
 // the operand pair it shares with the next group, starts the first MFMA and requests the following pair;
-// every group issues its share of the global loads, then the remaining MFMAs.
+// every group issues its share of the global loads, then the remaining MFMAs; the last groups also
+// store their share of the tile for the next step into the other LDS buffer, which nobody reads
+// between the barrier before this step and the barrier after it.
 template <class T, int BUF, int J, class AL, class BL>
 __device__ __forceinline__ void mfma_groups(const AL& al, const BL& bl, const typename AL::State& as,
                                             const typename BL::State& bs, const typename AL::Iter& ai,
-                                            const typename BL::Iter& bi, float (&ra)[AL::NLD], float (&rb)[BL::NLD],
+                                            const typename BL::Iter& bi, const StepRegs<AL, BL>& rg,
                                             uint32_t a_base, uint32_t b_base, floatx16 (&acc)[T::TM][T::TN],
                                             floatx2 (&af)[2][T::TM], floatx2 (&bf)[2][T::TN], int knext, int kend)
 {
@@ -718,25 +786,30 @@ __device__ __forceinline__ void mfma_groups(const AL& al, const BL& bl, const ty
         }
         acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[S][0][H], bf[S][0][H], acc[0][0], 0, 0, 0);
         if constexpr (H == 0 && J + 2 < G) request_operands<T, BUF, P + 1>(a_base, b_base, af[S ^ 1], bf[S ^ 1]);
-        group_load<J, 0, AL>(al, as, ai, ra, knext, kend);
-        group_load<J, 0, BL>(bl, bs, bi, rb, knext, kend);
+        group_load<J, 0, AL>(al, as, ai, rg.ra, knext, kend);
+        group_load<J, 0, BL>(bl, bs, bi, rg.rb, knext, kend);
 #pragma unroll
         for (int i = 0; i < T::TM; ++i)
 #pragma unroll
             for (int j = 0; j < T::TN; ++j)
                 if (i + j > 0)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[S][i][H], bf[S][j][H], acc[i][j], 0, 0, 0);
+        if constexpr (J >= G - kStoreGroups) {
+            al.template store_part<J - (G - kStoreGroups), kStoreGroups>(rg.a_store, rg.sa, rg.tid);
+            bl.template store_part<J - (G - kStoreGroups), kStoreGroups>(rg.b_store, rg.sb, rg.tid);
+        }
         // keep this group's LDS fetches, global loads and MFMAs together: the instruction scheduler
         // must not sink the loads to the end of the step
         __builtin_amdgcn_sched_barrier(0);
-        mfma_groups<T, BUF, J + 1, AL, BL>(al, bl, as, bs, ai, bi, ra, rb, a_base, b_base, acc, af, bf, knext, kend);
+        mfma_groups<T, BUF, J + 1, AL, BL>(al, bl, as, bs, ai, bi, rg, a_base, b_base, acc, af, bf, knext, kend);
     }
 }
 
-// Consumes LDS buffer BUF and loads the tile that starts at reduction index knext into (ra, rb).
+// Consumes LDS buffer BUF, loads the tile that starts at reduction index knext into (rg.ra, rg.rb)
+// and stores (rg.sa, rg.sb) into the other LDS buffer.
 template <class T, int BUF, class AL, class BL>
 __device__ __forceinline__ void step(const AL& al, const BL& bl, const typename AL::State& as,
-                                     const typename BL::State& bs, float (&ra)[AL::NLD], float (&rb)[BL::NLD],
+                                     const typename BL::State& bs, const StepRegs<AL, BL>& rg,
                                      uint32_t a_base, uint32_t b_base, floatx16 (&acc)[T::TM][T::TN], int knext,
                                      int kend)
 {
@@ -746,7 +819,7 @@ __device__ __forceinline__ void step(const AL& al, const BL& bl, const typename 
     request_operands<T, BUF, 0>(a_base, b_base, af[0], bf[0]);
     al.begin(as, ai, knext, kend);
     bl.begin(bs, bi, knext, kend);
-    mfma_groups<T, BUF, 0, AL, BL>(al, bl, as, bs, ai, bi, ra, rb, a_base, b_base, acc, af, bf, knext, kend);
+    mfma_groups<T, BUF, 0, AL, BL>(al, bl, as, bs, ai, bi, rg, a_base, b_base, acc, af, bf, knext, kend);
 }
 
 // The reduction loop of one tile over [kbeg, kend): adds into `acc`.  Leaves LDS free for reuse
@@ -762,7 +835,7 @@ __device__ __forceinline__ void tile_mainloop(const AL& al, const BL& bl, int m0
     bl.init(bs, n0, image, tid);
 
     // Register sets: during step s the loads of tile s+2 go to set (s & 1) while set ((s+1) & 1),
-    // filled during step s-1 with tile s+1, is stored to LDS at the end of the step.
+    // filled during step s-1 with tile s+1, is stored to the LDS buffer that step s does not read.
     float ra0[AL::NLD], rb0[BL::NLD], ra1[AL::NLD], rb1[BL::NLD];
     {   // tiles 0 and 1 (any kend, including an empty range: everything reads as zero)
         typename AL::Iter ai;
@@ -782,14 +855,12 @@ __device__ __forceinline__ void tile_mainloop(const AL& al, const BL& bl, int m0
 
     // Two steps per trip so that the register sets are named statically.  A reduction range with an
     // odd number of steps runs one extra step on a tile that lies beyond kend and therefore is zero.
+    // The stores of a trip's second step fill buffer 0 for the next trip (harmless after the last).
+    const StepRegs<AL, BL> even{ra0, rb0, ra1, rb1, As1, Bs1, tid}, odd{ra1, rb1, ra0, rb0, As0, Bs0, tid};
     for (int k0 = kbeg; k0 < kend; k0 += 2 * BK) {
-        step<T, 0>(al, bl, as, bs, ra0, rb0, a_base, b_base, acc, k0 + 2 * BK, kend);
-        al.store(As1, ra1, tid);
-        bl.store(Bs1, rb1, tid);
+        step<T, 0>(al, bl, as, bs, even, a_base, b_base, acc, k0 + 2 * BK, kend);
         __syncthreads();
-        step<T, 1>(al, bl, as, bs, ra1, rb1, a_base, b_base, acc, k0 + 3 * BK, kend);
-        al.store(As0, ra0, tid);
-        bl.store(Bs0, rb0, tid);
+        step<T, 1>(al, bl, as, bs, odd, a_base, b_base, acc, k0 + 3 * BK, kend);
         __syncthreads();
     }
 }
