@@ -27,9 +27,9 @@ HBM_PEAK_GBS = 8000.0
 
 # HBM-side bytes per launch of the forward kernel, from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE), each
 # scaled by what the same counter reads for a 256 MiB copy (factors 2.000 and 1.000):
-# main launch (197116.5 * 2.0 + 245760.0) KiB plus the fixup launch of its cut tiles (24631.4 * 2.0 + 4096.0) KiB.
+# main launch (197009.1 * 2.0 + 245760.0) KiB plus the fixup launch of its cut tiles (24632.4 * 2.0 + 4096.0) KiB.
 # The summary of those runs is profiles/cfg2_conv3x3_pmc_counters.md.
-MEASURED_TRAFFIC_BYTES = {"cfg2": int((197116.5 * 2.0 + 245760.0 + 24631.4 * 2.0 + 4096.0) * 1024)}
+MEASURED_TRAFFIC_BYTES = {"cfg2": int((197009.1 * 2.0 + 245760.0 + 24632.4 * 2.0 + 4096.0) * 1024)}
 
 
 def parse_args():
@@ -40,6 +40,8 @@ def parse_args():
     ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-vgg16", action="store_true", help="skip the VGG16 training-step extra of the default run")
+    ap.add_argument("--conv-layers", action="store_true",
+                    help="with --workload cfg5: also time forward / dW / dX of each distinct VGG16 convolution alone")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch a plain 256 MiB device copy (chan_eltwise_vec4_kernel with no epilogue) three "
                          "times, so that rocprofv3 FETCH_SIZE / WRITE_SIZE readings can be scaled to bytes")
@@ -246,6 +248,36 @@ def run_cfg5(torch, pd, args, steps=None, warmup=None):
     return ms, extra
 
 
+VGG16_CONVS = [(3, 64, 224), (64, 64, 224), (64, 128, 112), (128, 128, 112), (128, 256, 56), (256, 256, 56),
+               (256, 512, 28), (512, 512, 28), (512, 512, 14)]
+
+
+def vgg16_conv_layers(torch, n=64, reps=5):
+    """Each distinct 3x3 convolution of VGG16 alone, batch n: [ci, co, hw, GFLOP, fwd ms, dW ms, dX ms]."""
+    from pydtnn_amd.conv_gemm import ConvGemm
+    cg = ConvGemm()
+    rows = []
+    for ci, co, hw in VGG16_CONVS:
+        x = torch.randn(n, ci, hw, hw, device="cuda")
+        w = torch.randn(co, ci, 3, 3, device="cuda") * (2.0 / (9 * ci)) ** 0.5
+        dy = torch.randn(n, co, hw, hw, device="cuda")
+        dw, dx = torch.empty_like(w), torch.empty_like(x)
+        kw = dict(vpadding=1, hpadding=1)
+        calls = [lambda: cg.conv_gemm_nchw(w, x, **kw),
+                 lambda: cg.conv_gemm_nchw(dy, x, biases=dw, trans=True, **kw),
+                 lambda: cg.deconv_gemm_nchw(w, dy, dx, **kw)]
+        times = []
+        for fn in calls:
+            fn()
+            t = Timer(torch)
+            for _ in range(reps):
+                t(fn)
+            torch.cuda.synchronize()
+            times.append(round(t.mean_ms(), 4))
+        rows.append([ci, co, hw, round(2.0 * co * ci * 9 * n * hw * hw / 1e9, 1)] + times)
+    return rows
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -269,6 +301,8 @@ def main():
             extra.update(vgg)
     elif args.workload == "cfg5":
         ms, extra = run_cfg5(torch, pd, args)
+        if args.conv_layers:
+            extra["vgg16_conv_layers_ci_co_hw_gflop_fwd_dw_dx_ms"] = vgg16_conv_layers(torch)
         value, unit = 5929.5e9 / (ms * 1e-3) / 1e9, "GFLOP/s"
         workload = "cfg5: full VGG16 training step, fp32 NCHW, batch 64, 3x224x224, SGD momentum"
         roofline = {"bound": "mfma", "kernel": "whole step", "achieved": round(value / 1e3, 3),
