@@ -202,6 +202,32 @@ int pydtnn_hip_max_pool_2d_bwd_nhwc(const float *dy, const int32_t *idx_max, flo
                                     int kh, int kw, int vpadding, int hpadding, int vstride, int hstride,
                                     int vdilation, int hdilation, void *stream);
 
+/* ------------------------------------------------------------------------------------------
+ * The ReLU layer between two layers of a training step, done by its neighbours' stores instead of
+ * two passes of its own.  Results are those of the separate calls, bit for bit.
+ *   pydtnn_hip_sconvGemm_relu_mask: the forward of pydtnn_hip_sconvGemmNCHW / NHWC (nhwc = 0 / 1;
+ *       b, c, h, w name the input's batch, channels, height, width in either format) with
+ *       y = relu(conv(x) + bias_vector) and mask = (conv(x) + bias_vector) > 0 as int8, shaped like y:
+ *       what pydtnn_hip_relu_fwd (relu_cython.pyx:25-59) makes of the convolution's output.
+ *   pydtnn_hip_sconvGemm_back_gated: pydtnn_hip_sconvGemmNCHW_back / NHWC_back with dx multiplied by
+ *       gate (int8, shaped like dx): what pydtnn_hip_relu_bwd (relu_cpu.py:38-40) makes of dx when
+ *       the layer below the convolution is a ReLU whose mask is `gate`.  Same workspace.
+ *   pydtnn_hip_max_pool_2d_bwd_gated: the same for pydtnn_hip_max_pool_2d_bwd_nchw / nhwc.
+ * ---------------------------------------------------------------------------------------- */
+int pydtnn_hip_sconvGemm_relu_mask(int nhwc, unsigned b, unsigned c, unsigned h, unsigned w, unsigned kn, unsigned kh,
+                                   unsigned kw, unsigned vpadding, unsigned hpadding, unsigned vstride,
+                                   unsigned hstride, unsigned vdilation, unsigned hdilation, const float *weights,
+                                   const float *x, float *y, const float *bias_vector, int8_t *mask, void *workspace,
+                                   size_t workspace_bytes, void *stream);
+int pydtnn_hip_sconvGemm_back_gated(int nhwc, unsigned b, unsigned c, unsigned h, unsigned w, unsigned kn, unsigned kh,
+                                    unsigned kw, unsigned vstride, unsigned hstride, unsigned vpadding,
+                                    unsigned hpadding, unsigned vdilation, unsigned hdilation, const float *weights,
+                                    const float *dy, float *dx, const int8_t *gate, void *workspace,
+                                    size_t workspace_bytes, void *stream);
+int pydtnn_hip_max_pool_2d_bwd_gated(int nhwc, const float *dy, const int32_t *idx_max, float *dx, const int8_t *gate,
+                                     int b, int c, int h, int w, int kh, int kw, int vpadding, int hpadding,
+                                     int vstride, int hstride, int vdilation, int hdilation, void *stream);
+
 /* BatchNormalization in training mode (pydtnn/backends/cpu/layers/batch_normalization_cpu.py:59-82 and
  * :108-129; dx as pydtnn/cython_modules/bn_training_cython.pyx:236-243).  Tensors are viewed as
  * (outer, channels, inner): NCHW = (N, C, H*W); NHWC and 2-D = (rows, C, 1).  With n = outer * inner:

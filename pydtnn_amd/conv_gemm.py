@@ -8,7 +8,7 @@ the im2col matrix never exists in memory.
 import torch
 
 from . import native
-from .native import check, f32, lib, stream_ptr
+from .native import check, f32, lib, ptr, stream_ptr
 
 is_conv_gemm_available = True  # pydtnn/backends/cpu/libs/conv_gemm.py:32-36: probe result of load_library
 
@@ -40,9 +40,11 @@ class ConvGemm:
     # ------------------------------------------------------------------ forward / dW
     def conv_gemm_nchw(self, weights, x, biases=None, vpadding=0, hpadding=0, vstride=1, hstride=1,
                        vdilation=1, hdilation=1, biases_vector=None, trans=False, bn_running_mean=None,
-                       bn_inv_std=None, bn_gamma=None, bn_beta=None, relu=False):
+                       bn_inv_std=None, bn_gamma=None, bn_beta=None, relu=False, relu_mask=None):
         """``weights * im2col(x)`` (+ fused bias / BN / ReLU), or with ``trans`` the filter gradient
-        ``dy_cols * im2col(x)^T`` written into ``biases`` (pydtnn/backends/cpu/libs/conv_gemm.py:117-207)."""
+        ``dy_cols * im2col(x)^T`` written into ``biases`` (pydtnn/backends/cpu/libs/conv_gemm.py:117-207).
+        ``relu_mask`` (not in the reference; forward with ``relu`` and no BN only): an int8 tensor shaped
+        like the output that receives the mask a separate ReLU layer would keep for its backward."""
         b, c, h, w = x.shape
         if not trans:
             kn, ck, kh, kw = weights.shape
@@ -67,6 +69,13 @@ class ConvGemm:
             "this class was instantiated!"
         geom = (b, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
         ws, ws_bytes = native.conv_workspace(native.OP_DW if trans else native.OP_FWD, 0, geom)
+        if relu_mask is not None:
+            self._check_relu_mask(relu_mask, biases, trans, relu, bn_running_mean)
+            check(lib().pydtnn_hip_sconvGemm_relu_mask(
+                0, b, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation, f32(weights),
+                f32(x), f32(biases), f32(biases_vector), ptr(relu_mask), ws, ws_bytes, stream_ptr()),
+                "sconvGemm_relu_mask")
+            return biases
         check(lib().pydtnn_hip_sconvGemmNCHW(
             b'Y' if trans else b'N', b, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation,
             hdilation, f32(weights), f32(x), f32(biases), f32(biases_vector), f32(bn_running_mean), f32(bn_inv_std),
@@ -75,7 +84,7 @@ class ConvGemm:
 
     def conv_gemm_nhwc(self, weights, x, biases=None, vpadding=0, hpadding=0, vstride=1, hstride=1,
                        vdilation=1, hdilation=1, biases_vector=None, trans=False, bn_running_mean=None,
-                       bn_inv_std=None, bn_gamma=None, bn_beta=None, relu=False):
+                       bn_inv_std=None, bn_gamma=None, bn_beta=None, relu=False, relu_mask=None):
         """NHWC twin (pydtnn/backends/cpu/libs/conv_gemm.py:209-250): weights (c, kh, kw, kn)."""
         b, h, w, c = x.shape
         if not trans:
@@ -98,16 +107,37 @@ class ConvGemm:
         assert weights.dtype == x.dtype == biases.dtype, "All the matrices must have the same type of data!"
         geom = (b, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
         ws, ws_bytes = native.conv_workspace(native.OP_DW if trans else native.OP_FWD, 1, geom)
+        if relu_mask is not None:
+            self._check_relu_mask(relu_mask, biases, trans, relu, bn_running_mean)
+            check(lib().pydtnn_hip_sconvGemm_relu_mask(
+                1, b, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation, f32(weights),
+                f32(x), f32(biases), f32(biases_vector), ptr(relu_mask), ws, ws_bytes, stream_ptr()),
+                "sconvGemm_relu_mask")
+            return biases
         check(lib().pydtnn_hip_sconvGemmNHWC(
             b'Y' if trans else b'N', b, h, w, c, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation,
             hdilation, f32(weights), f32(x), f32(biases), f32(biases_vector), f32(bn_running_mean), f32(bn_inv_std),
             f32(bn_gamma), f32(bn_beta), bool(relu), ws, ws_bytes, stream_ptr()), "sconvGemmNHWC")
         return biases
 
+    @staticmethod
+    def _check_relu_mask(relu_mask, out, trans, relu, bn_running_mean):
+        assert not trans and relu and bn_running_mean is None, \
+            "relu_mask goes with a forward call that applies ReLU and no batch normalization"
+        assert relu_mask.dtype == torch.int8 and relu_mask.shape == out.shape and relu_mask.is_contiguous(), \
+            "relu_mask must be a contiguous int8 tensor shaped like the output"
+
+    @staticmethod
+    def _check_gate(gate, dx):
+        assert gate.dtype == torch.int8 and gate.shape == dx.shape and gate.is_contiguous(), \
+            "gate must be a contiguous int8 tensor shaped like dx"
+
     # ------------------------------------------------------------------ dX
     def deconv_gemm_nchw(self, weights, dy, dx, vpadding=0, hpadding=0, vstride=1, hstride=1,
-                         vdilation=1, hdilation=1):
-        """dx = col2im(weights_2D^T * dy_2D) (pydtnn/backends/cpu/libs/conv_gemm.py:252-309)."""
+                         vdilation=1, hdilation=1, gate=None):
+        """dx = col2im(weights_2D^T * dy_2D) (pydtnn/backends/cpu/libs/conv_gemm.py:252-309).
+        ``gate`` (not in the reference): the int8 mask of a ReLU layer that sits below this convolution;
+        dx is stored multiplied by it, which is that layer's backward."""
         kn, ck, kh, kw = weights.shape
         b2, kn2, ho, wo = dy.shape
         b, c, h, w = dx.shape
@@ -116,13 +146,19 @@ class ConvGemm:
         assert ck == c, "Number of channels in weights and x should be the same!"
         geom = (b, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
         ws, ws_bytes = native.conv_workspace(native.OP_DX, 0, geom)
+        if gate is not None:
+            self._check_gate(gate, dx)
+            check(lib().pydtnn_hip_sconvGemm_back_gated(
+                0, b, c, h, w, kn, kh, kw, vstride, hstride, vpadding, hpadding, vdilation, hdilation,
+                f32(weights), f32(dy), f32(dx), ptr(gate), ws, ws_bytes, stream_ptr()), "sconvGemm_back_gated")
+            return dx
         check(lib().pydtnn_hip_sconvGemmNCHW_back(
             b, c, h, w, kn, kh, kw, vstride, hstride, vpadding, hpadding, vdilation, hdilation,
             f32(weights), f32(dy), f32(dx), ws, ws_bytes, stream_ptr()), "sconvGemmNCHW_back")
         return dx
 
     def deconv_gemm_nhwc(self, weights, dy, dx, vpadding=0, hpadding=0, vstride=1, hstride=1,
-                         vdilation=1, hdilation=1):
+                         vdilation=1, hdilation=1, gate=None):
         """NHWC twin (pydtnn/backends/cpu/libs/conv_gemm.py:311-330)."""
         ck, kh, kw, kn = weights.shape
         b2, ho, wo, kn2 = dy.shape
@@ -132,6 +168,12 @@ class ConvGemm:
         assert ck == c, "Number of channels in weights and x should be the same!"
         geom = (b, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
         ws, ws_bytes = native.conv_workspace(native.OP_DX, 1, geom)
+        if gate is not None:
+            self._check_gate(gate, dx)
+            check(lib().pydtnn_hip_sconvGemm_back_gated(
+                1, b, c, h, w, kn, kh, kw, vstride, hstride, vpadding, hpadding, vdilation, hdilation,
+                f32(weights), f32(dy), f32(dx), ptr(gate), ws, ws_bytes, stream_ptr()), "sconvGemm_back_gated")
+            return dx
         check(lib().pydtnn_hip_sconvGemmNHWC_back(
             b, h, w, c, kn, kh, kw, vstride, hstride, vpadding, hpadding, vdilation, hdilation,
             f32(weights), f32(dy), f32(dx), ws, ws_bytes, stream_ptr()), "sconvGemmNHWC_back")

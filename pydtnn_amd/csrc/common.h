@@ -94,6 +94,33 @@ static inline ChanEpilogue no_epilogue()
     return e;
 }
 
+// Per-element byte masks a GEMM store can read or write beside its output, both indexed like the output:
+//   gate      (input)  the value is stored as v * gate[i], i.e. ReLU's backward dx = dy * mask
+//                      (pydtnn/backends/cpu/activations/relu_cpu.py:38-40) applied by the producer of dy;
+//   relu_mask (output) relu_mask[i] = v > 0, the mask ReLU's forward keeps for its backward
+//                      (pydtnn/cython_modules/relu_cython.pyx:25-59), written by a store that also rectifies.
+struct ElemMasks {
+    const int8_t* gate;
+    int8_t* relu_mask;
+};
+
+static inline ElemMasks no_masks()
+{
+    ElemMasks m = {nullptr, nullptr};
+    return m;
+}
+
+// Which of the two a store handles is a compile-time choice, so that no store tests a pointer per element.
+constexpr int kNoMasks = 0, kGate = 1, kReluMask = 2;
+
+template <int MASKS>
+__device__ __forceinline__ float elem_masks_apply(const ElemMasks& mk, long i, float v)
+{
+    if (MASKS == kGate) v *= (float)mk.gate[i];
+    if (MASKS == kReluMask) mk.relu_mask[i] = v > 0.0f ? 1 : 0;
+    return v;
+}
+
 #define HIP_RETURN_IF_LAUNCH_FAILED()                         \
     do {                                                      \
         hipError_t e__ = hipGetLastError();                   \

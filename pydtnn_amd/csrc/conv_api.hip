@@ -23,9 +23,9 @@ int launch_softmax_fwd(const float*, float*, int, int, hipStream_t);
 int launch_softmax_bwd(const float*, const float*, float*, int, int, hipStream_t);
 int launch_cce(const float*, const float*, float*, float*, float*, int, int, float, float, float, hipStream_t);
 int launch_max_pool_fwd_nchw(const float*, float*, int32_t*, const ConvGeom&, hipStream_t);
-int launch_max_pool_bwd_nchw(const float*, const int32_t*, float*, const ConvGeom&, hipStream_t);
+int launch_max_pool_bwd_nchw(const float*, const int32_t*, float*, const ConvGeom&, hipStream_t, const int8_t* gate);
 int launch_max_pool_fwd_nhwc(const float*, float*, int32_t*, const ConvGeom&, hipStream_t);
-int launch_max_pool_bwd_nhwc(const float*, const int32_t*, float*, const ConvGeom&, hipStream_t);
+int launch_max_pool_bwd_nhwc(const float*, const int32_t*, float*, const ConvGeom&, hipStream_t, const int8_t* gate);
 int launch_sgd_momentum(float*, const float*, float*, long, float, float, float, int, hipStream_t);
 
 namespace {
@@ -190,19 +190,27 @@ inline bool span_ok_k(long tile_rows, long ld, long group_images, long image_str
 }
 inline bool span_ok_mn(long ld) { return (long)BK * ld * 4 < kMaxSpanBytes; }
 
-inline EpiPlain epi_plain(float* out, long ldc, long split_stride, long m, long n, const ChanEpilogue& chan)
+template <int MASKS = kNoMasks>
+inline EpiPlainT<MASKS> epi_plain(float* out, long ldc, long split_stride, long m, long n, const ChanEpilogue& chan,
+                                  const ElemMasks& masks = no_masks())
 {
-    EpiPlain e;
+    EpiPlainT<MASKS> e;
     e.out = out; e.ldc = ldc; e.split_stride = split_stride; e.m_extent = (int)m; e.n_extent = (int)n; e.chan = chan;
+    e.masks = masks;
     return e;
 }
 
-inline EpiNchw epi_nchw(float* out, int channels, int howo, long p, const ChanEpilogue& chan)
+template <int MASKS = kNoMasks>
+inline EpiNchwT<MASKS> epi_nchw(float* out, int channels, int howo, long p, const ChanEpilogue& chan,
+                                const ElemMasks& masks = no_masks())
 {
-    EpiNchw e;
-    e.out = out; e.m_extent = channels; e.howo = howo; e.p = p; e.chan = chan;
+    EpiNchwT<MASKS> e;
+    e.out = out; e.m_extent = channels; e.howo = howo; e.p = p; e.chan = chan; e.masks = masks;
     return e;
 }
+
+// at most one of the two is ever set: the forward writes a ReLU mask, dX reads a gate
+inline int mask_kind(const ElemMasks& m) { return m.gate ? kGate : m.relu_mask ? kReluMask : kNoMasks; }
 
 // ---------------------------------------------------------------- forward (implicit)
 // The padding test works on tap masks of 31 usable bits: one word over i*kw + j when kh*kw <= 31,
@@ -217,7 +225,7 @@ constexpr size_t kBalanceBytes = (size_t)2 * kMaxResident * 128 * 128 * 4;
 
 template <bool WIDE>
 int conv_fwd_nchw_t(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan, float* ws,
-                    size_t ws_bytes, hipStream_t stream)
+                    size_t ws_bytes, hipStream_t stream, const ElemMasks& masks)
 {
     const TileSel sel = pick_tile(g.kn, g.p, g.k);
     int rc = PYDTNN_HIP_OK;
@@ -226,23 +234,34 @@ int conv_fwd_nchw_t(const ConvGeom& g, const float* w, const float* x, float* y,
         auto al = plain_k<T::BM, false>(w, (long)g.kn * g.k, g.k, 0, g.kn, 0);
         Im2colNchwMN<T::BN, WIDE> bl;
         bl.x = x; bl.g = g;
-        rc = launch_balanced<T>(al, bl, epi_nchw(y, g.kn, g.howo, g.p, chan), g.kn, g.p, g.k, ws, ws_bytes, stream);
+        switch (mask_kind(masks)) {
+        case kGate:
+            rc = launch_balanced<T>(al, bl, epi_nchw<kGate>(y, g.kn, g.howo, g.p, chan, masks), g.kn, g.p, g.k, ws,
+                                    ws_bytes, stream);
+            break;
+        case kReluMask:
+            rc = launch_balanced<T>(al, bl, epi_nchw<kReluMask>(y, g.kn, g.howo, g.p, chan, masks), g.kn, g.p, g.k, ws,
+                                    ws_bytes, stream);
+            break;
+        default:
+            rc = launch_balanced<T>(al, bl, epi_nchw(y, g.kn, g.howo, g.p, chan), g.kn, g.p, g.k, ws, ws_bytes, stream);
+        }
     })
     return rc;
 }
 
 // `ws` is optional: without it (or with less than kBalanceBytes) the launch is a plain grid of tiles.
 int conv_fwd_nchw(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan, float* ws,
-                  size_t ws_bytes, hipStream_t stream)
+                  size_t ws_bytes, hipStream_t stream, const ElemMasks& masks = no_masks())
 {
     if (!taps_supported(g)) return PYDTNN_HIP_ERR_UNSUPPORTED;
-    return taps_wide(g) ? conv_fwd_nchw_t<true>(g, w, x, y, chan, ws, ws_bytes, stream)
-                        : conv_fwd_nchw_t<false>(g, w, x, y, chan, ws, ws_bytes, stream);
+    return taps_wide(g) ? conv_fwd_nchw_t<true>(g, w, x, y, chan, ws, ws_bytes, stream, masks)
+                        : conv_fwd_nchw_t<false>(g, w, x, y, chan, ws, ws_bytes, stream, masks);
 }
 
 template <bool WIDE>
 int conv_fwd_nhwc_t(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan, float* ws,
-                    size_t ws_bytes, hipStream_t stream)
+                    size_t ws_bytes, hipStream_t stream, const ElemMasks& masks)
 {
     const TileSel sel = pick_tile(g.p, g.kn, g.k);
     int rc = PYDTNN_HIP_OK;
@@ -251,18 +270,29 @@ int conv_fwd_nhwc_t(const ConvGeom& g, const float* w, const float* x, float* y,
         al.x = x; al.g = g;
         FilterNhwcMN<T::BN> bl;
         bl.w = w; bl.g = g;
-        rc = launch_balanced<T>(al, bl, epi_plain(y, g.kn, 0, g.p, g.kn, chan), g.p, g.kn, g.k, ws, ws_bytes,
-                                stream);
+        switch (mask_kind(masks)) {
+        case kGate:
+            rc = launch_balanced<T>(al, bl, epi_plain<kGate>(y, g.kn, 0, g.p, g.kn, chan, masks), g.p, g.kn, g.k, ws,
+                                    ws_bytes, stream);
+            break;
+        case kReluMask:
+            rc = launch_balanced<T>(al, bl, epi_plain<kReluMask>(y, g.kn, 0, g.p, g.kn, chan, masks), g.p, g.kn, g.k,
+                                    ws, ws_bytes, stream);
+            break;
+        default:
+            rc = launch_balanced<T>(al, bl, epi_plain(y, g.kn, 0, g.p, g.kn, chan), g.p, g.kn, g.k, ws, ws_bytes,
+                                    stream);
+        }
     })
     return rc;
 }
 
 int conv_fwd_nhwc(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan, float* ws,
-                  size_t ws_bytes, hipStream_t stream)
+                  size_t ws_bytes, hipStream_t stream, const ElemMasks& masks = no_masks())
 {
     if (!taps_supported(g)) return PYDTNN_HIP_ERR_UNSUPPORTED;
-    return taps_wide(g) ? conv_fwd_nhwc_t<true>(g, w, x, y, chan, ws, ws_bytes, stream)
-                        : conv_fwd_nhwc_t<false>(g, w, x, y, chan, ws, ws_bytes, stream);
+    return taps_wide(g) ? conv_fwd_nhwc_t<true>(g, w, x, y, chan, ws, ws_bytes, stream, masks)
+                        : conv_fwd_nhwc_t<false>(g, w, x, y, chan, ws, ws_bytes, stream, masks);
 }
 
 // ---------------------------------------------------------------- filter gradient
@@ -345,8 +375,10 @@ inline bool dx_as_forward(const ConvGeom& g)
            g.hdilation * (g.kw - 1) >= g.hpadding;
 }
 
+// `gate` (optional, shaped like dx): dx is stored as gate ? dx : 0; after the scatter-add kernels this is
+// one more pass over dx.
 int conv_dx_i2c(const ConvGeom& g, int nhwc, const float* w, const float* dy, float* dx, float* ws, size_t ws_bytes,
-                hipStream_t stream)
+                hipStream_t stream, const int8_t* gate = nullptr)
 {
     const size_t need = (size_t)g.k * g.p * 4;
     if (!ws || ws_bytes < need) return PYDTNN_HIP_ERR_WORKSPACE;
@@ -366,7 +398,9 @@ int conv_dx_i2c(const ConvGeom& g, int nhwc, const float* w, const float* dy, fl
                            stream);
         })
         if (rc != PYDTNN_HIP_OK) return rc;
-        return launch_col2im_nchw(ws, dx, g, stream);
+        rc = launch_col2im_nchw(ws, dx, g, stream);
+        if (rc != PYDTNN_HIP_OK || !gate) return rc;
+        return launch_relu_bwd(dx, gate, dx, (long)g.n * g.c * g.h * g.w, stream);
     }
     // res(P x K) = dy_rows (P x kn) * W_rows^T : B(kk = filter, n = k) = w[n*kn + kk]
     const TileSel sel = pick_tile(g.p, g.k);
@@ -376,13 +410,15 @@ int conv_dx_i2c(const ConvGeom& g, int nhwc, const float* w, const float* dy, fl
         rc = launch<T>(al, bl, epi_plain(ws, g.k, 0, g.p, g.k, no_epilogue()), g.p, g.k, no_split(g.kn), 1, stream);
     })
     if (rc != PYDTNN_HIP_OK) return rc;
-    return launch_row2im_nhwc(ws, dx, g, stream);
+    rc = launch_row2im_nhwc(ws, dx, g, stream);
+    if (rc != PYDTNN_HIP_OK || !gate) return rc;
+    return launch_relu_bwd(dx, gate, dx, (long)g.n * g.c * g.h * g.w, stream);
 }
 
 int conv_dx(const ConvGeom& g, int nhwc, const float* w, const float* dy, float* dx, float* ws, size_t ws_bytes,
-            hipStream_t stream)
+            hipStream_t stream, const int8_t* gate = nullptr)
 {
-    if (!dx_as_forward(g)) return conv_dx_i2c(g, nhwc, w, dy, dx, ws, ws_bytes, stream);
+    if (!dx_as_forward(g)) return conv_dx_i2c(g, nhwc, w, dy, dx, ws, ws_bytes, stream, gate);
     const size_t need = (size_t)g.kn * g.k * 4;
     if (!ws || ws_bytes < need) return PYDTNN_HIP_ERR_WORKSPACE;
     int rc = launch_flip_filter(w, ws, nhwc, g.kn, g.c, g.kh, g.kw, stream);
@@ -396,8 +432,9 @@ int conv_dx(const ConvGeom& g, int nhwc, const float* w, const float* dy, float*
     const size_t used = (need + 255) & ~(size_t)255;
     float* rest = ws_bytes > used ? ws + used / 4 : nullptr;
     const size_t rest_bytes = ws_bytes > used ? ws_bytes - used : 0;
-    return nhwc ? conv_fwd_nhwc(gb, ws, dy, dx, no_epilogue(), rest, rest_bytes, stream)
-                : conv_fwd_nchw(gb, ws, dy, dx, no_epilogue(), rest, rest_bytes, stream);
+    const ElemMasks masks = {gate, nullptr};
+    return nhwc ? conv_fwd_nhwc(gb, ws, dy, dx, no_epilogue(), rest, rest_bytes, stream, masks)
+                : conv_fwd_nchw(gb, ws, dy, dx, no_epilogue(), rest, rest_bytes, stream, masks);
 }
 
 int geom_from_args(ConvGeom* g, long b, long c, long h, long w, long kn, long kh, long kw, long vpadding,
@@ -413,14 +450,17 @@ int geom_from_args(ConvGeom* g, long b, long c, long h, long w, long kn, long kh
 
 int sconv_gemm(int nhwc, char trans, const ConvGeom& g, const float* in1, const float* x, float* out,
                const float* bias, const float* mean, const float* inv_std, const float* gamma, const float* beta,
-               bool relu, void* ws, size_t ws_bytes, hipStream_t stream, int accumulate = 0)
+               bool relu, void* ws, size_t ws_bytes, hipStream_t stream, int accumulate = 0,
+               int8_t* relu_mask = nullptr)
 {
     if (!in1 || !x || !out) return PYDTNN_HIP_ERR_INVALID;
+    if (relu_mask && !relu) return PYDTNN_HIP_ERR_INVALID;
     if (trans == 'N') {
         if (!bn_args_consistent(mean, inv_std, gamma, beta)) return PYDTNN_HIP_ERR_INVALID;
         const ChanEpilogue chan = make_chan(bias, mean, inv_std, gamma, beta, relu ? 1 : 0);
-        return nhwc ? conv_fwd_nhwc(g, in1, x, out, chan, (float*)ws, ws_bytes, stream)
-                    : conv_fwd_nchw(g, in1, x, out, chan, (float*)ws, ws_bytes, stream);
+        const ElemMasks masks = {nullptr, relu_mask};
+        return nhwc ? conv_fwd_nhwc(g, in1, x, out, chan, (float*)ws, ws_bytes, stream, masks)
+                    : conv_fwd_nchw(g, in1, x, out, chan, (float*)ws, ws_bytes, stream, masks);
     }
     if (trans == 'Y') {
         if (bias || mean || inv_std || gamma || beta || relu) return PYDTNN_HIP_ERR_INVALID;
@@ -464,7 +504,8 @@ inline int plan_image_groups(ImageGroups* ig, long b, long c, long h, long w, lo
 int sconv_gemm_batched(int nhwc, char trans, long b, long c, long h, long w, long kn, long kh, long kw, long vpadding,
                        long hpadding, long vstride, long hstride, long vdilation, long hdilation, const float* in1,
                        const float* x, float* out, const float* bias, const float* mean, const float* inv_std,
-                       const float* gamma, const float* beta, bool relu, void* ws, size_t ws_bytes, hipStream_t stream)
+                       const float* gamma, const float* beta, bool relu, void* ws, size_t ws_bytes, hipStream_t stream,
+                       int8_t* relu_mask = nullptr)
 {
     if (!in1 || !x || !out) return PYDTNN_HIP_ERR_INVALID;
     ImageGroups ig;
@@ -481,7 +522,7 @@ int sconv_gemm_batched(int nhwc, char trans, long b, long c, long h, long w, lon
                             relu, ws, ws_bytes, stream, n0 > 0);
         else               // in1 = weights, out = y
             rc = sconv_gemm(nhwc, trans, g, in1, xg, out + n0 * ig.per_image_out, bias, mean, inv_std, gamma, beta,
-                            relu, ws, ws_bytes, stream);
+                            relu, ws, ws_bytes, stream, 0, relu_mask ? relu_mask + n0 * ig.per_image_out : nullptr);
         if (rc != PYDTNN_HIP_OK) return rc;
     }
     return PYDTNN_HIP_OK;
@@ -489,7 +530,7 @@ int sconv_gemm_batched(int nhwc, char trans, long b, long c, long h, long w, lon
 
 int conv_dx_batched(int nhwc, long b, long c, long h, long w, long kn, long kh, long kw, long vpadding, long hpadding,
                     long vstride, long hstride, long vdilation, long hdilation, const float* weights, const float* dy,
-                    float* dx, float* ws, size_t ws_bytes, hipStream_t stream)
+                    float* dx, float* ws, size_t ws_bytes, hipStream_t stream, const int8_t* gate = nullptr)
 {
     if (!weights || !dy || !dx) return PYDTNN_HIP_ERR_INVALID;
     ImageGroups ig;
@@ -500,7 +541,8 @@ int conv_dx_batched(int nhwc, long b, long c, long h, long w, long kn, long kh, 
         const long nb = b - n0 < ig.images ? b - n0 : ig.images;
         rc = geom_from_args(&g, nb, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation);
         if (rc != PYDTNN_HIP_OK) return rc;
-        rc = conv_dx(g, nhwc, weights, dy + n0 * ig.per_image_out, dx + n0 * ig.per_image_in, ws, ws_bytes, stream);
+        rc = conv_dx(g, nhwc, weights, dy + n0 * ig.per_image_out, dx + n0 * ig.per_image_in, ws, ws_bytes, stream,
+                     gate ? gate + n0 * ig.per_image_in : nullptr);
         if (rc != PYDTNN_HIP_OK) return rc;
     }
     return PYDTNN_HIP_OK;
@@ -798,7 +840,7 @@ int pydtnn_hip_max_pool_2d_bwd_nchw(const float* dy, const int32_t* idx_max, flo
     ConvGeom g;
     const int kn = 1;
     const int rc = geom_from_args(&g, GEOM_ARGS);
-    return rc != PYDTNN_HIP_OK ? rc : launch_max_pool_bwd_nchw(dy, idx_max, dx, g, as_stream(stream));
+    return rc != PYDTNN_HIP_OK ? rc : launch_max_pool_bwd_nchw(dy, idx_max, dx, g, as_stream(stream), nullptr);
 }
 
 int pydtnn_hip_max_pool_2d_fwd_nhwc(const float* x, float* y, int32_t* idx_max, int b, int h, int w, int c, int kh,
@@ -820,7 +862,42 @@ int pydtnn_hip_max_pool_2d_bwd_nhwc(const float* dy, const int32_t* idx_max, flo
     ConvGeom g;
     const int kn = 1;
     const int rc = geom_from_args(&g, GEOM_ARGS);
-    return rc != PYDTNN_HIP_OK ? rc : launch_max_pool_bwd_nhwc(dy, idx_max, dx, g, as_stream(stream));
+    return rc != PYDTNN_HIP_OK ? rc : launch_max_pool_bwd_nhwc(dy, idx_max, dx, g, as_stream(stream), nullptr);
+}
+
+int pydtnn_hip_max_pool_2d_bwd_gated(int nhwc, const float* dy, const int32_t* idx_max, float* dx, const int8_t* gate,
+                                     int b, int c, int h, int w, int kh, int kw, int vpadding, int hpadding,
+                                     int vstride, int hstride, int vdilation, int hdilation, void* stream)
+{
+    if (!dy || !dx || !idx_max || !gate) return PYDTNN_HIP_ERR_INVALID;
+    ConvGeom g;
+    const int kn = 1;
+    const int rc = geom_from_args(&g, GEOM_ARGS);
+    if (rc != PYDTNN_HIP_OK) return rc;
+    return nhwc ? launch_max_pool_bwd_nhwc(dy, idx_max, dx, g, as_stream(stream), gate)
+                : launch_max_pool_bwd_nchw(dy, idx_max, dx, g, as_stream(stream), gate);
+}
+
+int pydtnn_hip_sconvGemm_relu_mask(int nhwc, unsigned b, unsigned c, unsigned h, unsigned w, unsigned kn, unsigned kh,
+                                   unsigned kw, unsigned vpadding, unsigned hpadding, unsigned vstride,
+                                   unsigned hstride, unsigned vdilation, unsigned hdilation, const float* weights,
+                                   const float* x, float* y, const float* bias_vector, int8_t* mask, void* workspace,
+                                   size_t workspace_bytes, void* stream)
+{
+    if (!mask) return PYDTNN_HIP_ERR_INVALID;
+    return sconv_gemm_batched(nhwc, 'N', GEOM_ARGS, weights, x, y, bias_vector, nullptr, nullptr, nullptr, nullptr,
+                              true, workspace, workspace_bytes, as_stream(stream), mask);
+}
+
+int pydtnn_hip_sconvGemm_back_gated(int nhwc, unsigned b, unsigned c, unsigned h, unsigned w, unsigned kn, unsigned kh,
+                                    unsigned kw, unsigned vstride, unsigned hstride, unsigned vpadding,
+                                    unsigned hpadding, unsigned vdilation, unsigned hdilation, const float* weights,
+                                    const float* dy, float* dx, const int8_t* gate, void* workspace,
+                                    size_t workspace_bytes, void* stream)
+{
+    if (!gate) return PYDTNN_HIP_ERR_INVALID;
+    return conv_dx_batched(nhwc, GEOM_ARGS, weights, dy, dx, (float*)workspace, workspace_bytes, as_stream(stream),
+                           gate);
 }
 
 size_t pydtnn_hip_bn_training_workspace_bytes(int channels)

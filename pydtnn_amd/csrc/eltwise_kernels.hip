@@ -275,7 +275,8 @@ __global__ void __launch_bounds__(kThreads) max_pool_fwd_nchw_kernel(const float
 template <int KW>
 __global__ void __launch_bounds__(kThreads) max_pool_bwd_windows_nchw_kernel(const float* __restrict__ dy,
                                                                             const int32_t* __restrict__ idx_max,
-                                                                            float* __restrict__ dx, ConvGeom g)
+                                                                            float* __restrict__ dx, ConvGeom g,
+                                                                            const int8_t* __restrict__ gate)
 {
     const uint32_t win = blockIdx.x * kThreads + threadIdx.x;
     if (win >= (uint32_t)g.howo) return;
@@ -288,15 +289,22 @@ __global__ void __launch_bounds__(kThreads) max_pool_bwd_windows_nchw_kernel(con
         const float grad = 0.0f + dy[(size_t)plane * g.howo + win];
         const int ri = (int)fd_div(rec, g.fd_kh);
         const int rj = (int)(rec - fd_div(rec, g.fd_kw) * g.kw);
-        float* dst = dx + (size_t)plane * g.h * g.w + (size_t)(oy * g.kh) * g.w + ox * kw;
+        const size_t first = (size_t)plane * g.h * g.w + (size_t)(oy * g.kh) * g.w + ox * kw;
+        float* dst = dx + first;
+        const int8_t* gt = gate ? gate + first : nullptr;
         for (int ii = 0; ii < g.kh; ++ii) {
             if (KW == 2) {
-                *reinterpret_cast<float2*>(dst) =
-                    make_float2(ii == ri && rj == 0 ? grad : 0.0f, ii == ri && rj == 1 ? grad : 0.0f);
+                float2 v = make_float2(ii == ri && rj == 0 ? grad : 0.0f, ii == ri && rj == 1 ? grad : 0.0f);
+                if (gt) { v.x *= (float)gt[0]; v.y *= (float)gt[1]; }
+                *reinterpret_cast<float2*>(dst) = v;
             } else {
-                for (int jj = 0; jj < kw; ++jj) dst[jj] = ii == ri && jj == rj ? grad : 0.0f;
+                for (int jj = 0; jj < kw; ++jj) {
+                    const float v = ii == ri && jj == rj ? grad : 0.0f;
+                    dst[jj] = gt ? v * (float)gt[jj] : v;
+                }
             }
             dst += g.w;
+            if (gt) gt += g.w;
         }
     }
 }
@@ -310,7 +318,8 @@ __global__ void __launch_bounds__(kThreads) max_pool_bwd_windows_nchw_kernel(con
 template <bool TILED>
 __global__ void __launch_bounds__(kThreads) max_pool_bwd_nchw_kernel(const float* __restrict__ dy,
                                                                     const int32_t* __restrict__ idx_max,
-                                                                    float* __restrict__ dx, ConvGeom g)
+                                                                    float* __restrict__ dx, ConvGeom g,
+                                                                    const int8_t* __restrict__ gate)
 {
     const uint32_t hw = (uint32_t)(g.h * g.w);
     const uint32_t pix = blockIdx.x * kThreads + threadIdx.x;
@@ -331,6 +340,7 @@ __global__ void __launch_bounds__(kThreads) max_pool_bwd_nchw_kernel(const float
                 const uint32_t rj = rec - fd_div(rec, g.fd_kw) * g.kw;
                 if ((int)ri == ii && (int)rj == jj) acc = 0.0f + dy[(long)plane * g.howo + win];
             }
+            if (gate) acc *= (float)gate[(long)plane * hw + pix];
             dx[(long)plane * hw + pix] = acc;
         }
         return;
@@ -356,6 +366,7 @@ __global__ void __launch_bounds__(kThreads) max_pool_bwd_nchw_kernel(const float
                 if ((int)ri == ii && (int)rj == jj) acc += gy[oy * g.wo + ox];
             }
         }
+        if (gate) acc *= (float)gate[(long)plane * hw + pix];
         dx[(long)plane * hw + pix] = acc;
     }
 }
@@ -398,7 +409,8 @@ __global__ void __launch_bounds__(kThreads) max_pool_fwd_nhwc_kernel(const float
 // Gather form of the backward scatter: windows visited in ascending (oy, ox), i.e. descending taps.
 __global__ void __launch_bounds__(kThreads) max_pool_bwd_nhwc_kernel(const float* __restrict__ dy,
                                                                     const int32_t* __restrict__ idx_max,
-                                                                    float* __restrict__ dx, ConvGeom g, int c_exact)
+                                                                    float* __restrict__ dx, ConvGeom g, int c_exact,
+                                                                    const int8_t* __restrict__ gate)
 {
     const uint32_t per_image = (uint32_t)(g.h * g.w * g.c);
     const uint32_t e = blockIdx.x * kThreads + threadIdx.x;
@@ -428,6 +440,7 @@ __global__ void __launch_bounds__(kThreads) max_pool_bwd_nhwc_kernel(const float
                 if ((int)ri == ii && (int)rj == jj) acc += dy[at];
             }
         }
+        if (gate) acc *= (float)gate[(size_t)nn * per_image + e];
         dx[(size_t)nn * per_image + e] = acc;
     }
 }
@@ -836,8 +849,9 @@ int launch_max_pool_fwd_nchw(const float* x, float* y, int32_t* idx_max, const C
     return PYDTNN_HIP_OK;
 }
 
+// `gate` (optional, shaped like dx): dx is stored multiplied by it, ReLU's backward of the layer below.
 int launch_max_pool_bwd_nchw(const float* dy, const int32_t* idx_max, float* dx, const ConvGeom& g,
-                             hipStream_t stream)
+                             hipStream_t stream, const int8_t* gate)
 {
     const long planes = (long)g.n * g.c;
     dim3 grid(blocks_for((long)g.h * g.w), (unsigned)(planes < 65535 ? planes : 65535));
@@ -849,14 +863,14 @@ int launch_max_pool_bwd_nchw(const float* dy, const int32_t* idx_max, float* dx,
         dim3 wgrid(blocks_for(g.howo), (unsigned)(planes < 65535 ? planes : 65535));
         if (g.kw == 2 && (reinterpret_cast<uintptr_t>(dx) & 7) == 0)
             hipLaunchKernelGGL(max_pool_bwd_windows_nchw_kernel<2>, wgrid, dim3(kThreads), 0, stream, dy, idx_max, dx,
-                               g);
+                               g, gate);
         else
             hipLaunchKernelGGL(max_pool_bwd_windows_nchw_kernel<0>, wgrid, dim3(kThreads), 0, stream, dy, idx_max, dx,
-                               g);
+                               g, gate);
     } else if (tiled)
-        hipLaunchKernelGGL(max_pool_bwd_nchw_kernel<true>, grid, dim3(kThreads), 0, stream, dy, idx_max, dx, g);
+        hipLaunchKernelGGL(max_pool_bwd_nchw_kernel<true>, grid, dim3(kThreads), 0, stream, dy, idx_max, dx, g, gate);
     else
-        hipLaunchKernelGGL(max_pool_bwd_nchw_kernel<false>, grid, dim3(kThreads), 0, stream, dy, idx_max, dx, g);
+        hipLaunchKernelGGL(max_pool_bwd_nchw_kernel<false>, grid, dim3(kThreads), 0, stream, dy, idx_max, dx, g, gate);
     HIP_RETURN_IF_LAUNCH_FAILED();
     return PYDTNN_HIP_OK;
 }
@@ -873,13 +887,14 @@ int launch_max_pool_fwd_nhwc(const float* x, float* y, int32_t* idx_max, const C
 }
 
 int launch_max_pool_bwd_nhwc(const float* dy, const int32_t* idx_max, float* dx, const ConvGeom& g,
-                             hipStream_t stream)
+                             hipStream_t stream, const int8_t* gate)
 {
     const long per_image = (long)g.h * g.w * g.c;
     if (per_image >= (1l << 31) - kThreads) return PYDTNN_HIP_ERR_UNSUPPORTED;
     const int c_exact = (unsigned long)(per_image + kThreads) * (unsigned long)g.c < (1ul << 32);
     dim3 grid(blocks_for(per_image), (unsigned)(g.n < 65535 ? g.n : 65535));
-    hipLaunchKernelGGL(max_pool_bwd_nhwc_kernel, grid, dim3(kThreads), 0, stream, dy, idx_max, dx, g, c_exact);
+    hipLaunchKernelGGL(max_pool_bwd_nhwc_kernel, grid, dim3(kThreads), 0, stream, dy, idx_max, dx, g, c_exact,
+                       gate);
     HIP_RETURN_IF_LAUNCH_FAILED();
     return PYDTNN_HIP_OK;
 }

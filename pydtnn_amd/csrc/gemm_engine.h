@@ -641,14 +641,18 @@ struct Im2rowNhwcMN {
 // ---------------------------------------------------------------- epilogues
 // Row-major store C[split*split_stride + m*ldc + n]; the per-channel chain uses the column index
 // (NHWC convolution, FC forward).
-struct EpiPlain {
+// MASKS (kNoMasks, kGate, kReluMask): the store also applies the gate or writes the ReLU mask (separate
+// instantiations, so that no case carries a test per stored element).
+template <int MASKS>
+struct EpiPlainT {
     float* out;
     long ldc;
     long split_stride;
     int m_extent, n_extent;
     ChanEpilogue chan;
+    ElemMasks masks;  // only with a single split
     struct Col {
-        float* ptr;
+        long off;
         int n;
         bool ok;
     };
@@ -657,27 +661,30 @@ struct EpiPlain {
         Col c;
         c.n = n;
         c.ok = n < n_extent;
-        c.ptr = out + (long)split * split_stride + n;
+        c.off = (long)split * split_stride + n;
         return c;
     }
     __device__ __forceinline__ void store(const Col& c, int m, float v) const
     {
-        if (c.ok && m < m_extent) c.ptr[(long)m * ldc] = chan_epilogue_apply(chan, c.n, v);
+        if (c.ok && m < m_extent) {
+            const long i = c.off + (long)m * ldc;
+            const float r = chan_epilogue_apply(chan, c.n, v);
+            out[i] = elem_masks_apply<MASKS>(masks, i, r);
+        }
     }
 };
+using EpiPlain = EpiPlainT<kNoMasks>;
 
-// Direct store into an NCHW tensor: row m = output channel, column n = (img, pixel):
-// out[(img*m_extent + m)*howo + pixel].  This folds the reference's bias pass
-// (add_nchw_cython.pyx:57-58) and its (co,N,ho,wo)->(N,co,ho,wo) copy
-// (conv_2d_cpu.py:288) into the GEMM's only store.  Channel = row.
-struct EpiNchw {
+template <int MASKS>
+struct EpiNchwT {
     float* out;
     int m_extent;  // output channels
     int howo;
     long p;        // images * howo
     ChanEpilogue chan;
+    ElemMasks masks;
     struct Col {
-        float* ptr;
+        long off;
         bool ok;
     };
     __device__ __forceinline__ Col column(int n, int /*split*/) const
@@ -687,14 +694,20 @@ struct EpiNchw {
         const int nc = c.ok ? n : 0;
         const int img = nc / howo;
         const int pp = nc - img * howo;
-        c.ptr = out + (long)img * m_extent * howo + pp;
+        c.off = (long)img * m_extent * howo + pp;
         return c;
     }
     __device__ __forceinline__ void store(const Col& c, int m, float v) const
     {
-        if (c.ok && m < m_extent) c.ptr[(long)m * howo] = chan_epilogue_apply(chan, m, v);
+        if (c.ok && m < m_extent) {
+            const long i = c.off + (long)m * howo;
+            const float r = chan_epilogue_apply(chan, m, v);
+            out[i] = elem_masks_apply<MASKS>(masks, i, r);
+        }
     }
 };
+using EpiNchw = EpiNchwT<kNoMasks>;
+
 
 // ---------------------------------------------------------------- the kernel
 // Workgroups of one launch are handed to the 8 XCDs round-robin; remap the linear id so that each
@@ -878,9 +891,11 @@ __device__ __forceinline__ void clear_acc(floatx16 (&acc)[T::TM][T::TN])
 
 // Accumulator layout of v_mfma_f32_32x32x2_f32: register v of lane l holds
 // C[8*(v/4) + 4*(l/32) + v%4][l%32] of the 32x32 block.
+//
+// Generic tile store: one guarded store per element through the epilogue's own store().
 template <class T, class EP>
-__device__ __forceinline__ void store_tile(const EP& ep, const floatx16 (&acc)[T::TM][T::TN], int m0, int n0,
-                                           int split, int tid)
+__device__ __forceinline__ void store_tile_generic(const EP& ep, const floatx16 (&acc)[T::TM][T::TN], int m0, int n0,
+                                                   int split, int tid)
 {
     const int wave = tid >> 6, lane = tid & 63;
     const int wm0 = (wave % T::WGM) * T::WM, wn0 = (wave / T::WGM) * T::WN;
@@ -898,6 +913,130 @@ __device__ __forceinline__ void store_tile(const EP& ep, const floatx16 (&acc)[T
     }
 }
 
+__device__ __forceinline__ rsrc_t make_rsrc_bytes(const void* p, long bytes)
+{
+    bytes = bytes < 0 ? 0 : (bytes > kMaxSpanBytes ? kMaxSpanBytes : bytes);
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
+}
+
+// Tile store into an (images, channels, ho*wo) tensor, written as straight-line code: rows of C are
+// channels, so the per-channel epilogue parameters are per row; the tile's rows of them are staged in LDS
+// once (`lds`: at least 5*BM floats, free at this point) instead of being fetched from memory in front of
+// every store; out-of-range rows and columns get a buffer offset beyond the descriptor, which the hardware
+// drops, instead of a branch; the gate bytes of a tile are all requested before its first store (loads and
+// stores retire in issue order, so a load issued between two stores would wait for the first of them).
+// Needs the whole tensor inside one descriptor (fewer than 2^29 elements), which the host guarantees.
+template <class T, int MASKS>
+__device__ __forceinline__ void store_tile_nchw(const EpiNchwT<MASKS>& ep, const floatx16 (&acc)[T::TM][T::TN], int m0,
+                                                int n0, int tid, float* lds)
+{
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm0 = (wave % T::WGM) * T::WM, wn0 = (wave / T::WGM) * T::WN;
+    const int frag_r = lane & 31, frag_k = lane >> 5;
+    const ChanEpilogue ch = ep.chan;
+    const bool has_bias = ch.bias != nullptr, has_bn = ch.mean != nullptr;
+    if (has_bias || has_bn) {
+        if (tid < T::BM) {
+            const int m = min(m0 + tid, ep.m_extent - 1);
+            if (has_bias) lds[tid] = ch.bias[m];
+            if (has_bn) {
+                lds[T::BM + tid] = ch.mean[m];
+                lds[2 * T::BM + tid] = ch.inv_std[m];
+                lds[3 * T::BM + tid] = ch.gamma[m];
+                lds[4 * T::BM + tid] = ch.beta[m];
+            }
+        }
+        __syncthreads();
+    }
+    const long total = ep.p * ep.m_extent;
+    const rsrc_t out_rsrc = make_rsrc(ep.out, total);
+    // offset of (image, channel 4*frag_k, pixel) of each of this lane's columns, in floats' bytes (col_off4) and
+    // in elements (col_off1, for the byte masks), or kOob
+    uint32_t col_off4[T::TN];
+    [[maybe_unused]] uint32_t col_off1[T::TN];
+#pragma unroll
+    for (int j = 0; j < T::TN; ++j) {
+        const int n = n0 + wn0 + j * 32 + frag_r;
+        const bool ok = n < ep.p;
+        const int nc = ok ? n : 0;
+        const int img = nc / ep.howo;
+        const int pp = nc - img * ep.howo;
+        const uint32_t e = (uint32_t)((img * ep.m_extent + 4 * frag_k) * ep.howo + pp);
+        col_off4[j] = ok ? e * 4u : kOob;
+        col_off1[j] = ok ? e : kOob;
+    }
+    const int lane_m0 = m0 + wm0 + 4 * frag_k;  // this lane's first row
+    [[maybe_unused]] float gate[T::TM][16][T::TN];
+    if constexpr (MASKS == kGate) {
+        const rsrc_t gate_rsrc = make_rsrc_bytes(ep.masks.gate, total);
+#pragma unroll
+        for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int r = i * 32 + 8 * (v / 4) + (v % 4);
+                const bool row_ok = lane_m0 + r < ep.m_extent;
+                const uint32_t soff = (uint32_t)(m0 + wm0 + r) * (uint32_t)ep.howo;
+#pragma unroll
+                for (int j = 0; j < T::TN; ++j)
+                    gate[i][v][j] = (float)(int8_t)__builtin_amdgcn_raw_buffer_load_b8(
+                        gate_rsrc, (int)(row_ok ? col_off1[j] : kOob), (int)soff, 0);
+            }
+    }
+    [[maybe_unused]] rsrc_t mask_rsrc;
+    if constexpr (MASKS == kReluMask) mask_rsrc = make_rsrc_bytes(ep.masks.relu_mask, total);
+#pragma unroll
+    for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int r = i * 32 + 8 * (v / 4) + (v % 4);
+            const bool row_ok = lane_m0 + r < ep.m_extent;
+            const uint32_t soff = (uint32_t)(m0 + wm0 + r) * (uint32_t)ep.howo;
+            const int row = wm0 + 4 * frag_k + r;  // within the tile
+            float bias = 0.0f, mean = 0.0f, inv_std = 0.0f, gamma = 0.0f, beta = 0.0f;
+            if (has_bias) bias = lds[row];
+            if (has_bn) {
+                mean = lds[T::BM + row];
+                inv_std = lds[2 * T::BM + row];
+                gamma = lds[3 * T::BM + row];
+                beta = lds[4 * T::BM + row];
+            }
+#pragma unroll
+            for (int j = 0; j < T::TN; ++j) {
+                float val = acc[i][j][v];
+                if (has_bias) val += bias;
+                if (has_bn) {
+                    const float t = (val - mean) * inv_std;
+                    val = t * gamma + beta;
+                }
+                if (ch.relu) val = val > 0.0f ? val : 0.0f;
+                if constexpr (MASKS == kGate) val *= gate[i][v][j];
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, val), out_rsrc,
+                                                      (int)(row_ok ? col_off4[j] : kOob), (int)(soff * 4u), 0);
+                if constexpr (MASKS == kReluMask)
+                    __builtin_amdgcn_raw_buffer_store_b8((uint8_t)(val > 0.0f ? 1 : 0), mask_rsrc,
+                                                         (int)(row_ok ? col_off1[j] : kOob), (int)soff, 0);
+            }
+        }
+    // the staged parameters are read until here; the caller may refill LDS afterwards
+    if (has_bias || has_bn) __syncthreads();
+}
+
+template <class EP>
+struct IsEpiNchw { static constexpr bool value = false; };
+template <int MASKS>
+struct IsEpiNchw<EpiNchwT<MASKS>> { static constexpr bool value = true; };
+
+// `lds`: at least 5*BM floats that nobody else uses during the call.
+template <class T, class EP>
+__device__ __forceinline__ void store_tile(const EP& ep, const floatx16 (&acc)[T::TM][T::TN], int m0, int n0,
+                                           int split, int tid, float* lds)
+{
+    if constexpr (IsEpiNchw<EP>::value)
+        store_tile_nchw<T>(ep, acc, m0, n0, tid, lds);
+    else
+        store_tile_generic<T>(ep, acc, m0, n0, split, tid);
+}
+
 // LDS byte addresses of this lane's MFMA operand elements of buffer 0 at k-step 0, block (0, 0).
 template <class T>
 __device__ __forceinline__ void operand_bases(const float* As0, const float* Bs0, int tid, uint32_t* a_base,
@@ -911,7 +1050,7 @@ __device__ __forceinline__ void operand_bases(const float* As0, const float* Bs0
 }
 
 template <class T, class AL, class BL, class EP>
-__global__ void __launch_bounds__(kThreads) gemm_kernel(AL al, BL bl, EP ep, int tiles_m, SplitInfo si)
+__device__ __forceinline__ void gemm_body(const AL& al, const BL& bl, const EP& ep, int tiles_m, const SplitInfo& si)
 {
     __shared__ __align__(16) float As[2][BK * (T::BM + kPad)];
     __shared__ __align__(16) float Bs[2][BK * (T::BN + kPad)];
@@ -933,7 +1072,28 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(AL al, BL bl, EP ep, int
     floatx16 acc[T::TM][T::TN];
     clear_acc<T>(acc);
     tile_mainloop<T>(al, bl, m0, n0, image, kbeg, kend, As[0], As[1], Bs[0], Bs[1], a_base, b_base, acc, tid);
-    store_tile<T>(ep, acc, m0, n0, split, tid);
+    store_tile<T>(ep, acc, m0, n0, split, tid, As[0]);
+}
+
+// Three workgroups per compute unit need at most 168 registers per lane.  The kernel is built under that
+// limit unless the two loaders' per-thread state alone (precomputed offsets of every element a thread
+// loads) is so large that the limit would spill inside the reduction loop; those run two per CU.
+template <class AL, class BL>
+struct FitsThreePerCu {
+    static constexpr bool value = sizeof(typename AL::State) + sizeof(typename BL::State) <= 48 * 4;
+};
+
+template <class T, class AL, class BL, class EP>
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3)))
+gemm_kernel(AL al, BL bl, EP ep, int tiles_m, SplitInfo si)
+{
+    gemm_body<T>(al, bl, ep, tiles_m, si);
+}
+
+template <class T, class AL, class BL, class EP>
+__global__ void __launch_bounds__(kThreads) gemm_kernel_large_state(AL al, BL bl, EP ep, int tiles_m, SplitInfo si)
+{
+    gemm_body<T>(al, bl, ep, tiles_m, si);
 }
 
 template <class T, class AL, class BL, class EP>
@@ -943,7 +1103,11 @@ inline int launch(const AL& al, const BL& bl, const EP& ep, long m, long n, cons
     const long tiles_m = (m + T::BM - 1) / T::BM, tiles_n = (n + T::BN - 1) / T::BN;
     if (tiles_m * tiles_n >= (1l << 31) || splits > 65535 || splits < 1) return PYDTNN_HIP_ERR_UNSUPPORTED;
     dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)splits);
-    hipLaunchKernelGGL((gemm_kernel<T, AL, BL, EP>), grid, dim3(kThreads), 0, stream, al, bl, ep, (int)tiles_m, si);
+    if constexpr (FitsThreePerCu<AL, BL>::value)
+        hipLaunchKernelGGL((gemm_kernel<T, AL, BL, EP>), grid, dim3(kThreads), 0, stream, al, bl, ep, (int)tiles_m, si);
+    else
+        hipLaunchKernelGGL((gemm_kernel_large_state<T, AL, BL, EP>), grid, dim3(kThreads), 0, stream, al, bl, ep,
+                           (int)tiles_m, si);
     HIP_RETURN_IF_LAUNCH_FAILED();
     return PYDTNN_HIP_OK;
 }
@@ -1031,7 +1195,7 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3
         clear_acc<T>(acc);
         tile_mainloop<T>(al, bl, m0, n0, 0, kbeg, kend, As[0], As[1], Bs[0], Bs[1], a_base, b_base, acc, tid);
         if (whole) {
-            store_tile<T>(ep, acc, m0, n0, 0, tid);
+            store_tile<T>(ep, acc, m0, n0, 0, tid, As[0]);
         } else {
             float* dst = slot + tid;
 #pragma unroll
@@ -1116,6 +1280,10 @@ inline int launch_balanced(const AL& al, const BL& bl, const EP& ep, long m, lon
     const long tiles_m = (m + T::BM - 1) / T::BM, tiles_n = (n + T::BN - 1) / T::BN;
     const long tiles = tiles_m * tiles_n;
     if (tiles >= (1l << 31)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+    // the balanced kernel is built for three workgroups per CU; loaders too large for that take the plain grid
+    if constexpr (!FitsThreePerCu<AL, BL>::value) {
+        return launch<T>(al, bl, ep, m, n, no_split(k), 1, stream);
+    } else {
     const Residency res = resident_workgroups<T, AL, BL, EP>();
     const int resident = res.workgroups;
     const int units = (k + 2 * BK - 1) / (2 * BK);
@@ -1146,6 +1314,7 @@ inline int launch_balanced(const AL& al, const BL& bl, const EP& ep, long m, lon
         HIP_RETURN_IF_LAUNCH_FAILED();
     }
     return PYDTNN_HIP_OK;
+    }
 }
 
 }  // namespace gemm

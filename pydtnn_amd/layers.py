@@ -87,6 +87,9 @@ class Layer:
         self.model = None
         self.prev_shape = None
         self.is_block_layer = False
+        # set by Model.add when ReLU folding is enabled (see Relu)
+        self.relu_above = None
+        self.relu_below = None
 
     @property
     def canonical_name(self):
@@ -163,18 +166,35 @@ class Input(Layer):
 
 # --------------------------------------------------------------------------- activations
 class Relu(Layer):
-    """pydtnn/backends/cpu/activations/relu_cpu.py:25-40"""
+    """pydtnn/backends/cpu/activations/relu_cpu.py:25-40.
+
+    With ``Model(enable_relu_folding=True)`` and in TRAIN_MODE the neighbours may do this layer's work in their
+    own kernels: a convolution below hands over ``(y, mask)`` already rectified (``take_folded``), and the
+    layer above announces a dy it has already multiplied by the mask (``take_gated``).  Both are recognised by
+    the identity of the tensor passed to forward / backward, so any other caller gets the plain computation."""
 
     def __init__(self, shape=(1,)):
         super().__init__(shape)
         self.mask = None
         self.y = None
+        self._folded = None
+        self._gated = None
 
     def initialize(self, prev_shape, need_dx=True):
         super().initialize(prev_shape, need_dx)
         self.shape = prev_shape
 
+    def take_folded(self, y, mask):
+        self._folded = (y, mask)
+
+    def take_gated(self, dx):
+        self._gated = dx
+
     def forward(self, x):
+        folded, self._folded = self._folded, None
+        if folded is not None and folded[0] is x:
+            self.y, self.mask = folded
+            return x
         train = self.model.mode == TRAIN_MODE
         self.y, mask = ops.relu(x, with_mask=train)
         if train:
@@ -182,8 +202,17 @@ class Relu(Layer):
         return self.y
 
     def backward(self, dy):
+        gated, self._gated = self._gated, None
         if self.need_dx:
+            if gated is not None and gated is dy:
+                return dy
             return ops.relu_backward(dy, self.mask)
+
+    def gate_for(self, dx_shape):
+        """The mask the layer above may apply to its dx, or None."""
+        if self.need_dx and self.mask is not None and tuple(self.mask.shape) == tuple(dx_shape):
+            return self.mask
+        return None
 
 
 class Softmax(Layer):
@@ -397,12 +426,25 @@ class Conv2D(Layer):
             return dx
 
     # ---------------------------------------------------------------- cg, NHWC (conv_2d_cpu.py:211-227, :399-427)
+    def _folded_forward(self, conv_gemm, x, out_shape, biases_vector):
+        """TRAIN_MODE forward that also does the Relu layer above: y = relu(conv(x) + b) and that layer's mask."""
+        y = torch.empty(out_shape, dtype=x.dtype, device=x.device)
+        mask = torch.empty(out_shape, dtype=torch.int8, device=x.device)
+        conv_gemm(self.weights, x, biases=y, biases_vector=biases_vector, relu=True, relu_mask=mask,
+                  **self._cg_kwargs())
+        self.relu_above.take_folded(y, mask)
+        return y
+
     def _forward_nhwc_cg(self, x):
         if self.model.mode == TRAIN_MODE:
             self.cg_x = x
         biases_vector = self.biases if self.use_bias else None
         self._op(ev.PYDTNN_OPS_FORWARD_CONVGEMM)
-        y = self.cg.conv_gemm_nhwc(self.weights, x, biases_vector=biases_vector, **self._cg_kwargs())
+        if self.model.mode == TRAIN_MODE and self.relu_above is not None:
+            y = self._folded_forward(self.cg.conv_gemm_nhwc, x, (x.shape[0], self.ho, self.wo, self.co),
+                                     biases_vector)
+        else:
+            y = self.cg.conv_gemm_nhwc(self.weights, x, biases_vector=biases_vector, **self._cg_kwargs())
         self._end()
         return y
 
@@ -418,9 +460,12 @@ class Conv2D(Layer):
             self._end()
         if self.need_dx:
             dx = torch.empty((dy.shape[0], self.hi, self.wi, self.ci), dtype=dy.dtype, device=dy.device)
+            gate = self.relu_below.gate_for(dx.shape) if self.relu_below is not None else None
             self._op(ev.PYDTNN_OPS_BACKWARD_DECONV_GEMM)
-            self.cg.deconv_gemm_nhwc(self.weights, dy, dx, **self._cg_kwargs())
+            self.cg.deconv_gemm_nhwc(self.weights, dy, dx, gate=gate, **self._cg_kwargs())
             self._end()
+            if gate is not None:
+                self.relu_below.take_gated(dx)
             return dx
 
     # ---------------------------------------------------------------- cg, NCHW (conv_2d_cpu.py:293-308, :483-510)
@@ -429,7 +474,12 @@ class Conv2D(Layer):
             self.cg_x = x
         biases_vector = self.biases if self.use_bias else None
         self._op(ev.PYDTNN_OPS_FORWARD_CONVGEMM)
-        y = self.cg.conv_gemm_nchw(self.weights, x, biases=None, biases_vector=biases_vector, **self._cg_kwargs())
+        if self.model.mode == TRAIN_MODE and self.relu_above is not None:
+            y = self._folded_forward(self.cg.conv_gemm_nchw, x, (x.shape[0], self.co, self.ho, self.wo),
+                                     biases_vector)
+        else:
+            y = self.cg.conv_gemm_nchw(self.weights, x, biases=None, biases_vector=biases_vector,
+                                       **self._cg_kwargs())
         self._end()
         return y
 
@@ -445,9 +495,12 @@ class Conv2D(Layer):
             self._end()
         if self.need_dx:
             dx = torch.empty((dy.shape[0], self.ci, self.hi, self.wi), dtype=dy.dtype, device=dy.device)
+            gate = self.relu_below.gate_for(dx.shape) if self.relu_below is not None else None
             self._op(ev.PYDTNN_OPS_BACKWARD_DECONV_GEMM)
-            self.cg.deconv_gemm_nchw(self.weights, dy, dx, **self._cg_kwargs())
+            self.cg.deconv_gemm_nchw(self.weights, dy, dx, gate=gate, **self._cg_kwargs())
             self._end()
+            if gate is not None:
+                self.relu_below.take_gated(dx)
             return dx
 
 
@@ -535,10 +588,16 @@ class MaxPool2D(Layer):
 
     def backward(self, dy):
         if self.need_dx:
+            b = dy.shape[0]
             if self.model.tensor_format == PYDTNN_TENSOR_FORMAT_NCHW:
-                return ops.max_pool_2d_bwd_nchw(dy, self.idx_max, dy.shape[0], self.ci, self.hi, self.wi,
-                                                *self._geom())
-            return ops.max_pool_2d_bwd_nhwc(dy, self.idx_max, dy.shape[0], self.hi, self.wi, self.ci, *self._geom())
+                bwd, dims = ops.max_pool_2d_bwd_nchw, (b, self.ci, self.hi, self.wi)
+            else:
+                bwd, dims = ops.max_pool_2d_bwd_nhwc, (b, self.hi, self.wi, self.ci)
+            gate = self.relu_below.gate_for(dims) if self.relu_below is not None else None
+            dx = bwd(dy, self.idx_max, *dims, *self._geom(), gate=gate)
+            if gate is not None:
+                self.relu_below.take_gated(dx)
+            return dx
 
 
 class Flatten(Layer):

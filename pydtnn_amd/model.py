@@ -38,6 +38,12 @@ _DEFAULTS = dict(
     enable_fused_conv_relu=False,
     enable_fused_conv_bn=False,
     enable_fused_conv_bn_relu=False,
+    # Not a reference flag.  In TRAIN_MODE a Relu layer of the top-level sequence is computed by the stores of
+    # its neighbours (the convolution before it, the convolution or pooling layer after it) instead of by two
+    # passes of its own.  Losses, gradients, masks and updated weights are bit-identical either way; what
+    # changes is visible only between the layers: the convolution's forward returns the rectified tensor and
+    # the layer above the Relu returns a dx already multiplied by the mask.  Off by default for that reason.
+    enable_relu_folding=False,
 )
 
 
@@ -79,12 +85,25 @@ class Model:
     def add(self, layer):
         layer.set_model(self)
         need_dx = layer.id > 1
-        prev_shape = self.layers[-1].shape if layer.id > 0 else ()
+        prev = self.layers[-1] if self.layers else None
+        prev_shape = prev.shape if layer.id > 0 else ()
         layer.initialize(prev_shape, need_dx)
         self.nparams += layer.nparams
         self.layers.append(layer)
+        if self.kwargs["enable_relu_folding"]:
+            self._link_relu_neighbours(prev, layer)
         if layer.act:
             self.add(layer.act())
+
+    @staticmethod
+    def _link_relu_neighbours(prev, layer):
+        """Tells a convolution which Relu consumes its output, and a convolution / pooling layer which Relu
+        produced its input, so that their cg kernels can do that Relu's work in TRAIN_MODE.  Only layers of
+        the top-level sequence are linked: there each output has exactly one consumer."""
+        if type(layer) is L.Relu and type(prev) is L.Conv2D:
+            prev.relu_above = layer
+        elif type(prev) is L.Relu and type(layer) in (L.Conv2D, L.MaxPool2D):
+            layer.relu_below = prev
 
     def get_all_layers(self, from_layers=None):
         if from_layers is None:

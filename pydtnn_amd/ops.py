@@ -156,6 +156,11 @@ def eltw_sum(acc, x):
     return chan_eltwise(acc, channels=1, inner=1, residual=x, out=acc)
 
 
+def _need_gate(gate, dx):
+    if gate.dtype != torch.int8 or gate.shape != dx.shape or not gate.is_contiguous():
+        raise TypeError("gate must be a contiguous int8 tensor shaped like dx")
+
+
 def relu(x, with_mask=True):
     """pydtnn/cython_modules/relu_cython.pyx:25-39 -> (max(x, 0), int8 mask)"""
     _need_f32(x)
@@ -197,10 +202,17 @@ def max_pool_2d_fwd_nchw(x, kh, kw, vpadding, hpadding, vstride, hstride, vdilat
 
 
 def max_pool_2d_bwd_nchw(dy, idx_max, n, c, h, w, kh, kw, vpadding, hpadding, vstride, hstride,
-                         vdilation=1, hdilation=1):
-    """pydtnn/cython_modules/max_pool_2d_nchw_cython.pyx:140-166"""
+                         vdilation=1, hdilation=1, gate=None):
+    """pydtnn/cython_modules/max_pool_2d_nchw_cython.pyx:140-166.  ``gate``: int8 mask of a ReLU layer below
+    the pooling layer; dx is stored multiplied by it (that layer's backward, relu_cpu.py:38-40)."""
     _need_f32(dy)
     dx = torch.empty((n, c, h, w), dtype=dy.dtype, device=dy.device)
+    if gate is not None:
+        _need_gate(gate, dx)
+        check(lib().pydtnn_hip_max_pool_2d_bwd_gated(0, f32(dy), ptr(idx_max), f32(dx), ptr(gate), n, c, h, w, kh, kw,
+                                                     vpadding, hpadding, vstride, hstride, vdilation, hdilation,
+                                                     stream_ptr()), "max_pool_bwd_gated")
+        return dx
     check(lib().pydtnn_hip_max_pool_2d_bwd_nchw(f32(dy), ptr(idx_max), f32(dx), n, c, h, w, kh, kw, vpadding,
                                                 hpadding, vstride, hstride, vdilation, hdilation, stream_ptr()),
           "max_pool_bwd")
@@ -220,10 +232,16 @@ def max_pool_2d_fwd_nhwc(x, kh, kw, vpadding, hpadding, vstride, hstride, vdilat
 
 
 def max_pool_2d_bwd_nhwc(dy, idx_max, n, h, w, c, kh, kw, vpadding, hpadding, vstride, hstride,
-                         vdilation=1, hdilation=1):
-    """pydtnn/cython_modules/max_pool_2d_nhwc_cython.pyx:140-166"""
+                         vdilation=1, hdilation=1, gate=None):
+    """pydtnn/cython_modules/max_pool_2d_nhwc_cython.pyx:140-166; ``gate`` as in the NCHW twin."""
     _need_f32(dy)
     dx = torch.empty((n, h, w, c), dtype=dy.dtype, device=dy.device)
+    if gate is not None:
+        _need_gate(gate, dx)
+        check(lib().pydtnn_hip_max_pool_2d_bwd_gated(1, f32(dy), ptr(idx_max), f32(dx), ptr(gate), n, c, h, w, kh, kw,
+                                                     vpadding, hpadding, vstride, hstride, vdilation, hdilation,
+                                                     stream_ptr()), "max_pool_bwd_gated")
+        return dx
     check(lib().pydtnn_hip_max_pool_2d_bwd_nhwc(f32(dy), ptr(idx_max), f32(dx), n, h, w, c, kh, kw, vpadding,
                                                 hpadding, vstride, hstride, vdilation, hdilation, stream_ptr()),
           "max_pool_bwd")

@@ -545,6 +545,111 @@ def test_large_batches_run_as_image_groups(oracle, fmt, d):
         lib.pydtnn_hip_debug_set_tensor_floats_limit(before)
 
 
+# ------------------------------------------------------------------ ReLU done by the neighbouring layers' stores
+
+fold_grid = [D(2, 16, 30, 30, 130, 3, 3, 1, 1, 1, 1, 1, 1), D(5, 8, 19, 23, 20, 5, 3, 2, 1, 2, 1, 1, 1),
+             D(2, 33, 14, 14, 257, 1, 1, 0, 0, 1, 1, 1, 1), D(3, 1, 28, 28, 32, 3, 3, 1, 1, 1, 1, 1, 1),
+             D(16, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1, 1, 1)]  # the last one takes the balanced launch and its fixup
+
+
+@pytest.mark.parametrize("d", fold_grid, ids=repr)
+@pytest.mark.parametrize("fmt", ["NCHW", "NHWC"])
+def test_conv_forward_with_relu_mask_equals_conv_then_relu(ops, cg, fmt, d):
+    """y and mask of the folded call are, bit for bit, what relu_fwd makes of the plain convolution's output."""
+    announce("conv+relu+mask", fmt, d)
+    x, w, b, _ = case(d)
+    if fmt == "NCHW":
+        conv, xs, ws = cg.conv_gemm_nchw, dev(x), dev(w)
+    else:
+        conv, xs, ws = cg.conv_gemm_nhwc, dev(nhwc(x)), dev(w_nhwc(w))
+    plain = conv(ws, xs, biases_vector=dev(b), **_kw(d))
+    y_ref, mask_ref = ops.relu(plain)
+    mask = torch.full(plain.shape, 7, dtype=torch.int8, device="cuda")
+    y = torch.empty_like(plain)
+    conv(ws, xs, biases=y, biases_vector=dev(b), relu=True, relu_mask=mask, **_kw(d))
+    assert torch.equal(y, y_ref)
+    assert torch.equal(mask, mask_ref)
+    assert 0 < int(mask.sum()) < mask.numel()
+
+
+@pytest.mark.parametrize("d", fold_grid, ids=repr)
+@pytest.mark.parametrize("fmt", ["NCHW", "NHWC"])
+def test_conv_dx_with_gate_equals_dx_then_relu_backward(ops, cg, fmt, d):
+    """Both dX routes (as a forward kernel at stride 1, GEMM + col2im / row2im otherwise)."""
+    announce("gated dx", fmt, d)
+    x, w, _, dy = case(d)
+    gate_np = (np.random.default_rng(3).random(x.shape) < 0.6).astype(np.int8)
+    if fmt == "NCHW":
+        deconv, ws, dys, gate = cg.deconv_gemm_nchw, dev(w), dev(dy), dev(gate_np)
+    else:
+        deconv, ws, dys, gate = cg.deconv_gemm_nhwc, dev(w_nhwc(w)), dev(nhwc(dy)), dev(nhwc(gate_np))
+    plain = deconv(ws, dys, torch.empty(gate.shape, device="cuda"), **_kw(d))
+    ref = ops.relu_backward(plain, gate)
+    dx = deconv(ws, dys, torch.full(gate.shape, np.nan, device="cuda"), gate=gate, **_kw(d))
+    assert torch.equal(dx, ref)
+
+
+@pytest.mark.parametrize("fmt", ["NCHW", "NHWC"])
+def test_folded_relu_with_batches_run_as_image_groups(ops, cg, fmt):
+    from pydtnn_amd import native
+    d = D(7, 5, 12, 11, 6, 3, 3, 1, 1, 1, 1)
+    announce("folded relu, image groups", fmt, d)
+    x, w, b, dy = case(d)
+    gate_np = (np.random.default_rng(4).random(x.shape) < 0.5).astype(np.int8)
+    if fmt == "NCHW":
+        conv, deconv, xs, ws, dys, gate = cg.conv_gemm_nchw, cg.deconv_gemm_nchw, dev(x), dev(w), dev(dy), dev(gate_np)
+    else:
+        conv, deconv = cg.conv_gemm_nhwc, cg.deconv_gemm_nhwc
+        xs, ws, dys, gate = dev(nhwc(x)), dev(w_nhwc(w)), dev(nhwc(dy)), dev(nhwc(gate_np))
+    y_ref, mask_ref = ops.relu(conv(ws, xs, biases_vector=dev(b), **_kw(d)))
+    dx_ref = ops.relu_backward(deconv(ws, dys, torch.empty(gate.shape, device="cuda"), **_kw(d)), gate)
+    lib = native.lib()
+    before = lib.pydtnn_hip_debug_set_tensor_floats_limit(3 * max(d.c * d.h * d.w, d.kn * d.ho * d.wo) + 1)
+    try:
+        y, mask = torch.empty_like(y_ref), torch.empty_like(mask_ref)
+        conv(ws, xs, biases=y, biases_vector=dev(b), relu=True, relu_mask=mask, **_kw(d))
+        dx = deconv(ws, dys, torch.empty(gate.shape, device="cuda"), gate=gate, **_kw(d))
+    finally:
+        lib.pydtnn_hip_debug_set_tensor_floats_limit(before)
+    assert torch.equal(y, y_ref) and torch.equal(mask, mask_ref) and torch.equal(dx, dx_ref)
+
+
+def test_relu_mask_and_gate_arguments_are_checked(cg):
+    d = D(2, 3, 8, 8, 4, 3, 3, 1, 1, 1, 1)
+    x, w, b, dy = case(d)
+    y = torch.empty((2, 4, 8, 8), device="cuda")
+    good = torch.empty(y.shape, dtype=torch.int8, device="cuda")
+    with pytest.raises(AssertionError):  # a mask without ReLU
+        cg.conv_gemm_nchw(dev(w), dev(x), biases=y, relu_mask=good, **_kw(d))
+    with pytest.raises(AssertionError):  # wrong shape
+        cg.conv_gemm_nchw(dev(w), dev(x), biases=y, relu=True, relu_mask=good[:1], **_kw(d))
+    with pytest.raises(AssertionError):  # wrong dtype
+        cg.deconv_gemm_nchw(dev(w), dev(dy), torch.empty(x.shape, device="cuda"),
+                            gate=torch.ones(x.shape, device="cuda"), **_kw(d))
+
+
+def test_maxpool_backward_with_gate_equals_backward_then_relu_backward(ops):
+    rng = np.random.default_rng(12)
+    for (shape, kh, kw, s, p) in [((2, 3, 8, 10), 2, 2, 2, 0), ((2, 4, 9, 9), 3, 3, 2, 1), ((2, 3, 9, 11), 2, 2, 2, 0),
+                                  ((1, 2, 9, 12), 3, 3, 3, 0), ((3, 5, 14, 14), 2, 2, 2, 0), ((2, 3, 8, 9), 2, 3, 2, 0)]:
+        announce("gated maxpool bwd", shape, kh, kw, s, p)
+        x = rng.standard_normal(shape).astype(np.float32)
+        gate = dev((rng.random(shape) < 0.6).astype(np.int8))
+        y, idx = ops.max_pool_2d_fwd_nchw(dev(x), kh, kw, p, p, s, s)
+        dy = torch.randn(y.shape, device="cuda")
+        ref = ops.relu_backward(ops.max_pool_2d_bwd_nchw(dy, idx, *shape, kh, kw, p, p, s, s), gate)
+        got = ops.max_pool_2d_bwd_nchw(dy, idx, *shape, kh, kw, p, p, s, s, gate=gate)
+        assert torch.equal(got, ref)
+        xr = dev(nhwc(x))
+        gr = gate.permute(0, 2, 3, 1).contiguous()
+        n, c, h, w = shape
+        y2, idx2 = ops.max_pool_2d_fwd_nhwc(xr, kh, kw, p, p, s, s)
+        dy2 = dy.permute(0, 2, 3, 1).contiguous()
+        ref2 = ops.relu_backward(ops.max_pool_2d_bwd_nhwc(dy2, idx2, n, h, w, c, kh, kw, p, p, s, s), gr)
+        got2 = ops.max_pool_2d_bwd_nhwc(dy2, idx2, n, h, w, c, kh, kw, p, p, s, s, gate=gr)
+        assert torch.equal(got2, ref2)
+
+
 # ------------------------------------------------------------------ host-pointer compatibility ABI
 
 def test_libconvgemm_compat_abi_runs_like_the_reference_shim(oracle):

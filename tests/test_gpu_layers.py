@@ -249,13 +249,14 @@ def test_residual_block_with_fusion(pd, oracle):
 
 # ------------------------------------------------------------------ a small VGG-style training step
 
-def test_small_vgg_training_step_matches_the_oracle_chain(pd, oracle):
+@pytest.mark.parametrize("folding", [False, True], ids=["plain", "relu_folding"])
+def test_small_vgg_training_step_matches_the_oracle_chain(pd, oracle, folding):
     """conv-relu-conv-relu-pool-conv-relu-pool-flatten-fc-relu-fc-softmax, CCE, SGD momentum: one step,
     every gradient and updated weight compared with the oracle run end to end on the CPU."""
-    announce("small vgg step")
+    announce("small vgg step", folding)
     rng = np.random.default_rng(6)
     n, classes = 8, 10
-    model = pd.Model(tensor_format="NCHW", batch_size=n)
+    model = pd.Model(tensor_format="NCHW", batch_size=n, enable_relu_folding=folding)
     model.add(pd.Input(shape=(16, 16, 3)))
     for nf in (8, 8):
         model.add(pd.Conv2D(nfilters=nf, filter_shape=(3, 3), padding=1, activation="relu",
@@ -330,6 +331,72 @@ def test_small_vgg_training_step_matches_the_oracle_chain(pd, oracle):
             w_new, _ = oracle.sgd_update(w.copy(), dw, np.zeros_like(w), np.float32(0.01), np.float32(0.9))
             assert_close(host(l.weights), w_new, tol=1e-5, what=f"{l} updated weights")
             dcur = dx
+
+
+@pytest.mark.parametrize("fmt", ["NCHW", "NHWC"])
+def test_relu_folding_changes_no_bit_of_a_training_run(pd, fmt, monkeypatch):
+    """Two training steps of a small VGG with the Relu layers done by their neighbours' stores (the default) and
+    with separate Relu passes: losses, every gradient and every updated weight are identical, and the folded
+    run really skips the passes (only the FC layer's Relu calls the stand-alone kernels)."""
+    from pydtnn_amd import ops
+    announce("relu folding", fmt)
+    n, classes = 8, 10
+    rng = np.random.default_rng(16)
+    x = dev(rng.random((n, 3, 16, 16) if fmt == "NCHW" else (n, 16, 16, 3)).astype(np.float32))
+    y_targ = dev(np.eye(classes, dtype=np.float32)[rng.integers(0, classes, n)])
+    calls = {"fwd": 0, "bwd": 0}
+    relu, relu_backward = ops.relu, ops.relu_backward
+    monkeypatch.setattr(ops, "relu", lambda *a, **k: (calls.__setitem__("fwd", calls["fwd"] + 1), relu(*a, **k))[1])
+    monkeypatch.setattr(ops, "relu_backward",
+                        lambda *a, **k: (calls.__setitem__("bwd", calls["bwd"] + 1), relu_backward(*a, **k))[1])
+
+    def run(folding):
+        np.random.seed(5)
+        model = pd.Model(tensor_format=fmt, batch_size=n, enable_relu_folding=folding)
+        model.add(pd.Input(shape=(16, 16, 3)))
+        model.add(pd.Conv2D(nfilters=8, filter_shape=(3, 3), padding=1, activation="relu", weights_initializer="he_normal"))
+        model.add(pd.Conv2D(nfilters=8, filter_shape=(3, 3), padding=1, stride=2, weights_initializer="he_normal"))
+        model.add(pd.Relu())  # an explicit Relu layer after a strided convolution (dX by GEMM + col2im / row2im)
+        model.add(pd.Conv2D(nfilters=12, filter_shape=(3, 3), padding=1, activation="relu", weights_initializer="he_normal"))
+        model.add(pd.MaxPool2D(pool_shape=(2, 2), stride=2))
+        model.add(pd.Flatten())
+        model.add(pd.FC(shape=(32,), activation="relu", weights_initializer="he_normal"))
+        model.add(pd.FC(shape=(classes,), activation="softmax", weights_initializer="he_normal"))
+        loss_fn, opt = pd.CategoricalCrossEntropy(), pd.SGD(learning_rate=0.05, momentum=0.9)
+        calls["fwd"] = calls["bwd"] = 0
+        losses = [float(model.train_batch(x, y_targ, loss_fn, opt)) for _ in range(2)]
+        state = {}
+        for l in model.layers:
+            for var, grad in l.grad_vars.items():
+                state[f"{l.id}.{var}"] = getattr(l, var).clone()
+                state[f"{l.id}.{grad}"] = getattr(l, grad).clone()
+        masks = [l.mask.clone() for l in model.layers if l.canonical_name == "Relu"]
+        return losses, state, masks, dict(calls)
+
+    losses_a, state_a, masks_a, calls_a = run(True)
+    losses_b, state_b, masks_b, calls_b = run(False)
+    assert losses_a == losses_b
+    assert state_a.keys() == state_b.keys()
+    for k in state_a:
+        assert torch.equal(state_a[k], state_b[k]), k
+    assert all(torch.equal(a, b) for a, b in zip(masks_a, masks_b))
+    assert calls_b == {"fwd": 8, "bwd": 8}   # four Relu layers, two steps
+    assert calls_a == {"fwd": 2, "bwd": 2}   # only the Relu between the FC layers
+
+
+def test_relu_layer_called_by_hand_ignores_a_stale_hand_over(pd):
+    """The hand-over is recognised by tensor identity: a Relu given any other tensor computes normally."""
+    model = pd.Model(tensor_format="NCHW", batch_size=2, enable_relu_folding=True)
+    model.add(pd.Input(shape=(6, 6, 2)))
+    model.add(pd.Conv2D(nfilters=3, filter_shape=(3, 3), padding=1, activation="relu"))
+    model.mode = pd.TRAIN_MODE
+    conv, relu = model.layers[1], model.layers[2]
+    assert conv.relu_above is relu
+    y = conv.forward(torch.randn(2, 2, 6, 6, device="cuda"))       # hands (y, mask) to relu
+    other = torch.randn(2, 3, 6, 6, device="cuda")
+    out = relu.forward(other)                                       # ... which must not use it for `other`
+    assert torch.equal(out, torch.clamp(other, min=0)) and torch.equal(relu.mask, (other > 0).to(torch.int8))
+    assert relu.forward(y) is not y                                 # the hand-over was dropped, not kept
 
 
 # ------------------------------------------------------------------ BatchNormalization in training mode
