@@ -1021,8 +1021,73 @@ __device__ __forceinline__ void store_tile_nchw(const EpiNchwT<MASKS>& ep, const
     if (has_bias || has_bn) __syncthreads();
 }
 
+// Tile store into a row-major matrix whose columns are the channels.  A tile that lies wholly inside the
+// matrix (the common case) is stored without a test per element, with each column's epilogue parameters
+// fetched once and, for the gated form, with all gate bytes requested before the first store; border
+// tiles take the generic path.
+template <class T, int MASKS>
+__device__ __forceinline__ void store_tile_plain(const EpiPlainT<MASKS>& ep, const floatx16 (&acc)[T::TM][T::TN],
+                                                 int m0, int n0, int split, int tid)
+{
+    if (m0 + T::BM > ep.m_extent || n0 + T::BN > ep.n_extent) {
+        store_tile_generic<T>(ep, acc, m0, n0, split, tid);
+        return;
+    }
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm0 = (wave % T::WGM) * T::WM, wn0 = (wave / T::WGM) * T::WN;
+    const int frag_r = lane & 31, frag_k = lane >> 5;
+    const ChanEpilogue ch = ep.chan;
+    const bool has_bias = ch.bias != nullptr, has_bn = ch.mean != nullptr;
+    const long row0 = m0 + wm0 + 4 * frag_k;  // this lane's first row
+    [[maybe_unused]] float gate[T::TN][T::TM][16];
+    if constexpr (MASKS == kGate) {
+#pragma unroll
+        for (int j = 0; j < T::TN; ++j) {
+            const int8_t* src = ep.masks.gate + (long)split * ep.split_stride + (n0 + wn0 + j * 32 + frag_r);
+#pragma unroll
+            for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    gate[j][i][v] = (float)src[(row0 + i * 32 + 8 * (v / 4) + (v % 4)) * ep.ldc];
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < T::TN; ++j) {
+        const int n = n0 + wn0 + j * 32 + frag_r;
+        const long col = (long)split * ep.split_stride + n;
+        float bias = 0.0f, mean = 0.0f, inv_std = 0.0f, gamma = 0.0f, beta = 0.0f;
+        if (has_bias) bias = ch.bias[n];
+        if (has_bn) {
+            mean = ch.mean[n];
+            inv_std = ch.inv_std[n];
+            gamma = ch.gamma[n];
+            beta = ch.beta[n];
+        }
+#pragma unroll
+        for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const long at = col + (row0 + i * 32 + 8 * (v / 4) + (v % 4)) * ep.ldc;
+                float val = acc[i][j][v];
+                if (has_bias) val += bias;
+                if (has_bn) {
+                    const float t = (val - mean) * inv_std;
+                    val = t * gamma + beta;
+                }
+                if (ch.relu) val = val > 0.0f ? val : 0.0f;
+                if constexpr (MASKS == kGate) val *= gate[j][i][v];
+                ep.out[at] = val;
+                if constexpr (MASKS == kReluMask) ep.masks.relu_mask[at] = val > 0.0f ? 1 : 0;
+            }
+    }
+}
+
 template <class EP>
 struct IsEpiNchw { static constexpr bool value = false; };
+template <class EP>
+struct IsEpiPlain { static constexpr bool value = false; };
+template <int MASKS>
+struct IsEpiPlain<EpiPlainT<MASKS>> { static constexpr bool value = true; };
 template <int MASKS>
 struct IsEpiNchw<EpiNchwT<MASKS>> { static constexpr bool value = true; };
 
@@ -1033,6 +1098,8 @@ __device__ __forceinline__ void store_tile(const EP& ep, const floatx16 (&acc)[T
 {
     if constexpr (IsEpiNchw<EP>::value)
         store_tile_nchw<T>(ep, acc, m0, n0, tid, lds);
+    else if constexpr (IsEpiPlain<EP>::value)
+        store_tile_plain<T>(ep, acc, m0, n0, split, tid);
     else
         store_tile_generic<T>(ep, acc, m0, n0, split, tid);
 }
