@@ -192,11 +192,14 @@ inline bool span_ok_mn(long ld) { return (long)BK * ld * 4 < kMaxSpanBytes; }
 
 template <int MASKS = kNoMasks>
 inline EpiPlainT<MASKS> epi_plain(float* out, long ldc, long split_stride, long m, long n, const ChanEpilogue& chan,
-                                  const ElemMasks& masks = no_masks())
+                                  const ElemMasks& masks = no_masks(), int splits = 1)
 {
     EpiPlainT<MASKS> e;
     e.out = out; e.ldc = ldc; e.split_stride = split_stride; e.m_extent = (int)m; e.n_extent = (int)n; e.chan = chan;
     e.masks = masks;
+    // the branch-free tile store addresses the destination with 32-bit byte offsets
+    const long span = (long)(splits - 1) * split_stride + (m - 1) * ldc + n;
+    e.span = span < (1l << 29) && ldc < (1l << 24) ? span : 0;
     return e;
 }
 
@@ -287,9 +290,43 @@ int conv_fwd_nhwc_t(const ConvGeom& g, const float* w, const float* x, float* y,
     return rc;
 }
 
+// A 1x1 filter at stride 1 without padding makes x itself the (P x C) row matrix and the filter the
+// (C x kn) matrix: a plain GEMM, whose loaders carry no per-pixel offsets or tap masks.
+inline bool pointwise_nhwc(const ConvGeom& g)
+{
+    return g.khw == 1 && g.vstride == 1 && g.hstride == 1 && g.vpadding == 0 && g.hpadding == 0;
+}
+
+int conv_fwd_nhwc_pointwise(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan,
+                            float* ws, size_t ws_bytes, hipStream_t stream, const ElemMasks& masks)
+{
+    const TileSel sel = pick_tile(g.p, g.kn, g.k);
+    int rc = PYDTNN_HIP_OK;
+    WITH_TILE(sel, {
+        if (!span_ok_k(T::BM, g.c, 0, 0) || !span_ok_mn(g.kn)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+        auto al = plain_k<T::BM, false>(x, g.p * g.c, g.c, 0, g.p, 0);
+        auto bl = plain_mn<T::BN>(w, (long)g.c * g.kn, g.kn, 0, g.kn);
+        switch (mask_kind(masks)) {
+        case kGate:
+            rc = launch_balanced<T>(al, bl, epi_plain<kGate>(y, g.kn, 0, g.p, g.kn, chan, masks), g.p, g.kn, g.k, ws,
+                                    ws_bytes, stream);
+            break;
+        case kReluMask:
+            rc = launch_balanced<T>(al, bl, epi_plain<kReluMask>(y, g.kn, 0, g.p, g.kn, chan, masks), g.p, g.kn, g.k,
+                                    ws, ws_bytes, stream);
+            break;
+        default:
+            rc = launch_balanced<T>(al, bl, epi_plain(y, g.kn, 0, g.p, g.kn, chan), g.p, g.kn, g.k, ws, ws_bytes,
+                                    stream);
+        }
+    })
+    return rc;
+}
+
 int conv_fwd_nhwc(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan, float* ws,
                   size_t ws_bytes, hipStream_t stream, const ElemMasks& masks = no_masks())
 {
+    if (pointwise_nhwc(g)) return conv_fwd_nhwc_pointwise(g, w, x, y, chan, ws, ws_bytes, stream, masks);
     if (!taps_supported(g)) return PYDTNN_HIP_ERR_UNSUPPORTED;
     return taps_wide(g) ? conv_fwd_nhwc_t<true>(g, w, x, y, chan, ws, ws_bytes, stream, masks)
                         : conv_fwd_nhwc_t<false>(g, w, x, y, chan, ws, ws_bytes, stream, masks);
@@ -318,7 +355,7 @@ int conv_dw_nchw(const ConvGeom& g, const float* dy, const float* x, const float
         if (!span_ok_k(T::BM, g.howo, sp.si.ips, dy_img)) return PYDTNN_HIP_ERR_UNSUPPORTED;
         auto al = plain_k<T::BM, true>(dy, g.p * g.kn, g.howo, dy_img, g.kn, g.howo);
         al.fd_seg = group_div(g.howo, sp.si.ips);
-        const EpiPlain ep = epi_plain(ws, g.k, out_elems, g.kn, g.k, no_epilogue());
+        const EpiPlain ep = epi_plain(ws, g.k, out_elems, g.kn, g.k, no_epilogue(), no_masks(), sp.splits);
         if (cols) {
             // B(k = (image, pixel), n = row of cols) = cols[n][image*howo + pixel]
             if (!span_ok_k(T::BN, g.p, sp.si.ips, g.howo)) return PYDTNN_HIP_ERR_UNSUPPORTED;
@@ -347,7 +384,7 @@ int conv_dw_nhwc(const ConvGeom& g, const float* dy, const float* x, const float
     WITH_TILE(sel, {
         // B(k = (image, pixel), n = filter) = dy[(image*howo + pixel)*kn + n]
         auto bl = plain_mn<T::BN>(dy, g.p * g.kn, g.kn, (long)g.howo * g.kn, g.kn);
-        const EpiPlain ep = epi_plain(ws, g.kn, out_elems, g.k, g.kn, no_epilogue());
+        const EpiPlain ep = epi_plain(ws, g.kn, out_elems, g.k, g.kn, no_epilogue(), no_masks(), sp.splits);
         if (rows) {
             // A(m = column of rows, k) = rows[(image*howo + pixel)*K + m]
             auto al = plain_mn<T::BM>(rows, g.p * g.k, g.k, (long)g.howo * g.k, g.k);
@@ -649,7 +686,7 @@ int pydtnn_hip_sgemm(int transa, int transb, long m, long n, long k, const float
     const long a_total = transa ? (k - 1) * lda + m : (m - 1) * lda + k;
     const long b_total = transb ? (n - 1) * ldb + k : (k - 1) * ldb + n;
     WITH_TILE(sel, {
-        const EpiPlain ep = epi_plain(dst, dst_ld, m * n, m, n, gemm_chan);
+        const EpiPlain ep = epi_plain(dst, dst_ld, m * n, m, n, gemm_chan, no_masks(), sp.splits);
         if ((!transa && !span_ok_k(T::BM, lda, 0, 0)) || (transa && !span_ok_mn(lda)) ||
             (transb && !span_ok_k(T::BN, ldb, 0, 0)) || (!transb && !span_ok_mn(ldb)))
             return PYDTNN_HIP_ERR_UNSUPPORTED;

@@ -249,6 +249,7 @@ template <int BMN, bool SEG = false>
 struct PlainK {
     using Map = MapK<BMN>;
     static constexpr int NLD = Map::NLD;
+    static constexpr bool kLargeState = false;
     const float* base;
     long total;  // floats in the tensor
     long ld;
@@ -307,6 +308,7 @@ template <int BMN>
 struct PlainMN {
     using Map = MapMN<BMN>;
     static constexpr int NLD = Map::NLD;
+    static constexpr bool kLargeState = false;
     const float* base;
     long total;
     long ld;
@@ -356,6 +358,7 @@ template <int BN, bool WIDE = false>
 struct Im2colNchwMN {
     using Map = MapMN<BN>;
     static constexpr int NLD = Map::NLD;
+    static constexpr bool kLargeState = false;
     const float* x;
     ConvGeom g;
     struct State {
@@ -425,6 +428,8 @@ template <int BN>
 struct Im2colNchwK {
     using Map = MapK<BN>;
     static constexpr int NLD = Map::NLD;
+    // three precomputed words for each of 16 elements: too much for three workgroups per CU
+    static constexpr bool kLargeState = BN >= 256;
     const float* x;
     ConvGeom g;
     struct State {
@@ -486,6 +491,8 @@ template <int BM, bool WIDE = false>
 struct Im2rowNhwcK {
     using Map = MapK<BM>;
     static constexpr int NLD = Map::NLD;
+    // offset and tap mask(s) for each of 16 pixels: too much for three workgroups per CU
+    static constexpr bool kLargeState = BM >= 256;
     static constexpr int NMASK1 = WIDE ? NLD : 1;
     const float* x;
     ConvGeom g;
@@ -553,6 +560,7 @@ template <int BN>
 struct FilterNhwcMN {
     using Map = MapMN<BN>;
     static constexpr int NLD = Map::NLD;
+    static constexpr bool kLargeState = false;
     const float* w;
     ConvGeom g;
     struct State {
@@ -592,6 +600,7 @@ template <int BM>
 struct Im2rowNhwcMN {
     using Map = MapMN<BM>;
     static constexpr int NLD = Map::NLD;
+    static constexpr bool kLargeState = false;
     const float* x;
     ConvGeom g;
     struct State {
@@ -645,12 +654,14 @@ struct Im2rowNhwcMN {
 // instantiations, so that no case carries a test per stored element).
 template <int MASKS>
 struct EpiPlainT {
+    using Unmasked = EpiPlainT<kNoMasks>;
     float* out;
     long ldc;
     long split_stride;
     int m_extent, n_extent;
     ChanEpilogue chan;
     ElemMasks masks;  // only with a single split
+    long span;        // floats from `out` to the end of the last split if that is below 2^29, else 0
     struct Col {
         long off;
         int n;
@@ -677,6 +688,7 @@ using EpiPlain = EpiPlainT<kNoMasks>;
 
 template <int MASKS>
 struct EpiNchwT {
+    using Unmasked = EpiNchwT<kNoMasks>;
     float* out;
     int m_extent;  // output channels
     int howo;
@@ -1021,15 +1033,15 @@ __device__ __forceinline__ void store_tile_nchw(const EpiNchwT<MASKS>& ep, const
     if (has_bias || has_bn) __syncthreads();
 }
 
-// Tile store into a row-major matrix whose columns are the channels.  A tile that lies wholly inside the
-// matrix (the common case) is stored without a test per element, with each column's epilogue parameters
-// fetched once and, for the gated form, with all gate bytes requested before the first store; border
-// tiles take the generic path.
+// Tile store into a row-major matrix whose columns are the channels, written like store_tile_nchw: raw
+// buffer stores whose out-of-range rows / columns carry an offset beyond the descriptor, each column's
+// epilogue parameters fetched once, the gate bytes of a column requested before its first store.  Needs the
+// destination (all splits) inside one descriptor; larger ones (`span == 0`) take the generic path.
 template <class T, int MASKS>
 __device__ __forceinline__ void store_tile_plain(const EpiPlainT<MASKS>& ep, const floatx16 (&acc)[T::TM][T::TN],
                                                  int m0, int n0, int split, int tid)
 {
-    if (m0 + T::BM > ep.m_extent || n0 + T::BN > ep.n_extent) {
+    if (ep.span == 0) {
         store_tile_generic<T>(ep, acc, m0, n0, split, tid);
         return;
     }
@@ -1038,36 +1050,47 @@ __device__ __forceinline__ void store_tile_plain(const EpiPlainT<MASKS>& ep, con
     const int frag_r = lane & 31, frag_k = lane >> 5;
     const ChanEpilogue ch = ep.chan;
     const bool has_bias = ch.bias != nullptr, has_bn = ch.mean != nullptr;
-    const long row0 = m0 + wm0 + 4 * frag_k;  // this lane's first row
-    [[maybe_unused]] float gate[T::TN][T::TM][16];
-    if constexpr (MASKS == kGate) {
-#pragma unroll
-        for (int j = 0; j < T::TN; ++j) {
-            const int8_t* src = ep.masks.gate + (long)split * ep.split_stride + (n0 + wn0 + j * 32 + frag_r);
-#pragma unroll
-            for (int i = 0; i < T::TM; ++i)
-#pragma unroll
-                for (int v = 0; v < 16; ++v)
-                    gate[j][i][v] = (float)src[(row0 + i * 32 + 8 * (v / 4) + (v % 4)) * ep.ldc];
-        }
-    }
+    const rsrc_t out_rsrc = make_rsrc(ep.out, ep.span);
+    [[maybe_unused]] rsrc_t mask_rsrc;
+    if constexpr (MASKS == kGate) mask_rsrc = make_rsrc_bytes(ep.masks.gate, ep.span);
+    if constexpr (MASKS == kReluMask) mask_rsrc = make_rsrc_bytes(ep.masks.relu_mask, ep.span);
+    const int lane_m0 = m0 + wm0 + 4 * frag_k;  // this lane's first row
+    const uint32_t ldc = (uint32_t)ep.ldc;
 #pragma unroll
     for (int j = 0; j < T::TN; ++j) {
         const int n = n0 + wn0 + j * 32 + frag_r;
-        const long col = (long)split * ep.split_stride + n;
+        const bool col_ok = n < ep.n_extent;
+        const int nc = col_ok ? n : 0;
+        // element offset of (split, row 4*frag_k, column n); the uniform row offset rides in the scalar operand
+        const uint32_t e = (uint32_t)((long)split * ep.split_stride) + (uint32_t)(4 * frag_k) * ldc + (uint32_t)nc;
+        const uint32_t off4 = col_ok ? e * 4u : kOob, off1 = col_ok ? e : kOob;
         float bias = 0.0f, mean = 0.0f, inv_std = 0.0f, gamma = 0.0f, beta = 0.0f;
-        if (has_bias) bias = ch.bias[n];
+        if (has_bias) bias = ch.bias[nc];
         if (has_bn) {
-            mean = ch.mean[n];
-            inv_std = ch.inv_std[n];
-            gamma = ch.gamma[n];
-            beta = ch.beta[n];
+            mean = ch.mean[nc];
+            inv_std = ch.inv_std[nc];
+            gamma = ch.gamma[nc];
+            beta = ch.beta[nc];
+        }
+        [[maybe_unused]] float gate[T::TM][16];
+        if constexpr (MASKS == kGate) {
+#pragma unroll
+            for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int r = i * 32 + 8 * (v / 4) + (v % 4);
+                    const bool row_ok = lane_m0 + r < ep.m_extent;
+                    gate[i][v] = (float)(int8_t)__builtin_amdgcn_raw_buffer_load_b8(
+                        mask_rsrc, (int)(row_ok ? off1 : kOob), (int)((uint32_t)(m0 + wm0 + r) * ldc), 0);
+                }
         }
 #pragma unroll
         for (int i = 0; i < T::TM; ++i)
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const long at = col + (row0 + i * 32 + 8 * (v / 4) + (v % 4)) * ep.ldc;
+                const int r = i * 32 + 8 * (v / 4) + (v % 4);
+                const bool row_ok = lane_m0 + r < ep.m_extent;
+                const uint32_t soff = (uint32_t)(m0 + wm0 + r) * ldc;
                 float val = acc[i][j][v];
                 if (has_bias) val += bias;
                 if (has_bn) {
@@ -1075,9 +1098,12 @@ __device__ __forceinline__ void store_tile_plain(const EpiPlainT<MASKS>& ep, con
                     val = t * gamma + beta;
                 }
                 if (ch.relu) val = val > 0.0f ? val : 0.0f;
-                if constexpr (MASKS == kGate) val *= gate[j][i][v];
-                ep.out[at] = val;
-                if constexpr (MASKS == kReluMask) ep.masks.relu_mask[at] = val > 0.0f ? 1 : 0;
+                if constexpr (MASKS == kGate) val *= gate[i][v];
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, val), out_rsrc,
+                                                      (int)(row_ok ? off4 : kOob), (int)(soff * 4u), 0);
+                if constexpr (MASKS == kReluMask)
+                    __builtin_amdgcn_raw_buffer_store_b8((uint8_t)(val > 0.0f ? 1 : 0), mask_rsrc,
+                                                         (int)(row_ok ? off1 : kOob), (int)soff, 0);
             }
     }
 }
@@ -1142,12 +1168,13 @@ __device__ __forceinline__ void gemm_body(const AL& al, const BL& bl, const EP& 
     store_tile<T>(ep, acc, m0, n0, split, tid, As[0]);
 }
 
-// Three workgroups per compute unit need at most 168 registers per lane.  The kernel is built under that
-// limit unless the two loaders' per-thread state alone (precomputed offsets of every element a thread
-// loads) is so large that the limit would spill inside the reduction loop; those run two per CU.
+// Three workgroups per compute unit need at most 168 registers per lane.  The kernels are built under that
+// limit unless a loader's per-thread state (precomputed offsets / masks of 16 elements per step) is so large
+// that the limit would spill inside the reduction loop (`kLargeState`); those are built without it and run
+// two per CU.
 template <class AL, class BL>
 struct FitsThreePerCu {
-    static constexpr bool value = sizeof(typename AL::State) + sizeof(typename BL::State) <= 48 * 4;
+    static constexpr bool value = !(AL::kLargeState || BL::kLargeState);
 };
 
 template <class T, class AL, class BL, class EP>
@@ -1207,7 +1234,7 @@ __host__ __device__ inline long sk_first_unit(int g, long total_units, int sk_bl
 }
 
 template <class T, class AL, class BL, class EP>
-__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))) gemm_streamk_kernel(AL al, BL bl, EP ep, int tiles_m, StreamK sk)
+__device__ __forceinline__ void gemm_streamk_body(const AL& al, const BL& bl, const EP& ep, int tiles_m, const StreamK& sk)
 {
     __shared__ __align__(16) float As[2][BK * (T::BM + kPad)];
     __shared__ __align__(16) float Bs[2][BK * (T::BN + kPad)];
@@ -1275,6 +1302,19 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3
     }
 }
 
+template <class T, class AL, class BL, class EP>
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3)))
+gemm_streamk_kernel(AL al, BL bl, EP ep, int tiles_m, StreamK sk)
+{
+    gemm_streamk_body<T>(al, bl, ep, tiles_m, sk);
+}
+
+template <class T, class AL, class BL, class EP>
+__global__ void __launch_bounds__(kThreads) gemm_streamk_kernel_large_state(AL al, BL bl, EP ep, int tiles_m, StreamK sk)
+{
+    gemm_streamk_body<T>(al, bl, ep, tiles_m, sk);
+}
+
 // grid (sk_tiles, TM*TN*4): a workgroup owns four of the 16*TM*TN accumulator registers of one
 // tile; if the tile was cut, it adds their pieces in ascending reduction order and stores them.
 template <class T, class EP>
@@ -1319,6 +1359,16 @@ struct Residency {
 };
 
 template <class T, class AL, class BL, class EP>
+inline hipError_t streamk_blocks_per_cu(int* per_cu)
+{
+    if constexpr (FitsThreePerCu<AL, BL>::value)
+        return hipOccupancyMaxActiveBlocksPerMultiprocessor(per_cu, gemm_streamk_kernel<T, AL, BL, EP>, kThreads, 0);
+    else
+        return hipOccupancyMaxActiveBlocksPerMultiprocessor(per_cu, gemm_streamk_kernel_large_state<T, AL, BL, EP>,
+                                                            kThreads, 0);
+}
+
+template <class T, class AL, class BL, class EP>
 inline Residency resident_workgroups()
 {
     static Residency cached = {0, 0};
@@ -1326,8 +1376,7 @@ inline Residency resident_workgroups()
         int dev = 0, cus = 0, per_cu = 0;
         if (hipGetDevice(&dev) != hipSuccess ||
             hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-            hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_streamk_kernel<T, AL, BL, EP>, kThreads, 0) !=
-                hipSuccess ||
+            streamk_blocks_per_cu<T, AL, BL, EP>(&per_cu) != hipSuccess ||
             cus <= 0 || per_cu <= 0)
             return cached;
         cached.workgroups = cus * per_cu;
@@ -1347,11 +1396,9 @@ inline int launch_balanced(const AL& al, const BL& bl, const EP& ep, long m, lon
     const long tiles_m = (m + T::BM - 1) / T::BM, tiles_n = (n + T::BN - 1) / T::BN;
     const long tiles = tiles_m * tiles_n;
     if (tiles >= (1l << 31)) return PYDTNN_HIP_ERR_UNSUPPORTED;
-    // the balanced kernel is built for three workgroups per CU; loaders too large for that take the plain grid
-    if constexpr (!FitsThreePerCu<AL, BL>::value) {
-        return launch<T>(al, bl, ep, m, n, no_split(k), 1, stream);
-    } else {
-    const Residency res = resident_workgroups<T, AL, BL, EP>();
+    // The grid, and with it where the reduction ranges are cut, is that of the kernel without byte masks:
+    // a masked launch then adds the same pieces in the same order and gives the same bits.
+    const Residency res = resident_workgroups<T, AL, BL, typename EP::Unmasked>();
     const int resident = res.workgroups;
     const int units = (k + 2 * BK - 1) / (2 * BK);
     bool balanced = resident > 0 && partial && partial_bytes >= streamk_workspace_bytes(resident, T::BM, T::BN) &&
@@ -1372,8 +1419,12 @@ inline int launch_balanced(const AL& al, const BL& bl, const EP& ep, long m, lon
     sk.partial = partial;
     const long total = (long)sk.sk_tiles * units;
     sk.sk_blocks = (int)(total / 4 < resident ? (total / 4 > 0 ? total / 4 : 1) : resident);
-    hipLaunchKernelGGL((gemm_streamk_kernel<T, AL, BL, EP>), dim3((unsigned)resident), dim3(kThreads), 0, stream, al,
-                       bl, ep, (int)tiles_m, sk);
+    if constexpr (FitsThreePerCu<AL, BL>::value)
+        hipLaunchKernelGGL((gemm_streamk_kernel<T, AL, BL, EP>), dim3((unsigned)resident), dim3(kThreads), 0, stream,
+                           al, bl, ep, (int)tiles_m, sk);
+    else
+        hipLaunchKernelGGL((gemm_streamk_kernel_large_state<T, AL, BL, EP>), dim3((unsigned)resident),
+                           dim3(kThreads), 0, stream, al, bl, ep, (int)tiles_m, sk);
     HIP_RETURN_IF_LAUNCH_FAILED();
     if (sk.sk_tiles > 0) {
         hipLaunchKernelGGL((streamk_fixup_kernel<T, EP>), dim3((unsigned)sk.sk_tiles, T::TM * T::TN * 4), dim3(kThreads), 0,
@@ -1381,7 +1432,6 @@ inline int launch_balanced(const AL& al, const BL& bl, const EP& ep, long m, lon
         HIP_RETURN_IF_LAUNCH_FAILED();
     }
     return PYDTNN_HIP_OK;
-    }
 }
 
 }  // namespace gemm
