@@ -1,0 +1,118 @@
+// Filter-gradient launches and the explicit (GEMM + col2im / row2im) input gradient.
+#include "conv_internal.h"
+
+namespace convint {
+
+// ---------------------------------------------------------------- filter gradient
+// mat == nullptr: implicit (x gathered on the fly); otherwise the materialised x_cols / x_rows.
+SplitPlan plan_dw(const ConvGeom& g, int nhwc)
+{
+    const long m = nhwc ? g.k : g.kn, n = nhwc ? g.kn : g.k;
+    const TileSel sel = pick_tile(m, n);
+    return plan_pixel_split(tiles_of(sel, m, n), g.n, g.howo, (long)g.kn * g.k);
+}
+
+int conv_dw_nchw(const ConvGeom& g, const float* dy, const float* x, const float* cols, float* dw, float* ws,
+                 size_t ws_bytes, hipStream_t stream, int accumulate)
+{
+    const SplitPlan sp = plan_dw(g, 0);
+    const long out_elems = (long)g.kn * g.k;
+    if (!ws || ws_bytes < (size_t)sp.splits * out_elems * 4) return PYDTNN_HIP_ERR_WORKSPACE;
+    const TileSel sel = pick_tile(g.kn, g.k);
+    int rc = PYDTNN_HIP_OK;
+    WITH_TILE(sel, {
+        // A(m = filter, k = (image, pixel)) = dy[image][filter][pixel]
+        const long dy_img = (long)g.kn * g.howo;
+        if (!span_ok_k(T::BM, g.howo, sp.si.ips, dy_img)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+        auto al = plain_k<T::BM, true>(dy, g.p * g.kn, g.howo, dy_img, g.kn, g.howo);
+        al.fd_seg = group_div(g.howo, sp.si.ips);
+        const EpiPlain ep = epi_plain(ws, g.k, out_elems, g.kn, g.k, no_epilogue(), no_masks(), sp.splits);
+        if (cols) {
+            // B(k = (image, pixel), n = row of cols) = cols[n][image*howo + pixel]
+            if (!span_ok_k(T::BN, g.p, sp.si.ips, g.howo)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+            auto bl = plain_k<T::BN, true>(cols, (long)g.k * g.p, g.p, g.howo, g.k, g.howo);
+            bl.fd_seg = group_div(g.howo, sp.si.ips);
+            rc = launch<T>(al, bl, ep, g.kn, g.k, sp.si, sp.splits, stream);
+        } else {
+            Im2colNchwK<T::BN> bl;
+            bl.x = x; bl.g = g;
+            bl.g.fd_howo = group_div(g.howo, sp.si.ips);
+            rc = launch<T>(al, bl, ep, g.kn, g.k, sp.si, sp.splits, stream);
+        }
+    })
+    if (rc != PYDTNN_HIP_OK) return rc;
+    return launch_splitk_reduce(ws, dw, g.kn, g.k, out_elems, sp.splits, 0, 0, no_epilogue(), accumulate, stream);
+}
+
+int conv_dw_nhwc(const ConvGeom& g, const float* dy, const float* x, const float* rows, float* dw, float* ws,
+                 size_t ws_bytes, hipStream_t stream, int accumulate)
+{
+    const SplitPlan sp = plan_dw(g, 1);
+    const long out_elems = (long)g.kn * g.k;
+    if (!ws || ws_bytes < (size_t)sp.splits * out_elems * 4) return PYDTNN_HIP_ERR_WORKSPACE;
+    const TileSel sel = pick_tile(g.k, g.kn);
+    int rc = PYDTNN_HIP_OK;
+    WITH_TILE(sel, {
+        // B(k = (image, pixel), n = filter) = dy[(image*howo + pixel)*kn + n]
+        auto bl = plain_mn<T::BN>(dy, g.p * g.kn, g.kn, (long)g.howo * g.kn, g.kn);
+        const EpiPlain ep = epi_plain(ws, g.kn, out_elems, g.k, g.kn, no_epilogue(), no_masks(), sp.splits);
+        if (rows) {
+            // A(m = column of rows, k) = rows[(image*howo + pixel)*K + m]
+            auto al = plain_mn<T::BM>(rows, g.p * g.k, g.k, (long)g.howo * g.k, g.k);
+            rc = launch<T>(al, bl, ep, g.k, g.kn, sp.si, sp.splits, stream);
+        } else {
+            Im2rowNhwcMN<T::BM> al;
+            al.x = x; al.g = g;
+            al.g.fd_howo = group_div(g.howo, sp.si.ips);
+            rc = launch<T>(al, bl, ep, g.k, g.kn, sp.si, sp.splits, stream);
+        }
+    })
+    if (rc != PYDTNN_HIP_OK) return rc;
+    // implicit rows come out in (i, j, c) order; materialised x_rows already has the (c, i, j) order
+    const int perm_c = rows ? 0 : g.c;
+    return launch_splitk_reduce(ws, dw, g.k, g.kn, out_elems, sp.splits, perm_c, g.khw, no_epilogue(), accumulate,
+                                stream);
+}
+
+// `gate` (optional, shaped like dx): dx is stored as gate ? dx : 0; after the scatter-add kernels this is
+// one more pass over dx.
+int conv_dx_i2c(const ConvGeom& g, int nhwc, const float* w, const float* dy, float* dx, float* ws, size_t ws_bytes,
+                hipStream_t stream, const int8_t* gate)
+{
+    const size_t need = (size_t)g.k * g.p * 4;
+    if (!ws || ws_bytes < need) return PYDTNN_HIP_ERR_WORKSPACE;
+    if ((long)g.k * g.p >= (1l << 33)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+    int rc = PYDTNN_HIP_OK;
+    if (!nhwc) {
+        // res(K x P) = W^T (A(m = k, kk = filter) = w[kk*K + m]) * dy_cols (dy seen as a 1x1 im2col)
+        ConvGeom g1;
+        rc = make_conv_geom(&g1, g.n, g.kn, g.ho, g.wo, 1, 1, 1, 0, 0, 1, 1, 1, 1);
+        if (rc != PYDTNN_HIP_OK) return rc;
+        const TileSel sel = pick_tile(g.k, g.p);
+        WITH_TILE(sel, {
+            auto al = plain_mn<T::BM>(w, (long)g.kn * g.k, g.k, 0, g.k);
+            Im2colNchwMN<T::BN> bl;
+            bl.x = dy; bl.g = g1;
+            rc = launch<T>(al, bl, epi_plain(ws, g.p, 0, g.k, g.p, no_epilogue()), g.k, g.p, no_split(g.kn), 1,
+                           stream);
+        })
+        if (rc != PYDTNN_HIP_OK) return rc;
+        rc = launch_col2im_nchw(ws, dx, g, stream);
+        if (rc != PYDTNN_HIP_OK || !gate) return rc;
+        return launch_relu_bwd(dx, gate, dx, (long)g.n * g.c * g.h * g.w, stream);
+    }
+    // res(P x K) = dy_rows (P x kn) * W_rows^T : B(kk = filter, n = k) = w[n*kn + kk]
+    const TileSel sel = pick_tile(g.p, g.k);
+    WITH_TILE(sel, {
+        auto al = plain_k<T::BM, false>(dy, g.p * g.kn, g.kn, 0, g.p, 0);
+        auto bl = plain_k<T::BN, false>(w, (long)g.k * g.kn, g.kn, 0, g.k, 0);
+        rc = launch<T>(al, bl, epi_plain(ws, g.k, 0, g.p, g.k, no_epilogue()), g.p, g.k, no_split(g.kn), 1, stream);
+    })
+    if (rc != PYDTNN_HIP_OK) return rc;
+    rc = launch_row2im_nhwc(ws, dx, g, stream);
+    if (rc != PYDTNN_HIP_OK || !gate) return rc;
+    return launch_relu_bwd(dx, gate, dx, (long)g.n * g.c * g.h * g.w, stream);
+}
+
+
+}  // namespace convint

@@ -1,0 +1,43 @@
+// Implicit-GEMM forward (and stride-1 dX) launches, NCHW.
+#include "conv_internal.h"
+
+namespace convint {
+
+template <bool WIDE>
+int conv_fwd_nchw_t(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan, float* ws,
+                    size_t ws_bytes, hipStream_t stream, const ElemMasks& masks)
+{
+    const TileSel sel = pick_tile(g.kn, g.p, g.k);
+    int rc = PYDTNN_HIP_OK;
+    WITH_TILE(sel, {
+        if (!span_ok_k(T::BM, g.k, 0, 0)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+        auto al = plain_k<T::BM, false>(w, (long)g.kn * g.k, g.k, 0, g.kn, 0);
+        Im2colNchwMN<T::BN, WIDE> bl;
+        bl.x = x; bl.g = g;
+        switch (mask_kind(masks)) {
+        case kGate:
+            rc = launch_balanced<T>(al, bl, epi_nchw<kGate>(y, g.kn, g.howo, g.p, chan, masks), g.kn, g.p, g.k, ws,
+                                    ws_bytes, stream);
+            break;
+        case kReluMask:
+            rc = launch_balanced<T>(al, bl, epi_nchw<kReluMask>(y, g.kn, g.howo, g.p, chan, masks), g.kn, g.p, g.k, ws,
+                                    ws_bytes, stream);
+            break;
+        default:
+            rc = launch_balanced<T>(al, bl, epi_nchw(y, g.kn, g.howo, g.p, chan), g.kn, g.p, g.k, ws, ws_bytes, stream);
+        }
+    })
+    return rc;
+}
+
+// `ws` is optional: without it (or with less than kBalanceBytes) the launch is a plain grid of tiles.
+int conv_fwd_nchw(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan, float* ws,
+                  size_t ws_bytes, hipStream_t stream, const ElemMasks& masks)
+{
+    if (!taps_supported(g)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+    return taps_wide(g) ? conv_fwd_nchw_t<true>(g, w, x, y, chan, ws, ws_bytes, stream, masks)
+                        : conv_fwd_nchw_t<false>(g, w, x, y, chan, ws, ws_bytes, stream, masks);
+}
+
+
+}  // namespace convint
