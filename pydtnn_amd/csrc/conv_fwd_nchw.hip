@@ -3,29 +3,41 @@
 
 namespace convint {
 
+template <class T, class AL, class BL>
+int launch_planes_forward(const AL& al, const BL& bl, const ConvGeom& g, float* y, const ChanEpilogue& chan, float* ws,
+                          size_t ws_bytes, hipStream_t stream, const ElemMasks& masks)
+{
+    switch (mask_kind(masks)) {
+    case kGate:
+        return launch_balanced<T>(al, bl, epi_nchw<kGate>(y, g.kn, g.howo, g.p, chan, masks), g.kn, g.p, g.k, ws,
+                                  ws_bytes, stream);
+    case kReluMask:
+        return launch_balanced<T>(al, bl, epi_nchw<kReluMask>(y, g.kn, g.howo, g.p, chan, masks), g.kn, g.p, g.k, ws,
+                                  ws_bytes, stream);
+    default:
+        return launch_balanced<T>(al, bl, epi_nchw(y, g.kn, g.howo, g.p, chan), g.kn, g.p, g.k, ws, ws_bytes, stream);
+    }
+}
+
 template <bool WIDE>
 int conv_fwd_nchw_t(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan, float* ws,
                     size_t ws_bytes, hipStream_t stream, const ElemMasks& masks)
 {
     const TileSel sel = pick_tile(g.kn, g.p, g.k);
+    // filter rows of a multiple of 4 floats from an aligned tensor: 128-bit loads along the reduction axis
+    const bool quads = !WIDE && g.k % 4 == 0 && aligned16(w);
     int rc = PYDTNN_HIP_OK;
     WITH_TILE(sel, {
         if (!span_ok_k(T::BM, g.k, 0, 0)) return PYDTNN_HIP_ERR_UNSUPPORTED;
-        auto al = plain_k<T::BM, false>(w, (long)g.kn * g.k, g.k, 0, g.kn, 0);
         Im2colNchwMN<T::BN, WIDE> bl;
         bl.x = x; bl.g = g;
-        switch (mask_kind(masks)) {
-        case kGate:
-            rc = launch_balanced<T>(al, bl, epi_nchw<kGate>(y, g.kn, g.howo, g.p, chan, masks), g.kn, g.p, g.k, ws,
-                                    ws_bytes, stream);
-            break;
-        case kReluMask:
-            rc = launch_balanced<T>(al, bl, epi_nchw<kReluMask>(y, g.kn, g.howo, g.p, chan, masks), g.kn, g.p, g.k, ws,
-                                    ws_bytes, stream);
-            break;
-        default:
-            rc = launch_balanced<T>(al, bl, epi_nchw(y, g.kn, g.howo, g.p, chan), g.kn, g.p, g.k, ws, ws_bytes, stream);
+        if constexpr (!WIDE) {
+            if (quads)
+                return launch_planes_forward<T>(plain_k4<T::BM>(w, (long)g.kn * g.k, g.k, g.kn), bl, g, y, chan, ws,
+                                                ws_bytes, stream, masks);
         }
+        rc = launch_planes_forward<T>(plain_k<T::BM, false>(w, (long)g.kn * g.k, g.k, 0, g.kn, 0), bl, g, y, chan, ws,
+                                      ws_bytes, stream, masks);
     })
     return rc;
 }

@@ -8,25 +8,22 @@ int conv_fwd_nhwc_t(const ConvGeom& g, const float* w, const float* x, float* y,
                     size_t ws_bytes, hipStream_t stream, const ElemMasks& masks)
 {
     const TileSel sel = pick_tile(g.p, g.kn, g.k);
+    // channels in multiples of 16 from an aligned tensor: 128-bit loads along the channel axis
+    const bool quads = !WIDE && g.c % 16 == 0 && aligned16(x);
     int rc = PYDTNN_HIP_OK;
     WITH_TILE(sel, {
-        Im2rowNhwcK<T::BM, WIDE> al;
-        al.x = x; al.g = g;
         FilterNhwcMN<T::BN> bl;
         bl.w = w; bl.g = g;
-        switch (mask_kind(masks)) {
-        case kGate:
-            rc = launch_balanced<T>(al, bl, epi_plain<kGate>(y, g.kn, 0, g.p, g.kn, chan, masks), g.p, g.kn, g.k, ws,
-                                    ws_bytes, stream);
-            break;
-        case kReluMask:
-            rc = launch_balanced<T>(al, bl, epi_plain<kReluMask>(y, g.kn, 0, g.p, g.kn, chan, masks), g.p, g.kn, g.k,
-                                    ws, ws_bytes, stream);
-            break;
-        default:
-            rc = launch_balanced<T>(al, bl, epi_plain(y, g.kn, 0, g.p, g.kn, chan), g.p, g.kn, g.k, ws, ws_bytes,
-                                    stream);
+        if constexpr (!WIDE) {
+            if (quads) {
+                Im2rowNhwcK4<T::BM> al;
+                al.x = x; al.g = g;
+                return launch_rows_forward<T>(al, bl, g, y, chan, ws, ws_bytes, stream, masks);
+            }
         }
+        Im2rowNhwcK<T::BM, WIDE> al;
+        al.x = x; al.g = g;
+        rc = launch_rows_forward<T>(al, bl, g, y, chan, ws, ws_bytes, stream, masks);
     })
     return rc;
 }

@@ -177,6 +177,14 @@ inline PlainK<BMN, SEG> plain_k(const float* base, long total, long ld, long ima
 }
 
 template <int BMN>
+inline PlainK4<BMN> plain_k4(const float* base, long total, long ld, long extent)
+{
+    PlainK4<BMN> l;
+    l.base = base; l.total = total; l.ld = ld; l.extent = (int)extent;
+    return l;
+}
+
+template <int BMN>
 inline PlainMN<BMN> plain_mn(const float* base, long total, long ld, long image_stride, long extent)
 {
     PlainMN<BMN> l;
@@ -242,6 +250,26 @@ inline bool dx_as_forward(const ConvGeom& g)
 inline bool pointwise_nhwc(const ConvGeom& g)
 {
     return g.khw == 1 && g.vstride == 1 && g.hstride == 1 && g.vpadding == 0 && g.hpadding == 0;
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+// Row-major forward launch (y is P x kn) with the epilogue variant the masks ask for.
+template <class T, class AL, class BL>
+inline int launch_rows_forward(const AL& al, const BL& bl, const ConvGeom& g, float* y, const ChanEpilogue& chan,
+                               float* ws, size_t ws_bytes, hipStream_t stream, const ElemMasks& masks)
+{
+    switch (mask_kind(masks)) {
+    case kGate:
+        return gemm::launch_balanced<T>(al, bl, epi_plain<kGate>(y, g.kn, 0, g.p, g.kn, chan, masks), g.p, g.kn, g.k, ws,
+                                        ws_bytes, stream);
+    case kReluMask:
+        return gemm::launch_balanced<T>(al, bl, epi_plain<kReluMask>(y, g.kn, 0, g.p, g.kn, chan, masks), g.p, g.kn,
+                                        g.k, ws, ws_bytes, stream);
+    default:
+        return gemm::launch_balanced<T>(al, bl, epi_plain(y, g.kn, 0, g.p, g.kn, chan), g.p, g.kn, g.k, ws, ws_bytes,
+                                        stream);
+    }
 }
 
 // ---------------------------------------------------------------- defined in the conv_*.hip units

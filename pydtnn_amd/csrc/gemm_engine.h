@@ -94,6 +94,14 @@ __device__ __forceinline__ float buf_load(rsrc_t r, uint32_t voff_bytes, uint32_
     return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)voff_bytes, (int)soff_bytes, 0));
 }
 
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+// Four consecutive floats (each dword is range-checked against the descriptor on its own).
+__device__ __forceinline__ floatx4 buf_load4(rsrc_t r, uint32_t voff_bytes, uint32_t soff_bytes)
+{
+    return __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff_bytes, (int)soff_bytes, 0));
+}
+
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
 // Byte offset for buf_load, pushed beyond every descriptor when `invalid_bit` is 1.
@@ -230,6 +238,35 @@ struct MapK {
     }
 };
 
+// MapK4: four lanes cover the 16 reduction indices of a step with one 128-bit load each (k = 4q .. 4q+3,
+// q = tid % 4); 64 rows per pass.  For operands whose reduction axis is contiguous and 16-byte aligned.
+template <int BMN>
+struct MapK4 {
+    static_assert(BK == 16, "four lanes of four floats per step");
+    static constexpr int kMnPerPass = kThreads / 4;
+    static constexpr int NLD = BMN / kMnPerPass;
+    static __device__ __forceinline__ int kq(int tid) { return tid % 4; }
+    static __device__ __forceinline__ int mn(int tid, int e) { return tid / 4 + e * kMnPerPass; }
+    // In the tile layout (k, k+2) share a 64-bit word: the quad goes out as {k0, k2} and {k1, k3}.
+    template <int PART, int PARTS>
+    static __device__ __forceinline__ void store_part(float* lds, const floatx4 (&r)[NLD], int tid)
+    {
+        constexpr int P = LdsTile<BMN>::kRowPitch;
+        float* base = lds + (2 * (tid % 4)) * P + (tid / 4) * 2;
+#pragma unroll
+        for (int e = 0; e < NLD; ++e)
+            if (e * PARTS / NLD == PART) {
+                float* p = base + e * kMnPerPass * 2;
+                *reinterpret_cast<floatx2*>(p) = floatx2{r[e][0], r[e][2]};
+                *reinterpret_cast<floatx2*>(p + P) = floatx2{r[e][1], r[e][3]};
+            }
+    }
+    static __device__ __forceinline__ void store(float* lds, const floatx4 (&r)[NLD], int tid)
+    {
+        store_part<0, 1>(lds, r, tid);
+    }
+};
+
 // Every loader exposes
 //   State            per-thread data fixed for the whole tile
 //   Iter             per-thread / per-wave data of one reduction step
@@ -250,6 +287,7 @@ struct PlainK {
     using Map = MapK<BMN>;
     static constexpr int NLD = Map::NLD;
     static constexpr bool kLargeState = false;
+    using Reg = float;
     const float* base;
     long total;  // floats in the tensor
     long ld;
@@ -304,11 +342,61 @@ struct PlainK {
 // elem(mn, k) = base[image*image_stride + k*ld + mn]   (mn contiguous).  The descriptor is re-based to
 // row k0 at every step and sized to end with row kend-1, so rows of a partial step beyond the
 // reduction range read as zero; only BK*ld*4 < 2 GiB is needed (checked on the host).
+// PlainK with 128-bit loads: elem(mn, k) = base[mn*ld + k], one segment.  Needs ld % 4 == 0, a 16-byte
+// aligned base and reduction ranges that end on multiples of 4 (checked on the host).
+template <int BMN>
+struct PlainK4 {
+    using Map = MapK4<BMN>;
+    using Reg = floatx4;
+    static constexpr int NLD = Map::NLD;
+    static constexpr bool kLargeState = false;
+    const float* base;
+    long total;  // floats in the tensor
+    long ld;
+    int extent;  // valid mn range
+    struct State {
+        rsrc_t rsrc;
+        uint32_t rowoff[NLD];  // byte offset of (row e, this thread's quad)
+    };
+    struct Iter {
+        uint32_t voff;  // 0, or kOob when this thread's quad lies beyond kend
+        uint32_t soff;  // uniform byte offset of the step
+    };
+    __device__ __forceinline__ void init(State& s, int origin, int /*image0*/, int tid) const
+    {
+        const long first = (long)origin * ld;
+        s.rsrc = make_rsrc(base + first, total - first);
+        const int rows = min(BMN, extent - origin);
+#pragma unroll
+        for (int e = 0; e < NLD; ++e) {
+            const int row = min(Map::mn(tid, e), rows - 1);
+            s.rowoff[e] = (uint32_t)(row * ld + 4 * Map::kq(tid)) * 4u;
+        }
+    }
+    __device__ __forceinline__ void begin(const State&, Iter& it, int k0, int kend) const
+    {
+        it.voff = k0 + 4 * Map::kq(threadIdx.x) >= kend ? kOob : 0u;
+        it.soff = (uint32_t)k0 * 4u;
+    }
+    template <int E>
+    __device__ __forceinline__ floatx4 elem(const State& s, const Iter& it, int, int) const
+    {
+        return buf_load4(s.rsrc, s.rowoff[E] + it.voff, it.soff);
+    }
+    __device__ __forceinline__ void store(float* lds, const floatx4 (&r)[NLD], int tid) const { Map::store(lds, r, tid); }
+    template <int PART, int PARTS>
+    __device__ __forceinline__ void store_part(float* lds, const floatx4 (&r)[NLD], int tid) const
+    {
+        Map::template store_part<PART, PARTS>(lds, r, tid);
+    }
+};
+
 template <int BMN>
 struct PlainMN {
     using Map = MapMN<BMN>;
     static constexpr int NLD = Map::NLD;
     static constexpr bool kLargeState = false;
+    using Reg = float;
     const float* base;
     long total;
     long ld;
@@ -359,6 +447,7 @@ struct Im2colNchwMN {
     using Map = MapMN<BN>;
     static constexpr int NLD = Map::NLD;
     static constexpr bool kLargeState = false;
+    using Reg = float;
     const float* x;
     ConvGeom g;
     struct State {
@@ -430,6 +519,7 @@ struct Im2colNchwK {
     static constexpr int NLD = Map::NLD;
     // three precomputed words for each of 16 elements: too much for three workgroups per CU
     static constexpr bool kLargeState = BN >= 256;
+    using Reg = float;
     const float* x;
     ConvGeom g;
     struct State {
@@ -493,6 +583,7 @@ struct Im2rowNhwcK {
     static constexpr int NLD = Map::NLD;
     // offset and tap mask(s) for each of 16 pixels: too much for three workgroups per CU
     static constexpr bool kLargeState = BM >= 256;
+    using Reg = float;
     static constexpr int NMASK1 = WIDE ? NLD : 1;
     const float* x;
     ConvGeom g;
@@ -555,12 +646,74 @@ struct Im2rowNhwcK {
     }
 };
 
+// Im2rowNhwcK with 128-bit loads, for c % 16 == 0 and kh*kw <= 31: the reduction index is (tap, channel)
+// with the channel fastest, so a step of 16 lies inside one tap; that tap is decomposed once per step on
+// the scalar ALU and its offset rides in the load's scalar operand, and a thread keeps the pixel offset
+// and tap mask of BM/64 rows instead of BM/16.  The descriptor starts `lead` floats before x so that the
+// per-thread offset is never negative.
+template <int BM>
+struct Im2rowNhwcK4 {
+    using Map = MapK4<BM>;
+    using Reg = floatx4;
+    static constexpr int NLD = Map::NLD;
+    static constexpr bool kLargeState = false;
+    const float* x;
+    ConvGeom g;
+    struct State {
+        rsrc_t rsrc;
+        uint32_t base[NLD];  // byte offset of ((img*h + ih0)*w + iw0)*c + 4q from the shifted start
+        uint32_t inv0[NLD];  // combined tap mask of the row's pixel (bit 31 always set)
+    };
+    struct Iter {
+        uint32_t soff;  // byte offset of (di*w + dj)*c + first channel of the step
+        uint32_t sh;    // 31 - tap index (0 beyond kend: selects the always-set bit)
+    };
+    __device__ __forceinline__ void init(State& s, int origin, int /*image*/, int tid) const
+    {
+        const long lead = (long)(g.vpadding * g.w + g.hpadding) * g.c;
+        s.rsrc = make_rsrc(x - lead, (long)g.n * g.c * g.h * g.w + lead);
+#pragma unroll
+        for (int e = 0; e < NLD; ++e) {
+            long m = (long)origin + Map::mn(tid, e);
+            m = m < g.p ? m : g.p - 1;
+            const int img = (int)(m / g.howo);
+            const int pp = (int)(m - (long)img * g.howo);
+            const int yy = pp / g.wo, xx = pp - yy * g.wo;
+            const int ih0 = yy * g.vstride - g.vpadding;
+            const int iw0 = xx * g.hstride - g.hpadding;
+            s.base[e] = (uint32_t)((((long)img * g.h + ih0) * g.w + iw0) * g.c + lead + 4 * Map::kq(tid)) * 4u;
+            s.inv0[e] = tap_mask_combined(g, ih0, iw0);
+        }
+    }
+    __device__ __forceinline__ void begin(const State&, Iter& it, int k0, int kend) const
+    {
+        const uint32_t ij = fd_div((uint32_t)k0, g.fd_c);
+        const uint32_t c0 = (uint32_t)k0 - ij * g.c;
+        const uint32_t ii = fd_div(ij, g.fd_kw);
+        const uint32_t jj = ij - ii * g.kw;
+        it.soff = (uint32_t)(((int)ii * g.vdilation * g.w + (int)jj * g.hdilation) * g.c + (int)c0) * 4u;
+        it.sh = k0 < kend ? 31u - ij : 0u;
+    }
+    template <int E>
+    __device__ __forceinline__ floatx4 elem(const State& s, const Iter& it, int, int) const
+    {
+        return buf_load4(s.rsrc, ((s.inv0[E] << it.sh) & kOob) | s.base[E], it.soff);
+    }
+    __device__ __forceinline__ void store(float* lds, const floatx4 (&r)[NLD], int tid) const { Map::store(lds, r, tid); }
+    template <int PART, int PARTS>
+    __device__ __forceinline__ void store_part(float* lds, const floatx4 (&r)[NLD], int tid) const
+    {
+        Map::template store_part<PART, PARTS>(lds, r, tid);
+    }
+};
+
 // Filter in NHWC layout (c, kh, kw, kn) read as B(k in (i,j,c) order, n = filter).
 template <int BN>
 struct FilterNhwcMN {
     using Map = MapMN<BN>;
     static constexpr int NLD = Map::NLD;
     static constexpr bool kLargeState = false;
+    using Reg = float;
     const float* w;
     ConvGeom g;
     struct State {
@@ -601,6 +754,7 @@ struct Im2rowNhwcMN {
     using Map = MapMN<BM>;
     static constexpr int NLD = Map::NLD;
     static constexpr bool kLargeState = false;
+    using Reg = float;
     const float* x;
     ConvGeom g;
     struct State {
@@ -735,7 +889,7 @@ __device__ __forceinline__ int xcd_remap(int bid, int nblocks)
 // elements E with E*(BK/2)/NLD == J.
 template <int J, int E, class L>
 __device__ __forceinline__ void group_load(const L& l, const typename L::State& s, const typename L::Iter& it,
-                                           float (&r)[L::NLD], int k0, int kend)
+                                           typename L::Reg (&r)[L::NLD], int k0, int kend)
 {
     if constexpr (E < L::NLD) {
         if constexpr (E * (BK / 2) / L::NLD == J) r[E] = l.template elem<E>(s, it, k0, kend);
@@ -745,7 +899,7 @@ __device__ __forceinline__ void group_load(const L& l, const typename L::State& 
 
 template <int E, class L>
 __device__ __forceinline__ void load_all(const L& l, const typename L::State& s, const typename L::Iter& it,
-                                         float (&r)[L::NLD], int k0, int kend)
+                                         typename L::Reg (&r)[L::NLD], int k0, int kend)
 {
     if constexpr (E < L::NLD) {
         r[E] = l.template elem<E>(s, it, k0, kend);
@@ -778,10 +932,10 @@ __device__ __forceinline__ void request_operands(uint32_t a_base, uint32_t b_bas
 // LDS buffer it does not read.
 template <class AL, class BL>
 struct StepRegs {
-    float (&ra)[AL::NLD];
-    float (&rb)[BL::NLD];
-    const float (&sa)[AL::NLD];
-    const float (&sb)[BL::NLD];
+    typename AL::Reg (&ra)[AL::NLD];
+    typename BL::Reg (&rb)[BL::NLD];
+    const typename AL::Reg (&sa)[AL::NLD];
+    const typename BL::Reg (&sb)[BL::NLD];
     float* a_store;
     float* b_store;
     int tid;
@@ -861,7 +1015,8 @@ __device__ __forceinline__ void tile_mainloop(const AL& al, const BL& bl, int m0
 
     // Register sets: during step s the loads of tile s+2 go to set (s & 1) while set ((s+1) & 1),
     // filled during step s-1 with tile s+1, is stored to the LDS buffer that step s does not read.
-    float ra0[AL::NLD], rb0[BL::NLD], ra1[AL::NLD], rb1[BL::NLD];
+    typename AL::Reg ra0[AL::NLD], ra1[AL::NLD];
+    typename BL::Reg rb0[BL::NLD], rb1[BL::NLD];
     {   // tiles 0 and 1 (any kend, including an empty range: everything reads as zero)
         typename AL::Iter ai;
         typename BL::Iter bi;
