@@ -276,7 +276,11 @@ size_t pydtnn_hip_conv_workspace_bytes(int op, int nhwc, int b, int c, int h, in
         PYDTNN_HIP_OK)
         return 0;
     switch (op) {
-        case PYDTNN_HIP_OP_DW: return (size_t)plan_dw(g, nhwc).splits * g.kn * g.k * 4;
+        case PYDTNN_HIP_OP_DW: {
+            // partial sums of the split, or the partial tiles of the balanced launch
+            const size_t split = (size_t)plan_dw(g, nhwc).splits * g.kn * g.k * 4;
+            return split > kBalanceBytes ? split : kBalanceBytes;
+        }
         case PYDTNN_HIP_OP_FWD: return kBalanceBytes;  // optional: a smaller or absent workspace only costs speed
         case PYDTNN_HIP_OP_DX:
             return dx_as_forward(g) ? (((size_t)g.kn * g.k * 4 + 255) & ~(size_t)255) + kBalanceBytes

@@ -1544,9 +1544,13 @@ inline size_t streamk_workspace_bytes(int resident, int bm, int bn) { return (si
 
 // C = A*B over the full reduction range [0, k), balanced as described above when that pays and
 // `partial` is large enough; otherwise the plain grid of whole tiles.
+// `must_balance`: the caller has no use for the plain grid (few tiles, long reduction); returns
+// kNotBalanced without launching when the balanced form is not possible.
+constexpr int kNotBalanced = -1;
+
 template <class T, class AL, class BL, class EP>
 inline int launch_balanced(const AL& al, const BL& bl, const EP& ep, long m, long n, int k, float* partial,
-                           size_t partial_bytes, hipStream_t stream)
+                           size_t partial_bytes, hipStream_t stream, bool must_balance = false)
 {
     const long tiles_m = (m + T::BM - 1) / T::BM, tiles_n = (n + T::BN - 1) / T::BN;
     const long tiles = tiles_m * tiles_n;
@@ -1558,14 +1562,14 @@ inline int launch_balanced(const AL& al, const BL& bl, const EP& ep, long m, lon
     const int units = (k + 2 * BK - 1) / (2 * BK);
     bool balanced = resident > 0 && partial && partial_bytes >= streamk_workspace_bytes(resident, T::BM, T::BN) &&
                     tiles % resident != 0 && units >= 8;
-    if (balanced) {
+    if (balanced && !must_balance) {
         // A plain grid keeps every compute unit busy for ceil(tiles / CUs) tile times; balancing is
         // worth its partial-tile traffic only when more than a twentieth of that is idle.
         const double per_cu = (double)tiles / res.cus;
         const double rounds = (double)((tiles + res.cus - 1) / res.cus);
         balanced = per_cu / rounds < 0.95;
     }
-    if (!balanced) return launch<T>(al, bl, ep, m, n, no_split(k), 1, stream);
+    if (!balanced) return must_balance ? kNotBalanced : launch<T>(al, bl, ep, m, n, no_split(k), 1, stream);
     StreamK sk;
     sk.tiles = (int)tiles;
     sk.sk_tiles = (int)(tiles % resident);

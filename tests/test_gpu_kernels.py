@@ -294,6 +294,20 @@ def test_dw_split_over_several_images_and_chunks(cg, oracle):
         assert_close(host(dw2).transpose(3, 0, 1, 2), dw_ref, what="dw nhwc")
 
 
+def test_dw_with_many_tiles_takes_the_balanced_launch(cg, oracle):
+    """512 x 4608 filter matrix = 144 tiles: the reduction units of all tiles are dealt evenly over the chip and
+    pieces of a tile summed by the fixup kernel (NCHW); the result must not depend on that."""
+    for d in [D(4, 512, 8, 8, 512, 3, 3, 1, 1, 1, 1), D(6, 512, 14, 14, 512, 3, 3, 1, 1, 1, 1)]:
+        announce("dw balanced", d)
+        x, w, _, dy = case(d)
+        p = oracle.ConvParams(*d.geom())
+        _, x_cols = oracle.conv2d_forward_nchw_i2c(x, w, None, p)
+        dw_ref, _, _ = oracle.conv2d_backward_nchw_i2c(dy, x_cols, w, x.shape, p, need_dx=False)
+        dw = torch.full(w.shape, float("nan"), device="cuda")
+        cg.conv_gemm_nchw(dev(dy), dev(x), biases=dw, trans=True, **_kw(d))
+        assert_close(host(dw), dw_ref, what="dw nchw, balanced")
+
+
 # ------------------------------------------------------------------ elementwise kernels
 
 def test_chan_eltwise_matches_oracle(ops, oracle):
