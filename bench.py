@@ -177,6 +177,17 @@ def run_cfg2(torch, pd, args):
         extra[second + "_gbs"] = round(stream_bytes / (t2.median_ms() * 1e-3) / 1e9, 1)
     extra["im2col_pct_hbm_peak"] = round(100 * extra["im2col_gbs"] / HBM_PEAK_GBS, 1)
     extra["col2im_pct_hbm_peak"] = round(100 * extra["col2im_gbs"] / HBM_PEAK_GBS, 1)
+    # the bias -> BN(inference) -> ReLU epilogue as a stand-alone pass over y (2 * bytes(y)); fused into the
+    # GEMM's store it costs no traffic at all
+    ch = [torch.rand(256, device="cuda") + 0.5 for _ in range(5)]
+    t3 = Timer(torch)
+    for i in range(6):
+        fn = lambda: ops.chan_eltwise(xd, channels=256, inner=56 * 56, bias=ch[0], bn=(ch[1], ch[2], ch[3], ch[4]),
+                                      relu=True, out=back)
+        fn() if i == 0 else t3(fn)
+    torch.cuda.synchronize()
+    extra["epilogue_gbs"] = round(2 * x.nbytes / (t3.median_ms() * 1e-3) / 1e9, 1)
+    extra["epilogue_pct_hbm_peak"] = round(100 * extra["epilogue_gbs"] / HBM_PEAK_GBS, 1)
     del mat, back
     roofline = {"bound": "mfma", "kernel": "gemm_streamk_kernel<128x128, PlainK, Im2colNchwMN, EpiNchw> + streamk_fixup_kernel (forward)",
                 "achieved": round(achieved, 3), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
@@ -348,8 +359,16 @@ def main():
         del src, dst
 
     cpu = None
-    if not args.no_cpu_baseline and args.workload == "cfg2":
-        cpu = cpu_baseline_cfg2()
+    if not args.no_cpu_baseline:
+        from bench_configs import cpu_baseline_other, cpu_baseline_vgg16
+        if args.workload == "cfg2":
+            cpu = cpu_baseline_cfg2()
+            if not args.no_vgg16:
+                extra["vgg16_cpu_baseline"] = cpu_baseline_vgg16()
+        elif args.workload == "cfg5":
+            cpu = cpu_baseline_vgg16()
+        else:
+            cpu = cpu_baseline_other(args.workload)
 
     print(json.dumps({
         "metric": METRIC, "value": round(value, 1), "unit": unit, "n_gpus": 1, "steps": args.steps,

@@ -66,6 +66,157 @@ def build_cfg4_model(pd, torch, ws, bns, fused=True):
     return model
 
 
+# --------------------------------------------------------------------------- CPU baselines
+# The reference's CPU route (Cython im2col / im2row with OpenMP, NumPy @, separate bias / BN / ReLU passes)
+# as restated by the oracle, timed on this host.  Reported beside the GPU figure, never a target.
+
+def _cpu_cores():
+    import os
+    return int(os.environ.get("OMP_NUM_THREADS", min(16, os.cpu_count() or 1)))
+
+
+def _time_cpu(fn, budget_s, max_reps):
+    """One warm-up, then repetitions until `budget_s` of work or `max_reps`; returns (best, reps, total)."""
+    import time
+    from threadpoolctl import threadpool_limits
+    times = []
+    with threadpool_limits(limits=_cpu_cores()):
+        fn()
+        stop = time.perf_counter() + budget_s
+        while len(times) < max_reps and (not times or time.perf_counter() < stop):
+            t0 = time.perf_counter()
+            fn()
+            times.append(time.perf_counter() - t0)
+    return min(times), len(times), sum(times)
+
+
+def _cpu_report(value, unit, what, best, reps, total):
+    return {"value": round(value, 1), "unit": unit, "cores": _cpu_cores(), "kind": "port",
+            "sample": f"{what}, 1 warm-up then best of {reps} ({best:.3g} s each, {total:.1f} s in all); C/OpenMP "
+                      f"gathers and NumPy(OpenBLAS) matmul limited to {_cpu_cores()} threads"}
+
+
+def cpu_baseline_other(workload):
+    from oracle import cpu_ref
+    if workload == "cfg1":
+        x, w, b = make_cfg1()
+        p = cpu_ref.ConvParams(3, 3, 1, 1)
+        best, reps, total = _time_cpu(lambda: cpu_ref.conv2d_forward_nhwc_i2c(x, w, b, p), 10.0, 2000)
+        return _cpu_report(2.0 * 32 * 9 * 64 * 28 * 28 / best / 1e9, "GFLOP/s", "all 64 images of cfg1, forward", best,
+                           reps, total)
+    if workload == "cfg3":
+        x, w, b = make_cfg3()
+        p = cpu_ref.ConvParams(11, 11, 0, 0, 4, 4)
+
+        def fwd():
+            y, _ = cpu_ref.conv2d_forward_nchw_i2c(x, w, b, p)
+            cpu_ref.relu(y)
+
+        best, reps, total = _time_cpu(fwd, 12.0, 100)
+        return _cpu_report(2.0 * 96 * 363 * 64 * 55 * 55 / best / 1e9, "GFLOP/s",
+                           "all 64 images of cfg3, forward + bias + ReLU as separate passes", best, reps, total)
+    if workload == "cfg4":
+        import numpy as np
+        x, ws, bns = make_cfg4()
+        geoms = [cpu_ref.ConvParams(1, 1), cpu_ref.ConvParams(3, 3, 1, 1), cpu_ref.ConvParams(1, 1)]
+        stats = [(mean, (1.0 / np.sqrt(var + 1e-5)).astype(np.float32), gamma, beta) for gamma, beta, mean, var in bns]
+
+        def block():
+            cur = x
+            for i, (w, p, bn) in enumerate(zip(ws, geoms, stats)):
+                cur, _ = cpu_ref.conv2d_forward_nhwc_i2c(cur, w, None, p)
+                cur = cpu_ref.fused_epilogue(cur, "NHWC", bn=bn, relu_flag=i < 2)
+            cur = cpu_ref.eltw_sum(cur, x)
+            cpu_ref.relu(cur)
+
+        best, reps, total = _time_cpu(block, 12.0, 100)
+        flop = 2.0 * 64 * 56 * 56 * (256 * 64 + 576 * 64 + 64 * 256)
+        return _cpu_report(flop / best / 1e9, "GFLOP/s",
+                           "all 64 images of cfg4, unfused layers (conv, BN, ReLU, add as separate passes)", best, reps,
+                           total)
+    raise ValueError(workload)
+
+
+VGG16_PLAN = [(3, 64), (64, 64), "M", (64, 128), (128, 128), "M", (128, 256), (256, 256), (256, 256), "M",
+              (256, 512), (512, 512), (512, 512), "M", (512, 512), (512, 512), (512, 512), "M"]
+
+
+def cpu_baseline_vgg16(sample_images=16, budget_s=14.0):
+    """One VGG16 training step (forward, loss, backward, SGD with momentum) of the oracle on `sample_images`
+    images.  The FC and optimizer parts do not shrink with the batch, so the rate of a sample is a lower bound
+    of the full-batch rate."""
+    import numpy as np
+    from oracle import cpu_ref
+    rng = np.random.default_rng(0)
+    n = sample_images
+    x0 = rng.random((n, 3, 224, 224), dtype=np.float32)
+    y_targ = np.eye(1000, dtype=np.float32)[rng.integers(0, 1000, n)]
+    p3 = cpu_ref.ConvParams(3, 3, 1, 1)
+    params = []
+    for spec in VGG16_PLAN:
+        if spec != "M":
+            ci, co = spec
+            params.append([he_normal(rng, (co, ci, 3, 3), ci * 9), np.zeros(co, np.float32)])
+    for fi, fo in [(25088, 4096), (4096, 4096), (4096, 1000)]:
+        params.append([he_normal(rng, (fi, fo), fi), np.zeros(fo, np.float32)])
+    velocity = [[np.zeros_like(w), np.zeros_like(b)] for w, b in params]
+
+    def step():
+        saved, cur, pi = [], x0, 0
+        for spec in VGG16_PLAN:
+            if spec == "M":
+                shape = cur.shape
+                cur, idx = cpu_ref.max_pool_2d_fwd_nchw(cur, 2, 2, 0, 0, 2, 2)
+                saved.append(("pool", shape, idx))
+            else:
+                w, b = params[pi]
+                shape = cur.shape
+                cur, cols = cpu_ref.conv2d_forward_nchw_i2c(cur, w, b, p3)
+                cur, mask = cpu_ref.relu(cur)
+                saved.append(("conv", pi, shape, cols, mask))
+                pi += 1
+        flat_shape = cur.shape
+        cur = cur.reshape(n, -1)
+        fcs = []
+        for j in range(3):
+            w, b = params[pi + j]
+            fcs.append(cur)
+            cur = cpu_ref.fc_forward(cur, w, b)
+            if j < 2:
+                cur, mask = cpu_ref.relu(cur)
+                fcs.append(mask)
+        y = cpu_ref.softmax_forward(cur)
+        _, d = cpu_ref.categorical_cross_entropy(y, y_targ, n)
+        d = cpu_ref.softmax_backward(d, y)
+        grads = {}
+        for j in (2, 1, 0):
+            if j < 2:
+                d = d * fcs.pop()
+            w, _ = params[pi + j]
+            dw, db, d = cpu_ref.fc_backward(d, fcs.pop(), w)
+            grads[pi + j] = (dw, db)
+        d = d.reshape(flat_shape)
+        for item in reversed(saved):
+            if item[0] == "pool":
+                _, shape, idx = item
+                d = cpu_ref.max_pool_2d_bwd_nchw(d, idx, *shape, 2, 2, 0, 0, 2, 2)
+            else:
+                _, k, shape, cols, mask = item
+                d = d * mask
+                dw, db, d = cpu_ref.conv2d_backward_nchw_i2c(d, cols, params[k][0], shape, p3, need_dx=k > 0)
+                grads[k] = (dw, db)
+        for k, (dw, db) in grads.items():
+            params[k][0], velocity[k][0] = cpu_ref.sgd_update(params[k][0], dw.astype(np.float32), velocity[k][0],
+                                                              np.float32(0.01), np.float32(0.9))
+            params[k][1], velocity[k][1] = cpu_ref.sgd_update(params[k][1], db.astype(np.float32), velocity[k][1],
+                                                              np.float32(0.01), np.float32(0.9))
+
+    best, reps, total = _time_cpu(step, budget_s, 4)
+    return _cpu_report(n / best, "img/s", f"{n} of 64 images of cfg5 (one VGG16 training step; the FC and SGD parts "
+                                          f"do not shrink with the sample, so this understates the full batch)",
+                       best, reps, total)
+
+
 def run_other(torch, pd, args, Timer, timed_steps):
     from pydtnn_amd.conv_gemm import ConvGemm
     cg = ConvGemm()

@@ -54,6 +54,75 @@ __global__ void __launch_bounds__(kThreads) chan_eltwise_vec4_kernel(const float
     y[i4] = v;
 }
 
+// The two layouts that matter, without a division per element and with the per-channel parameters fetched
+// once per workgroup / thread instead of once per element.
+//
+// Planes (NCHW, inner % 4 == 0): grid.y walks the (image, channel) planes, so the channel is uniform in a
+// workgroup; grid.x * 256 threads walk one plane's float4s.
+__global__ void __launch_bounds__(kThreads) chan_eltwise_planes_kernel(const float4* __restrict__ x,
+                                                                      const float4* __restrict__ residual,
+                                                                      float4* __restrict__ y, int inner4, int planes,
+                                                                      int channels, ChanEpilogue epi)
+{
+    const int i = blockIdx.x * kThreads + threadIdx.x;
+    if (i >= inner4) return;
+    for (int plane = blockIdx.y; plane < planes; plane += gridDim.y) {
+        const int ch = plane % channels;
+        const size_t at = (size_t)plane * inner4 + i;
+        float4 v = x[at];
+        if (residual) {
+            const float4 r = residual[at];
+            v.x += r.x; v.y += r.y; v.z += r.z; v.w += r.w;
+        }
+        v.x = chan_epilogue_apply(epi, ch, v.x);
+        v.y = chan_epilogue_apply(epi, ch, v.y);
+        v.z = chan_epilogue_apply(epi, ch, v.z);
+        v.w = chan_epilogue_apply(epi, ch, v.w);
+        y[at] = v;
+    }
+}
+
+// Rows (NHWC and (rows, C) matrices, inner == 1) with C/4 a divisor of 256: a thread keeps one quad of
+// channels for all its rows, so its parameters live in registers; 256 / (C/4) rows per pass.
+__global__ void __launch_bounds__(kThreads) chan_eltwise_rows_kernel(const float4* __restrict__ x,
+                                                                    const float4* __restrict__ residual,
+                                                                    float4* __restrict__ y, long rows, int c4,
+                                                                    ChanEpilogue epi)
+{
+    const int q = threadIdx.x % c4, r0 = threadIdx.x / c4, rows_per_pass = kThreads / c4;
+    float bias[4] = {0, 0, 0, 0}, mean[4] = {0, 0, 0, 0}, inv_std[4] = {0, 0, 0, 0}, gamma[4] = {0, 0, 0, 0},
+          beta[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        if (epi.bias) bias[t] = epi.bias[4 * q + t];
+        if (epi.mean) {
+            mean[t] = epi.mean[4 * q + t];
+            inv_std[t] = epi.inv_std[4 * q + t];
+            gamma[t] = epi.gamma[4 * q + t];
+            beta[t] = epi.beta[4 * q + t];
+        }
+    }
+    for (long row = (long)blockIdx.x * rows_per_pass + r0; row < rows; row += (long)gridDim.x * rows_per_pass) {
+        const size_t at = (size_t)row * c4 + q;
+        float4 v4 = x[at];
+        float v[4] = {v4.x, v4.y, v4.z, v4.w};
+        if (residual) {
+            const float4 r = residual[at];
+            v[0] += r.x; v[1] += r.y; v[2] += r.z; v[3] += r.w;
+        }
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            if (epi.bias) v[t] += bias[t];
+            if (epi.mean) {
+                const float u = (v[t] - mean[t]) * inv_std[t];
+                v[t] = u * gamma[t] + beta[t];
+            }
+            if (epi.relu) v[t] = v[t] > 0.0f ? v[t] : 0.0f;
+        }
+        y[at] = make_float4(v[0], v[1], v[2], v[3]);
+    }
+}
+
 // ---------------------------------------------------------------- ReLU with mask
 // pydtnn/cython_modules/relu_cython.pyx:52-59 (strict x > 0); pydtnn/backends/cpu/activations/relu_cpu.py:38-40.
 // Four elements per thread (one 16-byte load, one 16-byte store, one 4-byte mask store) when the
@@ -735,7 +804,34 @@ int launch_chan_eltwise(const float* x, const float* residual, float* y, long to
     if (total <= 0 || inner <= 0 || channels <= 0) return PYDTNN_HIP_ERR_INVALID;
     const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y) |
                            reinterpret_cast<uintptr_t>(residual)) & 15) == 0;
-    const bool vec = aligned && total % 4 == 0 && (inner % 4 == 0 || (inner == 1 && channels % 4 == 0));
+    const bool no_params = !epi.bias && !epi.mean;
+    if (aligned && inner % 4 == 0 && total % inner == 0 && total / inner < (1l << 31) && !no_params) {
+        const long planes = total / inner;
+        const int inner4 = inner / 4;
+        dim3 grid(blocks_for(inner4), (unsigned)(planes < 65535 ? planes : 65535));
+        hipLaunchKernelGGL(chan_eltwise_planes_kernel, grid, dim3(kThreads), 0, stream,
+                           reinterpret_cast<const float4*>(x), reinterpret_cast<const float4*>(residual),
+                           reinterpret_cast<float4*>(y), inner4, (int)planes, channels, epi);
+        HIP_RETURN_IF_LAUNCH_FAILED();
+        return PYDTNN_HIP_OK;
+    }
+    if (aligned && inner == 1 && channels % 4 == 0 && kThreads % (channels / 4) == 0 && total % channels == 0 &&
+        !no_params) {
+        const long rows = total / channels;
+        const int c4 = channels / 4, rows_per_pass = kThreads / c4;
+        // a few passes per thread amortise the parameter fetch
+        long blocks = (rows + (long)rows_per_pass * 8 - 1) / ((long)rows_per_pass * 8);
+        if (blocks < 1) blocks = 1;
+        if (blocks > (1l << 30)) blocks = 1l << 30;
+        hipLaunchKernelGGL(chan_eltwise_rows_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, stream,
+                           reinterpret_cast<const float4*>(x), reinterpret_cast<const float4*>(residual),
+                           reinterpret_cast<float4*>(y), rows, c4, epi);
+        HIP_RETURN_IF_LAUNCH_FAILED();
+        return PYDTNN_HIP_OK;
+    }
+    // without per-channel parameters (residual add, ReLU only) the channel of an element does not matter
+    const bool vec = aligned && total % 4 == 0 &&
+                     (no_params || inner % 4 == 0 || (inner == 1 && channels % 4 == 0));
     if (vec)
         hipLaunchKernelGGL(chan_eltwise_vec4_kernel, dim3(blocks_for(total / 4)), dim3(kThreads), 0, stream,
                            reinterpret_cast<const float4*>(x), reinterpret_cast<const float4*>(residual),

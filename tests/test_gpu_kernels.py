@@ -312,7 +312,8 @@ def test_dw_with_many_tiles_takes_the_balanced_launch(cg, oracle):
 
 def test_chan_eltwise_matches_oracle(ops, oracle):
     rng = np.random.default_rng(7)
-    for shape, fmt in [((3, 7, 5, 6), "NCHW"), ((3, 8, 4, 4), "NCHW"), ((3, 5, 6, 7), "NHWC"), ((2, 4, 4, 8), "NHWC")]:
+    for shape, fmt in [((3, 7, 5, 6), "NCHW"), ((3, 8, 4, 4), "NCHW"), ((3, 5, 6, 7), "NHWC"), ((2, 4, 4, 8), "NHWC"),
+                       ((70, 64, 12, 12), "NCHW"), ((40, 9, 9, 256), "NHWC"), ((5, 33, 7, 1024), "NHWC")]:
         announce("chan_eltwise", shape, fmt)
         c = shape[1] if fmt == "NCHW" else shape[3]
         x = rng.standard_normal(shape).astype(np.float32)
@@ -332,6 +333,14 @@ def test_chan_eltwise_matches_oracle(ops, oracle):
     acc = dev(x2)
     ops.eltw_sum(acc, dev(2 * x2))
     assert np.array_equal(host(acc), oracle.eltw_sum(x2.copy(), 2 * x2))
+    # residual + bias + ReLU in one pass, both layouts (plane and row kernels) and a shape that takes neither
+    for shape, channels, inner in [((6, 16, 8, 8), 16, 64), ((50, 128), 128, 1), ((7, 10), 10, 1)]:
+        x3 = rng.standard_normal(shape).astype(np.float32)
+        r3 = rng.standard_normal(shape).astype(np.float32)
+        b3 = rng.standard_normal(channels).astype(np.float32)
+        got = ops.chan_eltwise(dev(x3), channels=channels, inner=inner, residual=dev(r3), bias=dev(b3), relu=True)
+        bshape = (1, channels, 1, 1) if inner > 1 else (1, channels)
+        assert np.array_equal(host(got), np.maximum((x3 + r3) + b3.reshape(bshape), 0))
 
 
 def test_relu_forward_backward(ops, oracle):
