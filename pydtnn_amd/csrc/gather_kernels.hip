@@ -249,6 +249,61 @@ __global__ void __launch_bounds__(kThreads) im2row_nhwc_kernel(const float* __re
     }
 }
 
+// The same matrix for channel counts 4, 8, ..., 1024 and KHW taps, by quads of channels: a thread owns
+// (pixel, 4 channels), fetches the quad of every tap with one 128-bit load each (a wavefront reads 1 KB
+// runs of x), turns its KHW x 4 values into the row's (channel, tap) order in registers, and the
+// workgroup's rows, which are one contiguous run of the matrix, go out through LDS with full-width
+// 128-bit stores.  256 / (c/4) pixels per workgroup; LDS 4096 * KHW bytes.
+template <int KHW>
+__global__ void __launch_bounds__(kThreads) im2row_nhwc_quads_kernel(const float* __restrict__ x,
+                                                                    float* __restrict__ rows, ConvGeom g)
+{
+    __shared__ float4 staged[kThreads * KHW];
+    const int c4n = g.c >> 2, rows_per_block = kThreads / c4n;
+    const int r = threadIdx.x / c4n, q = threadIdx.x - r * c4n;
+    const long p0 = (long)blockIdx.x * rows_per_block;
+    const long p = p0 + r;
+    float4 v[KHW];
+#pragma unroll
+    for (int t = 0; t < KHW; ++t) v[t] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (p < g.p) {
+        const uint32_t nn = (uint32_t)(p / g.howo);
+        const uint32_t pp = (uint32_t)(p - (long)nn * g.howo);
+        const uint32_t yy = fd_div(pp, g.fd_wo);
+        const uint32_t xx = pp - yy * g.wo;
+        const int ih0 = g.vstride * (int)yy - g.vpadding, iw0 = g.hstride * (int)xx - g.hpadding;
+        const float* src = x + ((size_t)nn * g.h * g.w) * g.c + 4 * q;
+#pragma unroll
+        for (int t = 0; t < KHW; ++t) {
+            const int ii = (int)fd_div((uint32_t)t, g.fd_kw), jj = t - ii * g.kw;
+            const int x_x = ih0 + g.vdilation * ii, x_y = iw0 + g.hdilation * jj;
+            if ((unsigned)x_x < (unsigned)g.h && (unsigned)x_y < (unsigned)g.w)
+                v[t] = *reinterpret_cast<const float4*>(src + (size_t)(x_x * g.w + x_y) * g.c);
+        }
+    }
+    // (tap, channel) -> (channel, tap): element u*KHW + t of the thread's run is channel u of tap t
+    float run[4 * KHW];
+#pragma unroll
+    for (int t = 0; t < KHW; ++t) {
+        run[0 * KHW + t] = v[t].x;
+        run[1 * KHW + t] = v[t].y;
+        run[2 * KHW + t] = v[t].z;
+        run[3 * KHW + t] = v[t].w;
+    }
+    float4* mine = staged + (size_t)threadIdx.x * KHW;  // thread (r, q) owns floats [(r*c4n + q) * 4*KHW, +4*KHW)
+#pragma unroll
+    for (int t = 0; t < KHW; ++t) mine[t] = make_float4(run[4 * t], run[4 * t + 1], run[4 * t + 2], run[4 * t + 3]);
+    __syncthreads();
+    const long left = g.p - p0;
+    const long valid4 = (left < rows_per_block ? left : (long)rows_per_block) * c4n * KHW;  // float4s of this block
+    float4* dst = reinterpret_cast<float4*>(rows + p0 * g.k);
+#pragma unroll
+    for (int t = 0; t < KHW; ++t) {
+        const int f4 = t * kThreads + threadIdx.x;
+        if (f4 < valid4) dst[f4] = staged[f4];
+    }
+}
+
 // ---------------------------------------------------------------- row2im NHWC (gather form)
 // grid.x * 256 threads walk one image of dx (h*w*c floats, lanes along c), grid.y walks
 // the images.
@@ -384,6 +439,18 @@ int launch_col2im_nchw(const float* cols, float* dx, const ConvGeom& g, hipStrea
 
 int launch_im2row_nhwc(const float* x, float* rows, const ConvGeom& g, hipStream_t stream)
 {
+    // channel quads: c a power of two in 4..1024 (c/4 divides the workgroup), 9 taps, aligned tensors
+    const bool pow2 = g.c >= 4 && g.c <= 1024 && (g.c & (g.c - 1)) == 0;
+    if (pow2 && g.khw == 9 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(rows)) & 15) == 0) {
+        const int rows_per_block = kThreads / (g.c / 4);
+        const long blocks = (g.p + rows_per_block - 1) / rows_per_block;
+        if (blocks < (1l << 31)) {
+            hipLaunchKernelGGL(im2row_nhwc_quads_kernel<9>, dim3((unsigned)blocks), dim3(kThreads), 0, stream, x, rows,
+                               g);
+            HIP_RETURN_IF_LAUNCH_FAILED();
+            return PYDTNN_HIP_OK;
+        }
+    }
     // About 2048 matrix elements per block, never more rows than one image holds.
     int rpb = 2048 / g.k;
     if (rpb > g.howo) rpb = g.howo;
@@ -396,8 +463,57 @@ int launch_im2row_nhwc(const float* x, float* rows, const ConvGeom& g, hipStream
     return PYDTNN_HIP_OK;
 }
 
+// The same sums with the work laid out for the caches: a workgroup owns 8 neighbouring pixels x 32
+// channels, so the 1152-byte runs of `rows` it touches (32 channels x 9 taps of one output pixel) are
+// shared by its pixels through L1, and the channel chunk is the fastest-running part of the workgroup
+// index, so that (workgroups being dealt to the 8 XCDs in turn) a chunk's runs are re-read, for the rows
+// of dx above and below, from the same L2.  Needs c % 32 == 0.
+template <bool UNIT, int CB>
+__global__ void __launch_bounds__(kThreads) row2im_nhwc_patch_kernel(const float* __restrict__ rows,
+                                                                    float* __restrict__ dx, ConvGeom g, int chunks)
+{
+    constexpr int PX = kThreads / CB;
+    const uint32_t cb = blockIdx.x % (uint32_t)chunks, pg = blockIdx.x / (uint32_t)chunks;
+    const uint32_t t = pg * PX + (threadIdx.x / CB);
+    const uint32_t hw = (uint32_t)(g.h * g.w);
+    if (t >= hw) return;
+    const uint32_t cc = cb * CB + (threadIdx.x % CB);
+    const int hh = (int)fd_div(t, g.fd_w);
+    const int ww = (int)t - hh * g.w;
+    for (uint32_t nn = blockIdx.y; nn < (uint32_t)g.n; nn += gridDim.y) {
+        const float* src = rows + (long)nn * g.howo * g.k + cc * g.khw;
+        float acc = 0.0f;
+        for (int ii = g.kh - 1; ii >= 0; --ii) {
+            int oy;
+            if (!out_coord<UNIT>(hh + g.vpadding - g.vdilation * ii, g.vstride, g.fd_vs, g.ho, &oy)) continue;
+            for (int jj = g.kw - 1; jj >= 0; --jj) {
+                int ox;
+                if (!out_coord<UNIT>(ww + g.hpadding - g.hdilation * jj, g.hstride, g.fd_hs, g.wo, &ox)) continue;
+                acc += src[(long)(oy * g.wo + ox) * g.k + ii * g.kw + jj];
+            }
+        }
+        dx[((long)nn * hw + t) * g.c + cc] = acc;
+    }
+}
+
 int launch_row2im_nhwc(const float* rows, float* dx, const ConvGeom& g, hipStream_t stream)
 {
+    constexpr int CB = 32;
+    if (g.c % CB == 0) {
+        const int chunks = g.c / CB;
+        const long groups = ((long)g.h * g.w + (kThreads / CB) - 1) / (kThreads / CB);
+        if (groups * chunks < (1l << 31)) {
+            dim3 pgrid((unsigned)(groups * chunks), grid_y_for(g.n));
+            if (g.vstride == 1 && g.hstride == 1)
+                hipLaunchKernelGGL((row2im_nhwc_patch_kernel<true, CB>), pgrid, dim3(kThreads), 0, stream, rows, dx, g,
+                                   chunks);
+            else
+                hipLaunchKernelGGL((row2im_nhwc_patch_kernel<false, CB>), pgrid, dim3(kThreads), 0, stream, rows, dx, g,
+                                   chunks);
+            HIP_RETURN_IF_LAUNCH_FAILED();
+            return PYDTNN_HIP_OK;
+        }
+    }
     const long hwc = (long)g.h * g.w * g.c;
     dim3 grid(blocks_for(hwc), grid_y_for(g.n));
     const int c_exact = fd_exact((unsigned long)hwc + kThreads, (unsigned long)g.c);
