@@ -463,6 +463,7 @@ int launch_im2row_nhwc(const float* x, float* rows, const ConvGeom& g, hipStream
     return PYDTNN_HIP_OK;
 }
 
+namespace {
 // The same sums with the work laid out for the caches: a workgroup owns 8 neighbouring pixels x 32
 // channels, so the 1152-byte runs of `rows` it touches (32 channels x 9 taps of one output pixel) are
 // shared by its pixels through L1, and the channel chunk is the fastest-running part of the workgroup
@@ -495,6 +496,8 @@ __global__ void __launch_bounds__(kThreads) row2im_nhwc_patch_kernel(const float
         dx[((long)nn * hw + t) * g.c + cc] = acc;
     }
 }
+
+}  // namespace
 
 int launch_row2im_nhwc(const float* rows, float* dx, const ConvGeom& g, hipStream_t stream)
 {
