@@ -256,8 +256,17 @@ __global__ void __launch_bounds__(kThreads) splitk_reduce_kernel(const float* __
 {
     const long idx = (long)blockIdx.x * kThreads + threadIdx.x;
     if (idx >= total) return;
+    // eight loads in flight, then added in slice order (the sum is the same as one load at a time)
     float acc = 0.0f;
-    for (int s = 0; s < slices; ++s) acc += partial[(long)s * stride + idx];
+    int s = 0;
+    for (; s + 8 <= slices; s += 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = partial[(long)(s + u) * stride + idx];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc += v[u];
+    }
+    for (; s < slices; ++s) acc += partial[(long)s * stride + idx];
     const int col = (int)(idx % ncols);
     long r = idx / ncols;
     if (perm_c > 0) {
