@@ -182,7 +182,7 @@ int pydtnn_hip_relu_bwd(const float *dy, const int8_t *mask, float *dx, long tot
 
 /* db = sum of dy over batch and pixels (pydtnn/backends/cpu/layers/conv_2d_cpu.py:377, :463; fc_cpu.py:70).
  * dy is (outer, channels, inner): inner = ho*wo for NCHW, 1 for NHWC / FC.
- * Workspace: pydtnn_hip_conv_workspace_bytes(PYDTNN_HIP_OP_DB, ...) or 256*channels bytes. */
+ * Workspace: pydtnn_hip_conv_workspace_bytes(PYDTNN_HIP_OP_DB, ...) or 2048*channels bytes. */
 int pydtnn_hip_bias_grad(const float *dy, float *db, long outer, int channels, int inner, void *workspace,
                          size_t workspace_bytes, void *stream);
 

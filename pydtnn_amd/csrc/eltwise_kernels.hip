@@ -234,14 +234,67 @@ __global__ void __launch_bounds__(kThreads) bias_grad_rows_stage1(const float* _
     if (rl == 0 && ch < c) partial[(long)blockIdx.x * c + ch] = (red[0][cl] + red[1][cl]) + (red[2][cl] + red[3][cl]);
 }
 
+// (rows, C) matrix whose row is `lanes` = C/4 quads with lanes a power of two <= kThreads, 16-byte aligned:
+// one workgroup reads kThreads/lanes whole rows per load, eight loads in flight per lane, and covers the row
+// slice [blockIdx.x*per, +per).  HBM-bound: 4*rows*C bytes read once.
+__global__ void __launch_bounds__(kThreads) bias_grad_rows_quads_stage1(const float4* __restrict__ dy,
+                                                                       float* __restrict__ partial, long rows,
+                                                                       int lanes, long per)
+{
+    constexpr int kInFlight = 8;
+    __shared__ float4 red[kThreads];
+    const int cl = threadIdx.x & (lanes - 1);
+    const int row_lanes = kThreads / lanes, rl = threadIdx.x / lanes;
+    const long r0 = (long)blockIdx.x * per;
+    const long r1 = r0 + per < rows ? r0 + per : rows;
+    float4 acc[kInFlight];
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u) acc[u] = float4{0.0f, 0.0f, 0.0f, 0.0f};
+    const float4* p = dy + cl;
+    for (long r = r0 + rl; r < r1; r += (long)row_lanes * kInFlight) {
+        float4 v[kInFlight];
+#pragma unroll
+        for (int u = 0; u < kInFlight; ++u) {
+            const long rr = r + (long)u * row_lanes;
+            v[u] = rr < r1 ? p[rr * lanes] : float4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+#pragma unroll
+        for (int u = 0; u < kInFlight; ++u) {
+            acc[u].x += v[u].x; acc[u].y += v[u].y; acc[u].z += v[u].z; acc[u].w += v[u].w;
+        }
+    }
+    float4 t = acc[0];
+#pragma unroll
+    for (int u = 1; u < kInFlight; ++u) { t.x += acc[u].x; t.y += acc[u].y; t.z += acc[u].z; t.w += acc[u].w; }
+    red[threadIdx.x] = t;
+    __syncthreads();
+    if (rl == 0) {
+        for (int i = 1; i < row_lanes; ++i) {
+            const float4 o = red[i * lanes + cl];
+            t.x += o.x; t.y += o.y; t.z += o.z; t.w += o.w;
+        }
+        reinterpret_cast<float4*>(partial + (long)blockIdx.x * lanes * 4)[cl] = t;
+    }
+}
+
+// db[ch] = sum over slices of partial[s*c + ch]: 16 channels x 16 slice lanes per workgroup, each lane adding
+// its slices in order, the lanes' sums added in lane order.
 __global__ void __launch_bounds__(kThreads) bias_grad_stage2(const float* __restrict__ partial,
                                                             float* __restrict__ db, int c, int slices)
 {
-    const int ch = blockIdx.x * kThreads + threadIdx.x;
-    if (ch >= c) return;
+    __shared__ float red[16][17];
+    const int cl = threadIdx.x & 15, sl = threadIdx.x >> 4;
+    const int ch = blockIdx.x * 16 + cl;
     float acc = 0.0f;
-    for (int s = 0; s < slices; ++s) acc += partial[(long)s * c + ch];
-    db[ch] = acc;
+    if (ch < c)
+        for (int s = sl; s < slices; s += 16) acc += partial[(long)s * c + ch];
+    red[sl][cl] = acc;
+    __syncthreads();
+    if (sl == 0 && ch < c) {
+        float t = red[0][cl];
+        for (int i = 1; i < 16; ++i) t += red[i][cl];
+        db[ch] = t;
+    }
 }
 
 // ---------------------------------------------------------------- split-K reduction
@@ -520,6 +573,53 @@ __global__ void __launch_bounds__(kThreads) max_pool_bwd_nhwc_kernel(const float
         }
         if (gate) acc *= (float)gate[(size_t)nn * per_image + e];
         dx[(size_t)nn * per_image + e] = acc;
+    }
+}
+
+// NHWC backward when square windows tile the image exactly (same conditions as the NCHW windows kernel) and
+// c % 4 == 0 with 16-byte aligned tensors: one thread owns four channels of one window, reads their indices
+// and gradients once and writes the window's kh x kw quads of dx.  Decode as in
+// max_pool_2d_nhwc_cython.pyx (ii = idx / kh, jj = idx % kw).
+template <int K>
+__global__ void __launch_bounds__(kThreads) max_pool_bwd_windows_nhwc_kernel(const float4* __restrict__ dy,
+                                                                            const int4* __restrict__ idx_max,
+                                                                            float4* __restrict__ dx, ConvGeom g,
+                                                                            const uint32_t* __restrict__ gate)
+{
+    const uint32_t cq = (uint32_t)g.c / 4;
+    const uint32_t per_image = (uint32_t)g.howo * cq;
+    const uint32_t e = blockIdx.x * kThreads + threadIdx.x;
+    if (e >= per_image) return;
+    const uint32_t win = e / cq, q = e - win * cq;
+    const int oy = (int)fd_div(win, g.fd_wo);
+    const int ox = (int)win - oy * g.wo;
+    const int kh = K > 0 ? K : g.kh, kw = K > 0 ? K : g.kw;
+    for (uint32_t nn = blockIdx.y; nn < (uint32_t)g.n; nn += gridDim.y) {
+        const int4 rec = idx_max[(size_t)nn * per_image + e];
+        const float4 grad = dy[(size_t)nn * per_image + e];
+        const int ri[4] = {(int)fd_div((uint32_t)rec.x, g.fd_kh), (int)fd_div((uint32_t)rec.y, g.fd_kh),
+                           (int)fd_div((uint32_t)rec.z, g.fd_kh), (int)fd_div((uint32_t)rec.w, g.fd_kh)};
+        const int rj[4] = {(int)((uint32_t)rec.x - fd_div((uint32_t)rec.x, g.fd_kw) * g.kw),
+                           (int)((uint32_t)rec.y - fd_div((uint32_t)rec.y, g.fd_kw) * g.kw),
+                           (int)((uint32_t)rec.z - fd_div((uint32_t)rec.z, g.fd_kw) * g.kw),
+                           (int)((uint32_t)rec.w - fd_div((uint32_t)rec.w, g.fd_kw) * g.kw)};
+        const float gr[4] = {0.0f + grad.x, 0.0f + grad.y, 0.0f + grad.z, 0.0f + grad.w};
+        const size_t first = (((size_t)nn * g.h + (size_t)(oy * kh)) * g.w + (size_t)(ox * kw)) * cq + q;
+#pragma unroll
+        for (int ii = 0; ii < kh; ++ii)
+#pragma unroll
+            for (int jj = 0; jj < kw; ++jj) {
+                const size_t at = first + ((size_t)ii * g.w + jj) * cq;
+                float v[4];
+#pragma unroll
+                for (int t = 0; t < 4; ++t) v[t] = ri[t] == ii && rj[t] == jj ? gr[t] : 0.0f;
+                if (gate) {
+                    const uint32_t gt = gate[at];
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) v[t] *= (float)(int8_t)(gt >> (8 * t));
+                }
+                dx[at] = float4{v[0], v[1], v[2], v[3]};
+            }
     }
 }
 
@@ -883,10 +983,12 @@ int launch_relu_bwd(const float* dy, const int8_t* mask, float* dx, long total, 
     return PYDTNN_HIP_OK;
 }
 
+constexpr int kBiasGradSlices = 512;
+
 size_t bias_grad_workspace_floats(long outer, int channels)
 {
     (void)outer;
-    return (size_t)64 * channels;
+    return (size_t)kBiasGradSlices * channels;
 }
 
 // inner > 1: dy is (outer, channels, inner) [NCHW]; inner == 1: dy is (outer, channels) rows.
@@ -908,14 +1010,28 @@ int launch_bias_grad(const float* dy, float* db, long outer, int channels, int i
             hipLaunchKernelGGL(bias_grad_nchw_stage1<false>, dim3(channels, slices), dim3(kThreads), 0, stream, dy,
                                workspace, n, channels, inner, per);
     } else {
-        slices = outer < 64 * 4 ? (int)((outer + 3) / 4) : 64;
-        const long per = (outer + slices - 1) / slices;
-        slices = (int)((outer + per - 1) / per);
-        hipLaunchKernelGGL(bias_grad_rows_stage1, dim3(slices, (channels + 63) / 64), dim3(kThreads), 0, stream, dy,
-                           workspace, outer, channels, per);
+        const int lanes = channels / 4;
+        const bool quads = channels % 4 == 0 && lanes <= kThreads && (lanes & (lanes - 1)) == 0 &&
+                           (reinterpret_cast<uintptr_t>(dy) & 15) == 0;
+        if (quads) {
+            // a slice is at least 32 rows per row lane; at most kBiasGradSlices of them
+            const long rows_per_load = kThreads / lanes;
+            const long want = (outer + rows_per_load * 32 - 1) / (rows_per_load * 32);
+            slices = (int)(want < kBiasGradSlices ? want : kBiasGradSlices);
+            const long per = (outer + slices - 1) / slices;
+            slices = (int)((outer + per - 1) / per);
+            hipLaunchKernelGGL(bias_grad_rows_quads_stage1, dim3(slices), dim3(kThreads), 0, stream,
+                               reinterpret_cast<const float4*>(dy), workspace, outer, lanes, per);
+        } else {
+            slices = outer < 64 * 4 ? (int)((outer + 3) / 4) : 64;
+            const long per = (outer + slices - 1) / slices;
+            slices = (int)((outer + per - 1) / per);
+            hipLaunchKernelGGL(bias_grad_rows_stage1, dim3(slices, (channels + 63) / 64), dim3(kThreads), 0, stream,
+                               dy, workspace, outer, channels, per);
+        }
     }
     HIP_RETURN_IF_LAUNCH_FAILED();
-    hipLaunchKernelGGL(bias_grad_stage2, dim3(blocks_for(channels)), dim3(kThreads), 0, stream, workspace, db,
+    hipLaunchKernelGGL(bias_grad_stage2, dim3((channels + 15) / 16), dim3(kThreads), 0, stream, workspace, db,
                        channels, slices);
     HIP_RETURN_IF_LAUNCH_FAILED();
     return PYDTNN_HIP_OK;
@@ -996,6 +1112,26 @@ int launch_max_pool_bwd_nhwc(const float* dy, const int32_t* idx_max, float* dx,
 {
     const long per_image = (long)g.h * g.w * g.c;
     if (per_image >= (1l << 31) - kThreads) return PYDTNN_HIP_ERR_UNSUPPORTED;
+    const bool tiled = g.kh == g.kw && g.kh == g.vstride && g.kw == g.hstride && g.vpadding == 0 &&
+                       g.hpadding == 0 && g.vdilation == 1 && g.hdilation == 1 && g.h == g.ho * g.kh &&
+                       g.w == g.wo * g.kw;
+    const auto aligned = [](const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; };
+    if (tiled && g.c % 4 == 0 && aligned(dy, 16) && aligned(idx_max, 16) && aligned(dx, 16) &&
+        (!gate || aligned(gate, 4))) {
+        dim3 wgrid(blocks_for((long)g.howo * (g.c / 4)), (unsigned)(g.n < 65535 ? g.n : 65535));
+        const auto dy4 = reinterpret_cast<const float4*>(dy);
+        const auto idx4 = reinterpret_cast<const int4*>(idx_max);
+        const auto dx4 = reinterpret_cast<float4*>(dx);
+        const auto gate4 = reinterpret_cast<const uint32_t*>(gate);
+        if (g.kh == 2)
+            hipLaunchKernelGGL(max_pool_bwd_windows_nhwc_kernel<2>, wgrid, dim3(kThreads), 0, stream, dy4, idx4, dx4, g,
+                               gate4);
+        else
+            hipLaunchKernelGGL(max_pool_bwd_windows_nhwc_kernel<0>, wgrid, dim3(kThreads), 0, stream, dy4, idx4, dx4, g,
+                               gate4);
+        HIP_RETURN_IF_LAUNCH_FAILED();
+        return PYDTNN_HIP_OK;
+    }
     const int c_exact = (unsigned long)(per_image + kThreads) * (unsigned long)g.c < (1ul << 32);
     dim3 grid(blocks_for(per_image), (unsigned)(g.n < 65535 ? g.n : 65535));
     hipLaunchKernelGGL(max_pool_bwd_nhwc_kernel, grid, dim3(kThreads), 0, stream, dy, idx_max, dx, g, c_exact,

@@ -183,7 +183,7 @@ def bias_grad(dy, channels, inner):
     _need_f32(dy)
     outer = dy.numel() // (channels * inner)
     db = torch.empty((channels,), dtype=dy.dtype, device=dy.device)
-    ws, ws_bytes = native.workspace(256 * channels)
+    ws, ws_bytes = native.workspace(2048 * channels)
     check(lib().pydtnn_hip_bias_grad(f32(dy), f32(db), outer, channels, inner, ws, ws_bytes, stream_ptr()),
           "bias_grad")
     return db

@@ -366,6 +366,18 @@ def test_bias_grad(ops):
         assert_close(host(db2), dy.astype(np.float64).sum(axis=(0, 2, 3)), tol=1e-5, what="db nhwc")
 
 
+@pytest.mark.parametrize("rows,channels", [(1, 4), (37, 8), (5000, 64), (70001, 64), (3000, 128), (1111, 256),
+                                           (9000, 512), (300, 1024), (129, 2048), (64, 1000), (513, 12)])
+def test_bias_grad_of_a_row_matrix(ops, rows, channels):
+    """Row-major dy (NHWC conv, FC): widths that take the 16-byte kernel (a power of two of quads up to 1024
+    channels), ones that do not, row counts that leave ragged slices, and more rows than one slice holds."""
+    rng = np.random.default_rng(rows + channels)
+    announce("bias_grad rows", rows, channels)
+    dy = rng.standard_normal((rows, channels)).astype(np.float32)
+    db = ops.bias_grad(dev(dy), channels, 1)
+    assert_close(host(db), dy.astype(np.float64).sum(axis=0), tol=1e-5, what="db rows")
+
+
 def test_maxpool_matches_oracle(ops, oracle):
     rng = np.random.default_rng(10)
     for (shape, k, s, p) in [((2, 3, 8, 10), 2, 2, 0), ((2, 4, 9, 9), 3, 2, 1), ((1, 2, 7, 7), 3, 1, 1),
@@ -412,7 +424,10 @@ def test_maxpool_nhwc_matches_oracle(ops, oracle):
     rng = np.random.default_rng(12)
     for (shape, kh, kw, p, s, dil) in [((2, 8, 10, 3), 2, 2, 0, 2, 1), ((2, 9, 9, 70), 3, 3, 1, 2, 1),
                                        ((1, 7, 11, 5), 3, 2, 1, 1, 1), ((1, 9, 9, 2), 2, 2, 1, 1, 2),
-                                       ((2, 8, 12, 4), 2, 3, 0, 1, 1), ((1, 8, 12, 3), 2, 3, 1, 2, 1)]:
+                                       ((2, 8, 12, 4), 2, 3, 0, 1, 1), ((1, 8, 12, 3), 2, 3, 1, 2, 1),
+                                       # windows that tile the image with c % 4 == 0: the window-owner kernel
+                                       ((2, 8, 10, 8), 2, 2, 0, 2, 1), ((3, 6, 9, 12), 3, 3, 0, 3, 1),
+                                       ((1, 4, 4, 256), 2, 2, 0, 2, 1), ((2, 9, 10, 8), 2, 2, 0, 2, 1)]:
         announce("maxpool nhwc", shape, kh, kw, p, s, dil)
         x = rng.standard_normal(shape).astype(np.float32)
         x[0, :2, :2, 0] = 1.5  # ties: the first tap must win
@@ -654,7 +669,8 @@ def test_relu_mask_and_gate_arguments_are_checked(cg):
 def test_maxpool_backward_with_gate_equals_backward_then_relu_backward(ops):
     rng = np.random.default_rng(12)
     for (shape, kh, kw, s, p) in [((2, 3, 8, 10), 2, 2, 2, 0), ((2, 4, 9, 9), 3, 3, 2, 1), ((2, 3, 9, 11), 2, 2, 2, 0),
-                                  ((1, 2, 9, 12), 3, 3, 3, 0), ((3, 5, 14, 14), 2, 2, 2, 0), ((2, 3, 8, 9), 2, 3, 2, 0)]:
+                                  ((1, 2, 9, 12), 3, 3, 3, 0), ((3, 5, 14, 14), 2, 2, 2, 0), ((2, 3, 8, 9), 2, 3, 2, 0), ((2, 4, 8, 10), 2, 2, 2, 0),
+                                  ((2, 8, 9, 12), 3, 3, 3, 0), ((1, 64, 6, 6), 2, 2, 2, 0)]:
         announce("gated maxpool bwd", shape, kh, kw, s, p)
         x = rng.standard_normal(shape).astype(np.float32)
         gate = dev((rng.random(shape) < 0.6).astype(np.int8))
