@@ -216,6 +216,39 @@ struct MapMN {
     }
 };
 
+// MapMNW: lanes run along m like MapMN, but a wavefront owns four consecutive k rows of the step
+// (k = 4*wave + row) and visits the BMN/64 groups of 64 columns in turn.  Element e is (row e / kPasses,
+// column group e % kPasses), so whatever a loader derives from the row alone (wave-uniform, scalar) is worked
+// out for four rows per wavefront and step, not for every element.
+template <int BMN>
+struct MapMNW {
+    static_assert(BMN % 64 == 0 && kThreads == 256 && BK == 16, "four wavefronts with four rows each");
+    static constexpr int kPasses = BMN / 64;
+    static constexpr int NLD = 4 * kPasses;
+    static constexpr int row_of(int e) { return e / kPasses; }
+    static constexpr int pass_of(int e) { return e % kPasses; }
+    static __device__ __forceinline__ int mn(int tid, int pass) { return (tid & 63) + 64 * pass; }
+    static __device__ __forceinline__ int krow0(int tid) { return uniform(tid >> 6) * 4; }
+    // Rows (0, 2) of the wavefront share the 64-bit words of one pitch, rows (1, 3) those of the next.
+    template <int PART, int PARTS>
+    static __device__ __forceinline__ void store_part(float* lds, const float (&r)[NLD], int tid)
+    {
+        constexpr int P = LdsTile<BMN>::kRowPitch;
+        float* base = lds + (2 * (tid >> 6)) * P + (tid & 63) * 2;
+#pragma unroll
+        for (int j = 0; j < kPasses; ++j)
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                if ((j * 2 + h) * PARTS / (NLD / 2) == PART)
+                    *reinterpret_cast<floatx2*>(base + h * P + j * 128) =
+                        floatx2{r[h * kPasses + j], r[(h + 2) * kPasses + j]};
+    }
+    static __device__ __forceinline__ void store(float* lds, const float (&r)[NLD], int tid)
+    {
+        store_part<0, 1>(lds, r, tid);
+    }
+};
+
 // MapK: lanes run along k; each thread owns NLD different m (or n) positions.
 template <int BMN>
 struct MapK {
@@ -444,18 +477,18 @@ struct PlainMN {
 // wave-uniform and is decomposed on the scalar ALU.  WIDE selects the two-word tap mask.
 template <int BN, bool WIDE = false>
 struct Im2colNchwMN {
-    using Map = MapMN<BN>;
+    using Map = MapMNW<BN>;
     static constexpr int NLD = Map::NLD;
     static constexpr bool kLargeState = false;
     using Reg = float;
     const float* x;
     ConvGeom g;
     struct State {
-        rsrc_t rsrc;     // starts `lead` floats before x, so that every thread's base offset is >= 0
-        uint32_t base;   // byte offset of (img, c=0, ih0, iw0) from there
-        uint32_t inv0;   // narrow: combined tap mask; wide: mask over i
-        uint32_t inv1;   // wide: mask over j
-        int krow;
+        rsrc_t rsrc;                  // starts `lead` floats before x, so that every thread's base offset is >= 0
+        uint32_t base[Map::kPasses];  // byte offset of (img, c=0, ih0, iw0) from there, per column group
+        uint32_t inv0[Map::kPasses];  // narrow: combined tap mask; wide: mask over i
+        uint32_t inv1[Map::kPasses];  // wide: mask over j
+        int krow0;
     };
     struct Iter {};
     __device__ __forceinline__ void init(State& s, int origin, int /*image*/, int tid) const
@@ -465,29 +498,33 @@ struct Im2colNchwMN {
         // operand of the load, which the hardware adds after its range check of the vector offset.
         const int lead = g.vpadding * g.w + g.hpadding;
         s.rsrc = make_rsrc(x - lead, (long)g.n * g.c * g.h * g.w + lead);
-        long n = (long)origin + Map::mn(tid);
-        n = n < g.p ? n : g.p - 1;
-        const int img = (int)(n / g.howo);
-        const int pp = (int)(n - (long)img * g.howo);
-        const int yy = pp / g.wo, xx = pp - yy * g.wo;
-        const int ih0 = yy * g.vstride - g.vpadding;
-        const int iw0 = xx * g.hstride - g.hpadding;
-        s.krow = Map::krow(tid);
-        s.base = (uint32_t)((img * g.c * g.h + ih0) * g.w + iw0 + lead) * 4u;
-        if (WIDE) {
-            s.inv0 = tap_mask_axis(ih0, g.kh, g.vdilation, g.h);
-            s.inv1 = tap_mask_axis(iw0, g.kw, g.hdilation, g.w);
-        } else {
-            s.inv0 = tap_mask_combined(g, ih0, iw0);
-            s.inv1 = 0;
+        s.krow0 = Map::krow0(tid);
+#pragma unroll
+        for (int j = 0; j < Map::kPasses; ++j) {
+            long n = (long)origin + Map::mn(tid, j);
+            n = n < g.p ? n : g.p - 1;
+            const int img = (int)(n / g.howo);
+            const int pp = (int)(n - (long)img * g.howo);
+            const int yy = pp / g.wo, xx = pp - yy * g.wo;
+            const int ih0 = yy * g.vstride - g.vpadding;
+            const int iw0 = xx * g.hstride - g.hpadding;
+            s.base[j] = (uint32_t)((img * g.c * g.h + ih0) * g.w + iw0 + lead) * 4u;
+            if (WIDE) {
+                s.inv0[j] = tap_mask_axis(ih0, g.kh, g.vdilation, g.h);
+                s.inv1[j] = tap_mask_axis(iw0, g.kw, g.hdilation, g.w);
+            } else {
+                s.inv0[j] = tap_mask_combined(g, ih0, iw0);
+                s.inv1[j] = 0;
+            }
         }
     }
     __device__ __forceinline__ void begin(const State&, Iter&, int, int) const {}
     template <int E>
     __device__ __forceinline__ float elem(const State& s, const Iter&, int k0, int kend) const
     {
-        // scalar: reduction index -> (c, i, j) -> byte offset of the tap inside one image
-        const uint32_t k = (uint32_t)(k0 + s.krow + E * Map::kRowsPerPass);
+        constexpr int R = Map::row_of(E), J = Map::pass_of(E);
+        // scalar, once per row: reduction index -> (c, i, j) -> byte offset of the tap inside one image
+        const uint32_t k = (uint32_t)(k0 + s.krow0 + R);
         const uint32_t cc = fd_div(k, g.fd_khw);
         const uint32_t rem = k - cc * g.khw;
         const uint32_t ii = fd_div(rem, g.fd_kw);
@@ -496,12 +533,12 @@ struct Im2colNchwMN {
         const bool live = (int)k < kend;
         if (WIDE) {
             const uint32_t invalid =
-                __builtin_amdgcn_ubfe(s.inv0, live ? ii : 31u, 1) | __builtin_amdgcn_ubfe(s.inv1, jj, 1);
-            return buf_load(s.rsrc, guarded_offset(invalid, s.base), off);
+                __builtin_amdgcn_ubfe(s.inv0[J], live ? ii : 31u, 1) | __builtin_amdgcn_ubfe(s.inv1[J], jj, 1);
+            return buf_load(s.rsrc, guarded_offset(invalid, s.base[J]), off);
         }
         // two vector instructions per element: move the tap's mask bit to bit 31, merge it into the offset
         const uint32_t bit = live ? rem : 31u;
-        return buf_load(s.rsrc, ((s.inv0 << (31u - bit)) & kOob) | s.base, off);
+        return buf_load(s.rsrc, ((s.inv0[J] << (31u - bit)) & kOob) | s.base[J], off);
     }
     __device__ __forceinline__ void store(float* lds, const float (&r)[NLD], int tid) const { Map::store(lds, r, tid); }
     template <int PART, int PARTS>
@@ -747,11 +784,11 @@ struct FilterNhwcMN {
     }
 };
 
-// dW view in NHWC: A(m = (i,j,c), k = (image, pixel)).  Lanes run along m (consecutive channels);
-// the pixel is wave-uniform and decomposed by the lanes in parallel.
+// dW view in NHWC: A(m = (i,j,c), k = (image, pixel)).  Lanes run along m (consecutive channels); the
+// pixel of a row is wave-uniform and decomposed on the scalar unit, once per row for all column groups.
 template <int BM>
 struct Im2rowNhwcMN {
-    using Map = MapMN<BM>;
+    using Map = MapMNW<BM>;
     static constexpr int NLD = Map::NLD;
     static constexpr bool kLargeState = false;
     using Reg = float;
@@ -759,39 +796,43 @@ struct Im2rowNhwcMN {
     ConvGeom g;
     struct State {
         rsrc_t rsrc;
-        int moff;  // (di*w + dj)*c + channel
-        int di, dj;
-        int krow;
+        int moff[Map::kPasses];  // (di*w + dj)*c + channel, per column group
+        int di[Map::kPasses], dj[Map::kPasses];
+        int krow0;
         int image0;
     };
     struct Iter {};
     __device__ __forceinline__ void init(State& s, int origin, int image0, int tid) const
     {
         s.rsrc = make_rsrc(x, (long)g.n * g.c * g.h * g.w);
-        const int m = min(origin + Map::mn(tid), g.k - 1);
-        const int ij = m / g.c, cc = m - ij * g.c;
-        const int ii = ij / g.kw, jj = ij - ii * g.kw;
-        s.di = ii * g.vdilation;
-        s.dj = jj * g.hdilation;
-        s.moff = (s.di * g.w + s.dj) * g.c + cc;
-        s.krow = Map::krow(tid);
+#pragma unroll
+        for (int j = 0; j < Map::kPasses; ++j) {
+            const int m = min(origin + Map::mn(tid, j), g.k - 1);
+            const int ij = m / g.c, cc = m - ij * g.c;
+            const int ii = ij / g.kw, jj = ij - ii * g.kw;
+            s.di[j] = ii * g.vdilation;
+            s.dj[j] = jj * g.hdilation;
+            s.moff[j] = (s.di[j] * g.w + s.dj[j]) * g.c + cc;
+        }
+        s.krow0 = Map::krow0(tid);
         s.image0 = image0;
     }
     __device__ __forceinline__ void begin(const State&, Iter&, int, int) const {}
     template <int E>
     __device__ __forceinline__ float elem(const State& s, const Iter&, int k0, int kend) const
     {
+        constexpr int R = Map::row_of(E), J = Map::pass_of(E);
         // scalar: reduction index -> (image within the group, y, x) -> first input row / column of the window
-        const uint32_t k = (uint32_t)(k0 + s.krow + E * Map::kRowsPerPass);
+        const uint32_t k = (uint32_t)(k0 + s.krow0 + R);
         const uint32_t img = fd_div(k, g.fd_howo);
         const uint32_t pp = k - img * g.howo;
         const uint32_t yy = fd_div(pp, g.fd_wo);
         const uint32_t xx = pp - yy * g.wo;
         const int ih0 = (int)k < kend ? (int)yy * g.vstride - g.vpadding : 0x2000;  // beyond kend: fails the row test
         const int iw0 = (int)xx * g.hstride - g.hpadding;
-        const int pix = ((s.image0 + (int)img) * g.h + ih0) * g.w + iw0;
-        const bool ok = (unsigned)(ih0 + s.di) < (unsigned)g.h && (unsigned)(iw0 + s.dj) < (unsigned)g.w;
-        return buf_load(s.rsrc, ok ? (uint32_t)(pix * g.c + s.moff) * 4u : kOob, 0);
+        const int pixc = (((s.image0 + (int)img) * g.h + ih0) * g.w + iw0) * g.c;
+        const bool ok = (unsigned)(ih0 + s.di[J]) < (unsigned)g.h && (unsigned)(iw0 + s.dj[J]) < (unsigned)g.w;
+        return buf_load(s.rsrc, ok ? (uint32_t)(pixc + s.moff[J]) * 4u : kOob, 0);
     }
     __device__ __forceinline__ void store(float* lds, const float (&r)[NLD], int tid) const { Map::store(lds, r, tid); }
     template <int PART, int PARTS>
@@ -1304,10 +1345,13 @@ __device__ __forceinline__ void gemm_body(const AL& al, const BL& bl, const EP& 
     __shared__ __align__(16) float Bs[2][BK * (T::BN + kPad)];
 
     const int tid = threadIdx.x;
-    const int tile = xcd_remap(blockIdx.x, gridDim.x);
+    // all workgroups of the launch in one sequence, tile fastest: the tiles of one reduction chunk, which
+    // read the same rows of both operands, run on one XCD
+    const int seq = xcd_remap((int)(blockIdx.y * gridDim.x + blockIdx.x), (int)(gridDim.x * gridDim.y));
+    const int split = seq / (int)gridDim.x;
+    const int tile = seq - split * (int)gridDim.x;
     const int tm_idx = tile % tiles_m, tn_idx = tile / tiles_m;
     const int m0 = tm_idx * T::BM, n0 = tn_idx * T::BN;
-    const int split = blockIdx.y;
     const int group = split / si.cpg;
     const int chunk_idx = split - group * si.cpg;
     const int image = group * si.ips;  // first image of this workgroup's group
@@ -1350,7 +1394,7 @@ inline int launch(const AL& al, const BL& bl, const EP& ep, long m, long n, cons
                   hipStream_t stream)
 {
     const long tiles_m = (m + T::BM - 1) / T::BM, tiles_n = (n + T::BN - 1) / T::BN;
-    if (tiles_m * tiles_n >= (1l << 31) || splits > 65535 || splits < 1) return PYDTNN_HIP_ERR_UNSUPPORTED;
+    if (tiles_m * tiles_n * splits >= (1l << 31) || splits > 65535 || splits < 1) return PYDTNN_HIP_ERR_UNSUPPORTED;
     dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)splits);
     if constexpr (FitsThreePerCu<AL, BL>::value)
         hipLaunchKernelGGL((gemm_kernel<T, AL, BL, EP>), grid, dim3(kThreads), 0, stream, al, bl, ep, (int)tiles_m, si);
