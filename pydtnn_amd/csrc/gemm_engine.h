@@ -747,7 +747,7 @@ struct Im2rowNhwcK4 {
 // Filter in NHWC layout (c, kh, kw, kn) read as B(k in (i,j,c) order, n = filter).
 template <int BN>
 struct FilterNhwcMN {
-    using Map = MapMN<BN>;
+    using Map = MapMNW<BN>;
     static constexpr int NLD = Map::NLD;
     static constexpr bool kLargeState = false;
     using Reg = float;
@@ -755,26 +755,28 @@ struct FilterNhwcMN {
     ConvGeom g;
     struct State {
         rsrc_t rsrc;
-        uint32_t voff;
-        int krow;
+        uint32_t voff[Map::kPasses];
+        int krow0;
     };
     struct Iter {};
     __device__ __forceinline__ void init(State& s, int origin, int /*image*/, int tid) const
     {
         s.rsrc = make_rsrc(w, (long)g.k * g.kn);
-        s.voff = (uint32_t)min(origin + Map::mn(tid), g.kn - 1) * 4u;
-        s.krow = Map::krow(tid);
+#pragma unroll
+        for (int j = 0; j < Map::kPasses; ++j) s.voff[j] = (uint32_t)min(origin + Map::mn(tid, j), g.kn - 1) * 4u;
+        s.krow0 = Map::krow0(tid);
     }
     __device__ __forceinline__ void begin(const State&, Iter&, int, int) const {}
     template <int E>
     __device__ __forceinline__ float elem(const State& s, const Iter&, int k0, int kend) const
     {
-        // scalar: reduction index in (i,j,c) order -> filter row c*kh*kw + i*kw + j
-        const uint32_t k = (uint32_t)(k0 + s.krow + E * Map::kRowsPerPass);
+        constexpr int R = Map::row_of(E), J = Map::pass_of(E);
+        // scalar, once per row: reduction index in (i,j,c) order -> filter row c*kh*kw + i*kw + j
+        const uint32_t k = (uint32_t)(k0 + s.krow0 + R);
         const uint32_t ij = fd_div(k, g.fd_c);
         const uint32_t cc = k - ij * g.c;
         const uint32_t rowoff = (int)k < kend ? (cc * g.khw + ij) * (uint32_t)g.kn * 4u : kOob;
-        return buf_load(s.rsrc, s.voff + rowoff, 0);
+        return buf_load(s.rsrc, s.voff[J] + rowoff, 0);
     }
     __device__ __forceinline__ void store(float* lds, const float (&r)[NLD], int tid) const { Map::store(lds, r, tid); }
     template <int PART, int PARTS>
