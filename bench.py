@@ -41,7 +41,7 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-vgg16", action="store_true", help="skip the VGG16 training-step extra of the default run")
     ap.add_argument("--no-folding-extra", action="store_true",
-                    help="skip the second VGG16 run (enable_relu_folding=True) that is reported beside the headline one")
+                    help="skip the extra VGG16 runs (enable_relu_folding=True; NHWC) that are reported beside the headline one")
     ap.add_argument("--conv-layers", action="store_true",
                     help="with --workload cfg5: also time forward / dW / dX of each distinct VGG16 convolution alone")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -226,8 +226,8 @@ def cpu_baseline_cfg2(sample_images=64, reps=30):
                       f"matmul limited to {cores} threads"}
 
 
-def build_vgg16(pd, n=64, **flags):
-    model = pd.Model(tensor_format="NCHW", batch_size=n, **flags)
+def build_vgg16(pd, n=64, tensor_format="NCHW", **flags):
+    model = pd.Model(tensor_format=tensor_format, batch_size=n, **flags)
     model.add(pd.Input(shape=(224, 224, 3)))
     for nlayers, nfilters in [[2, 64], [2, 128], [3, 256], [3, 512], [3, 512]]:
         for _ in range(nlayers):
@@ -272,6 +272,19 @@ def run_cfg5(torch, pd, args, steps=None, warmup=None):
     if not args.no_folding_extra:
         folded_ms, _ = timed_steps(torch, folded_step, steps or args.steps,
                                    warmup if warmup is not None else args.warmup)
+    # the same step in the reference's other tensor format (its default on the CPU), also beside the headline
+    nhwc_ms = None
+    if not args.no_folding_extra:
+        del folded_model
+        np.random.seed(0)
+        nhwc_model = build_vgg16(pd, n, tensor_format="NHWC")
+        x_nhwc = x.permute(0, 2, 3, 1).contiguous()
+        nhwc_opt = pd.SGD(learning_rate=0.01, momentum=0.9)
+
+        def nhwc_step(timers):
+            nhwc_model.train_batch(x_nhwc, y_targ, loss_fn, nhwc_opt)
+
+        nhwc_ms, _ = timed_steps(torch, nhwc_step, steps or args.steps, warmup if warmup is not None else args.warmup)
     flop = 5929.5e9
     extra = {"vgg16_train_img_per_s": round(n / (ms * 1e-3), 1), "vgg16_ms_per_step": round(ms, 2),
              "vgg16_tflops": round(flop / (ms * 1e-3) / 1e12, 2),
@@ -282,6 +295,9 @@ def run_cfg5(torch, pd, args, steps=None, warmup=None):
         extra.update({"vgg16_relu_folding_img_per_s": round(n / (folded_ms * 1e-3), 1),
                       "vgg16_relu_folding_ms_per_step": round(folded_ms, 2),
                       "vgg16_relu_folding_same_losses": [float(a) for a in losses] == [float(b) for b in folded_losses]})
+    if nhwc_ms is not None:
+        extra.update({"vgg16_nhwc_train_img_per_s": round(n / (nhwc_ms * 1e-3), 1),
+                      "vgg16_nhwc_ms_per_step": round(nhwc_ms, 2)})
     return ms, extra
 
 

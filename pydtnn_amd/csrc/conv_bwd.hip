@@ -5,11 +5,25 @@ namespace convint {
 
 // ---------------------------------------------------------------- filter gradient
 // mat == nullptr: implicit (x gathered on the fly); otherwise the materialised x_cols / x_rows.
+// With at most 64 filters the filter gradient is one tile wide and kh*kw*c long; where 256-long tiles would
+// be padding for a tenth or more of their length (576 = 2.25 x 256 = 3 x 192) the implicit launches use
+// 192-long tiles instead.
+typedef Tile<192, 64, 2, 2> T192x64;
+typedef Tile<64, 192, 2, 2> T64x192;
+
+static bool dw_tile_192(const ConvGeom& g, int nhwc)
+{
+    const long m = nhwc ? g.k : g.kn, n = nhwc ? g.kn : g.k;
+    if (g.kn > 64 || pick_tile(m, n) != (nhwc ? SEL_256x64 : SEL_64x256)) return false;
+    return round_up(g.k, 192) * 10 <= round_up(g.k, 256) * 9;
+}
+
 SplitPlan plan_dw(const ConvGeom& g, int nhwc)
 {
     const long m = nhwc ? g.k : g.kn, n = nhwc ? g.kn : g.k;
     const TileSel sel = pick_tile(m, n);
-    return plan_pixel_split(tiles_of(sel, m, n), g.n, g.howo, (long)g.kn * g.k);
+    const long tiles = dw_tile_192(g, nhwc) ? (g.k + 191) / 192 : tiles_of(sel, m, n);
+    return plan_pixel_split(tiles, g.n, g.howo, (long)g.kn * g.k);
 }
 
 int conv_dw_nchw(const ConvGeom& g, const float* dy, const float* x, const float* cols, float* dw, float* ws,
@@ -41,6 +55,20 @@ int conv_dw_nchw(const ConvGeom& g, const float* dy, const float* x, const float
         })
         if (rc != kNotBalanced) return rc;
         rc = PYDTNN_HIP_OK;
+    }
+    if (!cols && dw_tile_192(g, 0)) {
+        typedef T64x192 T;
+        const long dy_img = (long)g.kn * g.howo;
+        if (!span_ok_k(T::BM, g.howo, sp.si.ips, dy_img)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+        auto al = plain_k<T::BM, true>(dy, g.p * g.kn, g.howo, dy_img, g.kn, g.howo);
+        al.fd_seg = group_div(g.howo, sp.si.ips);
+        Im2colNchwK<T::BN> bl;
+        bl.x = x; bl.g = g;
+        bl.g.fd_howo = group_div(g.howo, sp.si.ips);
+        rc = launch<T>(al, bl, epi_plain(ws, g.k, out_elems, g.kn, g.k, no_epilogue(), no_masks(), sp.splits), g.kn,
+                       g.k, sp.si, sp.splits, stream);
+        if (rc != PYDTNN_HIP_OK) return rc;
+        return launch_splitk_reduce(ws, dw, g.kn, g.k, out_elems, sp.splits, 0, 0, no_epilogue(), accumulate, stream);
     }
     WITH_TILE(sel, {
         // A(m = filter, k = (image, pixel)) = dy[image][filter][pixel]
@@ -74,6 +102,18 @@ int conv_dw_nhwc(const ConvGeom& g, const float* dy, const float* x, const float
     if (!ws || ws_bytes < (size_t)sp.splits * out_elems * 4) return PYDTNN_HIP_ERR_WORKSPACE;
     const TileSel sel = pick_tile(g.k, g.kn);
     int rc = PYDTNN_HIP_OK;
+    if (!rows && dw_tile_192(g, 1)) {
+        typedef T192x64 T;
+        auto bl = plain_mn<T::BN>(dy, g.p * g.kn, g.kn, (long)g.howo * g.kn, g.kn);
+        Im2rowNhwcMN<T::BM> al;
+        al.x = x; al.g = g;
+        al.g.fd_howo = group_div(g.howo, sp.si.ips);
+        rc = launch<T>(al, bl, epi_plain(ws, g.kn, out_elems, g.k, g.kn, no_epilogue(), no_masks(), sp.splits), g.k,
+                       g.kn, sp.si, sp.splits, stream);
+        if (rc != PYDTNN_HIP_OK) return rc;
+        return launch_splitk_reduce(ws, dw, g.k, g.kn, out_elems, sp.splits, g.c, g.khw, no_epilogue(), accumulate,
+                                    stream);
+    }
     WITH_TILE(sel, {
         // B(k = (image, pixel), n = filter) = dy[(image*howo + pixel)*kn + n]
         auto bl = plain_mn<T::BN>(dy, g.p * g.kn, g.kn, (long)g.howo * g.kn, g.kn);

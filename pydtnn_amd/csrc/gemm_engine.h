@@ -555,7 +555,7 @@ struct Im2colNchwK {
     using Map = MapK<BN>;
     static constexpr int NLD = Map::NLD;
     // three precomputed words for each of 16 elements: too much for three workgroups per CU
-    static constexpr bool kLargeState = BN >= 256;
+    static constexpr bool kLargeState = BN >= 192;
     using Reg = float;
     const float* x;
     ConvGeom g;

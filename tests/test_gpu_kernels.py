@@ -294,6 +294,25 @@ def test_dw_split_over_several_images_and_chunks(cg, oracle):
         assert_close(host(dw2).transpose(3, 0, 1, 2), dw_ref, what="dw nhwc")
 
 
+def test_dw_of_narrow_filter_sets_takes_the_192_long_tiles(cg, oracle):
+    """At most 64 filters and kh*kw*c = 576 or 1152: three (six) 192-long tiles instead of 256-long ones, in both
+    formats; ragged filter counts, strides, padding and a split over several images included."""
+    for d in [D(3, 64, 9, 11, 64, 3, 3, 1, 1, 1, 1), D(5, 64, 12, 12, 40, 3, 3, 1, 1, 2, 2),
+              D(2, 128, 7, 9, 64, 3, 3, 0, 1, 1, 1), D(20, 64, 6, 6, 33, 3, 3, 1, 1, 1, 1),
+              D(2, 16, 20, 20, 64, 6, 6, 2, 2, 1, 1)]:
+        announce("dw 192", d)
+        x, w, _, dy = case(d)
+        p = oracle.ConvParams(*d.geom())
+        _, x_cols = oracle.conv2d_forward_nchw_i2c(x, w, None, p)
+        dw_ref, _, _ = oracle.conv2d_backward_nchw_i2c(dy, x_cols, w, x.shape, p, need_dx=False)
+        dw = torch.full(w.shape, float("nan"), device="cuda")
+        cg.conv_gemm_nchw(dev(dy), dev(x), biases=dw, trans=True, **_kw(d))
+        assert_close(host(dw), dw_ref, what="dw nchw, 192-long tiles")
+        dw2 = torch.full(w_nhwc(w).shape, float("nan"), device="cuda")
+        cg.conv_gemm_nhwc(dev(nhwc(dy)), dev(nhwc(x)), biases=dw2, trans=True, **_kw(d))
+        assert_close(host(dw2).transpose(3, 0, 1, 2), dw_ref, what="dw nhwc, 192-long tiles")
+
+
 def test_dw_with_many_tiles_takes_the_balanced_launch(cg, oracle):
     """512 x 4608 filter matrix = 144 tiles: the reduction units of all tiles are dealt evenly over the chip and
     pieces of a tile summed by the fixup kernel (NCHW); the result must not depend on that."""
