@@ -27,9 +27,9 @@ HBM_PEAK_GBS = 8000.0
 
 # HBM-side bytes per launch of the forward kernel, from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE), each
 # scaled by what the same counter reads for a 256 MiB copy (factors 2.000 and 1.000):
-# main launch (195289.1 * 2.0 + 245760.0) KiB plus the fixup launch of its cut tiles (24625.0 * 2.0 + 4096.0) KiB.
+# main launch (202440.7 * 2.0 + 245760.0) KiB plus the fixup launch of its cut tiles (24630.5 * 2.0 + 4096.0) KiB.
 # The summary of those runs is profiles/cfg2_conv3x3_pmc_counters.md.
-MEASURED_TRAFFIC_BYTES = {"cfg2": int((195289.1 * 2.0 + 245760.0 + 24625.0 * 2.0 + 4096.0) * 1024)}
+MEASURED_TRAFFIC_BYTES = {"cfg2": int((202440.7 * 2.0 + 245760.0 + 24630.5 * 2.0 + 4096.0) * 1024)}
 
 
 def parse_args():

@@ -554,7 +554,7 @@ template <int BN>
 struct Im2colNchwK {
     using Map = MapK<BN>;
     static constexpr int NLD = Map::NLD;
-    // three precomputed words for each of 16 elements: too much for three workgroups per CU
+    // three precomputed words for each of 12 or 16 elements: built without the three-per-CU register limit
     static constexpr bool kLargeState = BN >= 192;
     using Reg = float;
     const float* x;
