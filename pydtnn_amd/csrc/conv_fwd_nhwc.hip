@@ -11,6 +11,17 @@ int conv_fwd_nhwc_t(const ConvGeom& g, const float* w, const float* x, float* y,
     // channels in multiples of 16 from an aligned tensor: 128-bit loads along the channel axis
     const bool quads = !WIDE && g.c % 16 == 0 && aligned16(x);
     int rc = PYDTNN_HIP_OK;
+    if (g.c <= 4) {
+        // a first layer: lanes along the pixels (3 floats apart for RGB) and the reduction index in the filter's own
+        // (c, i, j) row order; with lanes along 27 reduction indices the loads of a tile are a chain of latencies
+        WITH_TILE(sel, {
+            Im2colNchwMN<T::BM, WIDE, true> al;
+            al.x = x; al.g = g;
+            auto bl = plain_mn<T::BN>(w, (long)g.k * g.kn, g.kn, 0, g.kn);
+            rc = launch_rows_forward<T>(al, bl, g, y, chan, ws, ws_bytes, stream, masks);
+        })
+        return rc;
+    }
     WITH_TILE(sel, {
         FilterNhwcMN<T::BN> bl;
         bl.w = w; bl.g = g;

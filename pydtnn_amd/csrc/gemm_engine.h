@@ -475,7 +475,9 @@ struct PlainMN {
 // pydtnn/cython_modules/im2col_nchw_cython.pyx:104-124, never written to memory.
 // Lanes run along the pixel axis (contiguous in x for a fixed tap); the tap (c,i,j) of an element is
 // wave-uniform and is decomposed on the scalar ALU.  WIDE selects the two-word tap mask.
-template <int BN, bool WIDE = false>
+// NHWC: the same matrix read from an (N,H,W,C) tensor, X[img, ih, iw, c]; lanes are then c floats apart, which
+// only pays for very few channels (a first layer), where the rows of one tap's channels share cache lines.
+template <int BN, bool WIDE = false, bool NHWC = false>
 struct Im2colNchwMN {
     using Map = MapMNW<BN>;
     static constexpr int NLD = Map::NLD;
@@ -496,7 +498,7 @@ struct Im2colNchwMN {
         // ih0*w + iw0 >= -(vpadding*w + hpadding): shifting the descriptor back by that much keeps the
         // per-thread offset unsigned, and the tap's own offset (>= 0) can then ride in the scalar offset
         // operand of the load, which the hardware adds after its range check of the vector offset.
-        const int lead = g.vpadding * g.w + g.hpadding;
+        const int lead = (g.vpadding * g.w + g.hpadding) * (NHWC ? g.c : 1);
         s.rsrc = make_rsrc(x - lead, (long)g.n * g.c * g.h * g.w + lead);
         s.krow0 = Map::krow0(tid);
 #pragma unroll
@@ -508,7 +510,8 @@ struct Im2colNchwMN {
             const int yy = pp / g.wo, xx = pp - yy * g.wo;
             const int ih0 = yy * g.vstride - g.vpadding;
             const int iw0 = xx * g.hstride - g.hpadding;
-            s.base[j] = (uint32_t)((img * g.c * g.h + ih0) * g.w + iw0 + lead) * 4u;
+            s.base[j] = NHWC ? (uint32_t)(((img * g.h + ih0) * g.w + iw0) * g.c + lead) * 4u
+                             : (uint32_t)((img * g.c * g.h + ih0) * g.w + iw0 + lead) * 4u;
             if (WIDE) {
                 s.inv0[j] = tap_mask_axis(ih0, g.kh, g.vdilation, g.h);
                 s.inv1[j] = tap_mask_axis(iw0, g.kw, g.hdilation, g.w);
@@ -529,7 +532,9 @@ struct Im2colNchwMN {
         const uint32_t rem = k - cc * g.khw;
         const uint32_t ii = fd_div(rem, g.fd_kw);
         const uint32_t jj = rem - ii * g.kw;
-        const uint32_t off = (uint32_t)(((int)cc * g.h + (int)ii * g.vdilation) * g.w + (int)jj * g.hdilation) * 4u;
+        const uint32_t off =
+            NHWC ? (uint32_t)(((int)ii * g.vdilation * g.w + (int)jj * g.hdilation) * g.c + (int)cc) * 4u
+                 : (uint32_t)(((int)cc * g.h + (int)ii * g.vdilation) * g.w + (int)jj * g.hdilation) * 4u;
         const bool live = (int)k < kend;
         if (WIDE) {
             const uint32_t invalid =
