@@ -505,9 +505,11 @@ struct Im2colNchwMN {
         for (int j = 0; j < Map::kPasses; ++j) {
             long n = (long)origin + Map::mn(tid, j);
             n = n < g.p ? n : g.p - 1;
-            const int img = (int)(n / g.howo);
+            // 32-bit division whenever the pixel count allows it (a launch-wide condition): a third of the
+            // instructions of the 64-bit one, which counts for tiles with only a few reduction steps
+            const int img = g.p < (1l << 31) ? (int)((uint32_t)n / (uint32_t)g.howo) : (int)(n / g.howo);
             const int pp = (int)(n - (long)img * g.howo);
-            const int yy = pp / g.wo, xx = pp - yy * g.wo;
+            const int yy = (int)((uint32_t)pp / (uint32_t)g.wo), xx = pp - yy * g.wo;
             const int ih0 = yy * g.vstride - g.vpadding;
             const int iw0 = xx * g.hstride - g.hpadding;
             s.base[j] = NHWC ? (uint32_t)(((img * g.h + ih0) * g.w + iw0) * g.c + lead) * 4u
