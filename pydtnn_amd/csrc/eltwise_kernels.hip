@@ -399,6 +399,35 @@ __global__ void __launch_bounds__(kThreads) max_pool_fwd_nchw_kernel(const float
     }
 }
 
+// Forward for 2x2 windows that tile the plane exactly (stride 2, no padding or dilation, h == 2*ho, w == 2*wo,
+// 8-byte aligned x): a thread reads its window as two 64-bit loads and tests the four values in the reference's
+// order (first maximum wins).
+__global__ void __launch_bounds__(kThreads) max_pool_fwd_windows2_nchw_kernel(const float* __restrict__ x,
+                                                                             float* __restrict__ y,
+                                                                             int32_t* __restrict__ idx_max,
+                                                                             ConvGeom g)
+{
+    const uint32_t win = blockIdx.x * kThreads + threadIdx.x;
+    if (win >= (uint32_t)g.howo) return;
+    const int oy = (int)fd_div(win, g.fd_wo);
+    const int ox = (int)win - oy * g.wo;
+    const uint32_t planes = (uint32_t)(g.n * g.c);
+    const size_t first = (size_t)(2 * oy) * g.w + 2 * ox;
+    for (uint32_t plane = blockIdx.y; plane < planes; plane += gridDim.y) {
+        const float* src = x + (size_t)plane * g.h * g.w + first;
+        const float2 r0 = *reinterpret_cast<const float2*>(src);
+        const float2 r1 = *reinterpret_cast<const float2*>(src + g.w);
+        float maxval = -3.402823466e+38f;
+        int best = 0;
+        if (r0.x > maxval) { maxval = r0.x; best = 0; }
+        if (r0.y > maxval) { maxval = r0.y; best = 1; }
+        if (r1.x > maxval) { maxval = r1.x; best = 2; }
+        if (r1.y > maxval) { maxval = r1.y; best = 3; }
+        y[(size_t)plane * g.howo + win] = maxval;
+        idx_max[(size_t)plane * g.howo + win] = best;
+    }
+}
+
 // Backward when square windows tile the plane exactly (kh == kw == both strides, no padding or
 // dilation, h == ho*kh, w == wo*kw): one thread owns one window, reads its index and gradient once
 // and writes the window's kh x kw elements of dx (the decoded element gets 0 + dy, the others 0).
@@ -534,6 +563,37 @@ __global__ void __launch_bounds__(kThreads) max_pool_fwd_nhwc_kernel(const float
         }
         y[(size_t)nn * per_image + e] = maxval;
         idx_max[(size_t)nn * per_image + e] = best;
+    }
+}
+
+// NHWC forward for 2x2 windows that tile the image exactly, c % 4 == 0 and 16-byte aligned tensors: a thread owns
+// four channels of a window and reads each of its four pixels with one 128-bit load.
+__global__ void __launch_bounds__(kThreads) max_pool_fwd_windows2_nhwc_kernel(const float4* __restrict__ x,
+                                                                             float4* __restrict__ y,
+                                                                             int4* __restrict__ idx_max, ConvGeom g)
+{
+    const uint32_t cq = (uint32_t)g.c / 4;
+    const uint32_t per_image = (uint32_t)g.howo * cq;
+    const uint32_t e = blockIdx.x * kThreads + threadIdx.x;
+    if (e >= per_image) return;
+    const uint32_t win = e / cq, q = e - win * cq;
+    const int oy = (int)fd_div(win, g.fd_wo);
+    const int ox = (int)win - oy * g.wo;
+    const size_t first = ((size_t)(2 * oy) * g.w + (size_t)(2 * ox)) * cq + q;
+    for (uint32_t nn = blockIdx.y; nn < (uint32_t)g.n; nn += gridDim.y) {
+        const float4* src = x + (size_t)nn * g.h * g.w * cq + first;
+        const float4 v[4] = {src[0], src[cq], src[(size_t)g.w * cq], src[(size_t)g.w * cq + cq]};
+        float m[4] = {-3.402823466e+38f, -3.402823466e+38f, -3.402823466e+38f, -3.402823466e+38f};
+        int b[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const float c4[4] = {v[t].x, v[t].y, v[t].z, v[t].w};
+#pragma unroll
+            for (int l = 0; l < 4; ++l)
+                if (c4[l] > m[l]) { m[l] = c4[l]; b[l] = t; }
+        }
+        y[(size_t)nn * per_image + e] = float4{m[0], m[1], m[2], m[3]};
+        idx_max[(size_t)nn * per_image + e] = int4{b[0], b[1], b[2], b[3]};
     }
 }
 
@@ -1065,6 +1125,14 @@ int launch_max_pool_fwd_nchw(const float* x, float* y, int32_t* idx_max, const C
 {
     const long planes = (long)g.n * g.c;
     dim3 grid(blocks_for(g.howo), (unsigned)(planes < 65535 ? planes : 65535));
+    const bool windows2 = g.kh == 2 && g.kw == 2 && g.vstride == 2 && g.hstride == 2 && g.vpadding == 0 &&
+                          g.hpadding == 0 && g.vdilation == 1 && g.hdilation == 1 && g.h == 2 * g.ho &&
+                          g.w == 2 * g.wo;
+    if (windows2 && (reinterpret_cast<uintptr_t>(x) & 7) == 0) {
+        hipLaunchKernelGGL(max_pool_fwd_windows2_nchw_kernel, grid, dim3(kThreads), 0, stream, x, y, idx_max, g);
+        HIP_RETURN_IF_LAUNCH_FAILED();
+        return PYDTNN_HIP_OK;
+    }
     hipLaunchKernelGGL(max_pool_fwd_nchw_kernel, grid, dim3(kThreads), 0, stream, x, y, idx_max, g);
     HIP_RETURN_IF_LAUNCH_FAILED();
     return PYDTNN_HIP_OK;
@@ -1100,6 +1168,19 @@ int launch_max_pool_fwd_nhwc(const float* x, float* y, int32_t* idx_max, const C
 {
     const long per_image = (long)g.howo * g.c;
     if (per_image >= (1l << 31) - kThreads) return PYDTNN_HIP_ERR_UNSUPPORTED;
+    const bool windows2 = g.kh == 2 && g.kw == 2 && g.vstride == 2 && g.hstride == 2 && g.vpadding == 0 &&
+                          g.hpadding == 0 && g.vdilation == 1 && g.hdilation == 1 && g.h == 2 * g.ho &&
+                          g.w == 2 * g.wo;
+    if (windows2 && g.c % 4 == 0 &&
+        ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(idx_max)) & 15) ==
+            0) {
+        dim3 wgrid(blocks_for(per_image / 4), (unsigned)(g.n < 65535 ? g.n : 65535));
+        hipLaunchKernelGGL(max_pool_fwd_windows2_nhwc_kernel, wgrid, dim3(kThreads), 0, stream,
+                           reinterpret_cast<const float4*>(x), reinterpret_cast<float4*>(y),
+                           reinterpret_cast<int4*>(idx_max), g);
+        HIP_RETURN_IF_LAUNCH_FAILED();
+        return PYDTNN_HIP_OK;
+    }
     const int c_exact = (unsigned long)(per_image + kThreads) * (unsigned long)g.c < (1ul << 32);
     dim3 grid(blocks_for(per_image), (unsigned)(g.n < 65535 ? g.n : 65535));
     hipLaunchKernelGGL(max_pool_fwd_nhwc_kernel, grid, dim3(kThreads), 0, stream, x, y, idx_max, g, c_exact);
