@@ -23,10 +23,20 @@ template <bool WIDE>
 int conv_fwd_nchw_t(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan, float* ws,
                     size_t ws_bytes, hipStream_t stream, const ElemMasks& masks)
 {
-    const TileSel sel = pick_tile(g.kn, g.p, g.k);
     // filter rows of a multiple of 4 floats from an aligned tensor: 128-bit loads along the reduction axis
     const bool quads = !WIDE && g.k % 4 == 0 && aligned16(w);
+    const TileSel sel = quads ? pick_tile_fwd(g.kn, g.p, g.k) : pick_tile(g.kn, g.p, g.k);
     int rc = PYDTNN_HIP_OK;
+    if constexpr (!WIDE) {
+        if (sel == SEL_256x128) {
+            typedef T256x128 T;
+            if (!span_ok_k(T::BM, g.k, 0, 0)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+            Im2colNchwMN<T::BN, false> bl;
+            bl.x = x; bl.g = g;
+            return launch_planes_forward<T>(plain_k4<T::BM>(w, (long)g.kn * g.k, g.k, g.kn), bl, g, y, chan, ws,
+                                            ws_bytes, stream, masks);
+        }
+    }
     WITH_TILE(sel, {
         if (!span_ok_k(T::BM, g.k, 0, 0)) return PYDTNN_HIP_ERR_UNSUPPORTED;
         Im2colNchwMN<T::BN, WIDE> bl;

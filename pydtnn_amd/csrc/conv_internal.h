@@ -39,13 +39,18 @@ typedef Tile<64, 256, 1, 4> T64x256;
 typedef Tile<256, 64, 4, 1> T256x64;
 typedef Tile<64, 64, 2, 2> T64x64;
 
-enum TileSel { SEL_128x128, SEL_64x256, SEL_256x64, SEL_64x64, SEL_COUNT };
+// eight MFMA blocks per wavefront, two workgroups per CU: forward / dX launches with long reductions only.
+// (The 128x256 twin measured 2-4 % slower than 128x128 on VGG16's 128-filter layers and is not built.)
+typedef Tile<256, 128, 4, 1> T256x128;
+
+enum TileSel { SEL_128x128, SEL_64x256, SEL_256x64, SEL_64x64, SEL_COUNT, SEL_256x128 = SEL_COUNT, SEL_ALL };
 
 struct TileShape {
     long bm, bn;
     double efficiency;  // matrix-core rate of the shape relative to 128x128 (fewer MFMAs per load and barrier)
 };
-constexpr TileShape kTileShapes[SEL_COUNT] = {{128, 128, 1.0}, {64, 256, 0.93}, {256, 64, 0.93}, {64, 64, 0.6}};
+constexpr TileShape kTileShapes[SEL_ALL] = {{128, 128, 1.0}, {64, 256, 0.93}, {256, 64, 0.93}, {64, 64, 0.6},
+                                           {256, 128, 1.02}};
 
 inline long tiles_of(TileSel sel, long m, long n)
 {
@@ -66,6 +71,24 @@ inline TileSel pick_tile(long m, long n, long k = 1l << 30)
         const TileShape& t = kTileShapes[s];
         const double cost = (double)tiles_of((TileSel)s, m, n) * (double)(t.bm * t.bn) / t.efficiency;
         if (s == 0 || cost < best_cost) { best = (TileSel)s; best_cost = cost; }
+    }
+    return best;
+}
+
+// Forward / dX: as pick_tile, but a choice of 128x128 moves up to the 256x128 tile when the reduction is long
+// (its prologue and tile store are twice as long) and there are enough of them to fill the chip, which holds
+// 512 at once.
+constexpr long kBigTileMinTiles = 512;
+inline TileSel pick_tile_fwd(long m, long n, long k)
+{
+    TileSel best = pick_tile(m, n, k);
+    if (best != SEL_128x128 || k < 16 * BK) return best;
+    double best_cost = (double)tiles_of(best, m, n) * 128.0 * 128.0;
+    for (int s = SEL_256x128; s < SEL_ALL; ++s) {
+        const TileShape& t = kTileShapes[s];
+        const long tiles = tiles_of((TileSel)s, m, n);
+        const double cost = (double)tiles * (double)(t.bm * t.bn) / t.efficiency;
+        if (tiles >= kBigTileMinTiles && cost < best_cost) { best = (TileSel)s; best_cost = cost; }
     }
     return best;
 }

@@ -1378,16 +1378,24 @@ __device__ __forceinline__ void gemm_body(const AL& al, const BL& bl, const EP& 
 
 // Three workgroups per compute unit need at most 168 registers per lane.  The kernels are built under that
 // limit unless a loader's per-thread state (precomputed offsets / masks of 16 elements per step) is so large
-// that the limit would spill inside the reduction loop (`kLargeState`); those are built without it and run
-// two per CU.
-template <class AL, class BL>
-struct FitsThreePerCu {
-    static constexpr bool value = !(AL::kLargeState || BL::kLargeState);
+// that the limit would spill inside the reduction loop (`kLargeState`); those are built without it.  Tiles of
+// eight MFMA blocks per wavefront (256x128) hold 128 accumulator registers and are built for two
+// workgroups per CU (256 registers).
+template <class T, class AL, class BL>
+struct WorkgroupsPerCu {
+    static constexpr int value = T::TM * T::TN > 4 ? 2 : (AL::kLargeState || BL::kLargeState) ? 0 : 3;  // 0: no limit
 };
 
 template <class T, class AL, class BL, class EP>
 __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3)))
 gemm_kernel(AL al, BL bl, EP ep, int tiles_m, SplitInfo si)
+{
+    gemm_body<T>(al, bl, ep, tiles_m, si);
+}
+
+template <class T, class AL, class BL, class EP>
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
+gemm_kernel_big_tile(AL al, BL bl, EP ep, int tiles_m, SplitInfo si)
 {
     gemm_body<T>(al, bl, ep, tiles_m, si);
 }
@@ -1405,8 +1413,12 @@ inline int launch(const AL& al, const BL& bl, const EP& ep, long m, long n, cons
     const long tiles_m = (m + T::BM - 1) / T::BM, tiles_n = (n + T::BN - 1) / T::BN;
     if (tiles_m * tiles_n * splits >= (1l << 31) || splits > 65535 || splits < 1) return PYDTNN_HIP_ERR_UNSUPPORTED;
     dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)splits);
-    if constexpr (FitsThreePerCu<AL, BL>::value)
+    constexpr int kPerCu = WorkgroupsPerCu<T, AL, BL>::value;
+    if constexpr (kPerCu == 3)
         hipLaunchKernelGGL((gemm_kernel<T, AL, BL, EP>), grid, dim3(kThreads), 0, stream, al, bl, ep, (int)tiles_m, si);
+    else if constexpr (kPerCu == 2)
+        hipLaunchKernelGGL((gemm_kernel_big_tile<T, AL, BL, EP>), grid, dim3(kThreads), 0, stream, al, bl, ep,
+                           (int)tiles_m, si);
     else
         hipLaunchKernelGGL((gemm_kernel_large_state<T, AL, BL, EP>), grid, dim3(kThreads), 0, stream, al, bl, ep,
                            (int)tiles_m, si);
@@ -1518,6 +1530,13 @@ gemm_streamk_kernel(AL al, BL bl, EP ep, int tiles_m, StreamK sk)
 }
 
 template <class T, class AL, class BL, class EP>
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
+gemm_streamk_kernel_big_tile(AL al, BL bl, EP ep, int tiles_m, StreamK sk)
+{
+    gemm_streamk_body<T>(al, bl, ep, tiles_m, sk);
+}
+
+template <class T, class AL, class BL, class EP>
 __global__ void __launch_bounds__(kThreads) gemm_streamk_kernel_large_state(AL al, BL bl, EP ep, int tiles_m, StreamK sk)
 {
     gemm_streamk_body<T>(al, bl, ep, tiles_m, sk);
@@ -1569,8 +1588,12 @@ struct Residency {
 template <class T, class AL, class BL, class EP>
 inline hipError_t streamk_blocks_per_cu(int* per_cu)
 {
-    if constexpr (FitsThreePerCu<AL, BL>::value)
+    constexpr int kPerCu = WorkgroupsPerCu<T, AL, BL>::value;
+    if constexpr (kPerCu == 3)
         return hipOccupancyMaxActiveBlocksPerMultiprocessor(per_cu, gemm_streamk_kernel<T, AL, BL, EP>, kThreads, 0);
+    else if constexpr (kPerCu == 2)
+        return hipOccupancyMaxActiveBlocksPerMultiprocessor(per_cu, gemm_streamk_kernel_big_tile<T, AL, BL, EP>,
+                                                            kThreads, 0);
     else
         return hipOccupancyMaxActiveBlocksPerMultiprocessor(per_cu, gemm_streamk_kernel_large_state<T, AL, BL, EP>,
                                                             kThreads, 0);
@@ -1631,9 +1654,13 @@ inline int launch_balanced(const AL& al, const BL& bl, const EP& ep, long m, lon
     sk.partial = partial;
     const long total = (long)sk.sk_tiles * units;
     sk.sk_blocks = (int)(total / 4 < resident ? (total / 4 > 0 ? total / 4 : 1) : resident);
-    if constexpr (FitsThreePerCu<AL, BL>::value)
+    constexpr int kPerCu = WorkgroupsPerCu<T, AL, BL>::value;
+    if constexpr (kPerCu == 3)
         hipLaunchKernelGGL((gemm_streamk_kernel<T, AL, BL, EP>), dim3((unsigned)resident), dim3(kThreads), 0, stream,
                            al, bl, ep, (int)tiles_m, sk);
+    else if constexpr (kPerCu == 2)
+        hipLaunchKernelGGL((gemm_streamk_kernel_big_tile<T, AL, BL, EP>), dim3((unsigned)resident), dim3(kThreads), 0,
+                           stream, al, bl, ep, (int)tiles_m, sk);
     else
         hipLaunchKernelGGL((gemm_streamk_kernel_large_state<T, AL, BL, EP>), dim3((unsigned)resident),
                            dim3(kThreads), 0, stream, al, bl, ep, (int)tiles_m, sk);
