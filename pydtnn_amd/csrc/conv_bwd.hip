@@ -18,8 +18,22 @@ static bool dw_tile_192(const ConvGeom& g, int nhwc)
     return round_up(g.k, 192) * 10 <= round_up(g.k, 256) * 9;
 }
 
+// A filter matrix that 256x128 tiles cover without padding rows (NCHW: a multiple of 256 filters; NHWC: kh*kw*c a
+// multiple of 256 and a multiple of 128 filters) and that is at least 1152 long: those tiles, two workgroups per
+// CU, so the reduction is split for 512 of them.  The loaders' per-element vector and scalar instructions are
+// spread over twice the MFMAs.
+static bool dw_tile_big(const ConvGeom& g, int nhwc)
+{
+    if (g.k < 1152) return false;
+    return nhwc ? g.k % 256 == 0 && g.kn % 128 == 0 : g.kn % 256 == 0;
+}
+
 SplitPlan plan_dw(const ConvGeom& g, int nhwc)
 {
+    if (dw_tile_big(g, nhwc)) {
+        const long tiles = nhwc ? (g.k / 256) * (g.kn / 128) : (g.kn / 256) * ((g.k + 127) / 128);
+        return plan_pixel_split(tiles, g.n, g.howo, (long)g.kn * g.k, 512);
+    }
     const long m = nhwc ? g.k : g.kn, n = nhwc ? g.kn : g.k;
     const TileSel sel = pick_tile(m, n);
     const long tiles = dw_tile_192(g, nhwc) ? (g.k + 191) / 192 : tiles_of(sel, m, n);
@@ -40,7 +54,7 @@ int conv_dw_nchw(const ConvGeom& g, const float* dy, const float* x, const float
     // tiles (512 filters, 28x28), 3 % slower at 72, hence the tile bound.
     const long tiles = tiles_of(sel, g.kn, g.k);
     const long split_blocks = (long)sp.splits * tiles;
-    if (!cols && !accumulate && sp.si.ips == g.n && tiles >= 96 && split_blocks * 100 < kTargetBlocks * 97 &&
+    if (!cols && !accumulate && !dw_tile_big(g, 0) && sp.si.ips == g.n && tiles >= 96 && split_blocks * 100 < kTargetBlocks * 97 &&
         ws_bytes >= kBalanceBytes && g.p < (1l << 31)) {
         WITH_TILE(sel, {
             const long dy_img = (long)g.kn * g.howo;
@@ -55,6 +69,20 @@ int conv_dw_nchw(const ConvGeom& g, const float* dy, const float* x, const float
         })
         if (rc != kNotBalanced) return rc;
         rc = PYDTNN_HIP_OK;
+    }
+    if (!cols && dw_tile_big(g, 0)) {
+        typedef T256x128 T;
+        const long dy_img = (long)g.kn * g.howo;
+        if (!span_ok_k(T::BM, g.howo, sp.si.ips, dy_img)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+        auto al = plain_k<T::BM, true>(dy, g.p * g.kn, g.howo, dy_img, g.kn, g.howo);
+        al.fd_seg = group_div(g.howo, sp.si.ips);
+        Im2colNchwK<T::BN> bl;
+        bl.x = x; bl.g = g;
+        bl.g.fd_howo = group_div(g.howo, sp.si.ips);
+        rc = launch<T>(al, bl, epi_plain(ws, g.k, out_elems, g.kn, g.k, no_epilogue(), no_masks(), sp.splits), g.kn,
+                       g.k, sp.si, sp.splits, stream);
+        if (rc != PYDTNN_HIP_OK) return rc;
+        return launch_splitk_reduce(ws, dw, g.kn, g.k, out_elems, sp.splits, 0, 0, no_epilogue(), accumulate, stream);
     }
     if (!cols && dw_tile_192(g, 0)) {
         typedef T64x192 T;
@@ -102,6 +130,18 @@ int conv_dw_nhwc(const ConvGeom& g, const float* dy, const float* x, const float
     if (!ws || ws_bytes < (size_t)sp.splits * out_elems * 4) return PYDTNN_HIP_ERR_WORKSPACE;
     const TileSel sel = pick_tile(g.k, g.kn);
     int rc = PYDTNN_HIP_OK;
+    if (!rows && dw_tile_big(g, 1)) {
+        typedef T256x128 T;
+        auto bl = plain_mn<T::BN>(dy, g.p * g.kn, g.kn, (long)g.howo * g.kn, g.kn);
+        Im2rowNhwcMN<T::BM> al;
+        al.x = x; al.g = g;
+        al.g.fd_howo = group_div(g.howo, sp.si.ips);
+        rc = launch<T>(al, bl, epi_plain(ws, g.kn, out_elems, g.k, g.kn, no_epilogue(), no_masks(), sp.splits), g.k,
+                       g.kn, sp.si, sp.splits, stream);
+        if (rc != PYDTNN_HIP_OK) return rc;
+        return launch_splitk_reduce(ws, dw, g.k, g.kn, out_elems, sp.splits, g.c, g.khw, no_epilogue(), accumulate,
+                                    stream);
+    }
     if (!rows && dw_tile_192(g, 1)) {
         typedef T192x64 T;
         auto bl = plain_mn<T::BN>(dy, g.p * g.kn, g.kn, (long)g.howo * g.kn, g.kn);

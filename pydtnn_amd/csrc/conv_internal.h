@@ -118,10 +118,10 @@ struct SplitPlan {
 
 // Reduction over `images` segments of `seg` elements (pixels of one image): equal chunks of the whole
 // run of images where the index arithmetic allows it, else groups of whole images.
-inline SplitPlan plan_pixel_split(long tiles, int images, int seg, long out_elems)
+inline SplitPlan plan_pixel_split(long tiles, int images, int seg, long out_elems, long target_blocks = kTargetBlocks)
 {
     const long total = (long)images * seg;
-    long want = tiles >= kTargetBlocks ? 1 : kTargetBlocks / tiles;
+    long want = tiles >= target_blocks ? 1 : target_blocks / tiles;
     const long max_by_ws = (long)(kMaxPartialBytes / ((size_t)out_elems * 4));
     if (want > max_by_ws) want = max_by_ws < 1 ? 1 : max_by_ws;
     long chunk = round_up((total + want - 1) / want, BK);

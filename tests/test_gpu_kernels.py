@@ -313,6 +313,25 @@ def test_dw_of_narrow_filter_sets_takes_the_192_long_tiles(cg, oracle):
         assert_close(host(dw2).transpose(3, 0, 1, 2), dw_ref, what="dw nhwc, 192-long tiles")
 
 
+def test_dw_of_wide_filter_sets_takes_the_256x128_tiles(cg, oracle):
+    """A multiple of 256 filters (NCHW) / kh*kw*c a multiple of 256 and a multiple of 128 filters (NHWC), filter
+    matrix at least 1152 long: 256x128 tiles, reduction split for 512 workgroups; a shape that qualifies in one
+    format only, a stride, and a split that spans images included."""
+    for d in [D(3, 128, 9, 9, 256, 3, 3, 1, 1, 1, 1), D(2, 256, 8, 10, 128, 3, 3, 1, 1, 1, 1),
+              D(12, 256, 6, 6, 256, 3, 3, 1, 1, 2, 2), D(2, 72, 12, 12, 512, 4, 4, 1, 1, 1, 1)]:
+        announce("dw 256x128", d)
+        x, w, _, dy = case(d)
+        p = oracle.ConvParams(*d.geom())
+        _, x_cols = oracle.conv2d_forward_nchw_i2c(x, w, None, p)
+        dw_ref, _, _ = oracle.conv2d_backward_nchw_i2c(dy, x_cols, w, x.shape, p, need_dx=False)
+        dw = torch.full(w.shape, float("nan"), device="cuda")
+        cg.conv_gemm_nchw(dev(dy), dev(x), biases=dw, trans=True, **_kw(d))
+        assert_close(host(dw), dw_ref, what="dw nchw, 256x128 tiles")
+        dw2 = torch.full(w_nhwc(w).shape, float("nan"), device="cuda")
+        cg.conv_gemm_nhwc(dev(nhwc(dy)), dev(nhwc(x)), biases=dw2, trans=True, **_kw(d))
+        assert_close(host(dw2).transpose(3, 0, 1, 2), dw_ref, what="dw nhwc, 256x128 tiles")
+
+
 def test_dw_with_many_tiles_takes_the_balanced_launch(cg, oracle):
     """512 x 4608 filter matrix = 144 tiles: the reduction units of all tiles are dealt evenly over the chip and
     pieces of a tile summed by the fixup kernel (NCHW); the result must not depend on that."""
