@@ -27,9 +27,9 @@ HBM_PEAK_GBS = 8000.0
 
 # HBM-side bytes per launch of the forward kernel, from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE), each
 # scaled by what the same counter reads for a 256 MiB copy (factors 2.000 and 1.000):
-# main launch (202440.7 * 2.0 + 245760.0) KiB plus the fixup launch of its cut tiles (24630.5 * 2.0 + 4096.0) KiB.
+# main launch (166125.0 * 2.0 + 262144.0) KiB plus the fixup launch of its cut tiles (32822.9 * 2.0 + 4096.0) KiB.
 # The summary of those runs is profiles/cfg2_conv3x3_pmc_counters.md.
-MEASURED_TRAFFIC_BYTES = {"cfg2": int((202440.7 * 2.0 + 245760.0 + 24630.5 * 2.0 + 4096.0) * 1024)}
+MEASURED_TRAFFIC_BYTES = {"cfg2": int((166125.0 * 2.0 + 262144.0 + 32822.9 * 2.0 + 4096.0) * 1024)}
 
 
 def parse_args():
@@ -189,7 +189,7 @@ def run_cfg2(torch, pd, args):
     extra["epilogue_gbs"] = round(2 * x.nbytes / (t3.median_ms() * 1e-3) / 1e9, 1)
     extra["epilogue_pct_hbm_peak"] = round(100 * extra["epilogue_gbs"] / HBM_PEAK_GBS, 1)
     del mat, back
-    roofline = {"bound": "mfma", "kernel": "gemm_streamk_kernel<128x128, PlainK, Im2colNchwMN, EpiNchw> + streamk_fixup_kernel (forward)",
+    roofline = {"bound": "mfma", "kernel": "gemm_streamk_kernel_big_tile<256x128, PlainK4, Im2colNchwMN, EpiNchw> + streamk_fixup_kernel (forward)",
                 "achieved": round(achieved, 3), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES["cfg2"]}
     workload = ("cfg2: VGG16-style 3x3 conv layer fwd+dW+db+dX, fp32 NCHW, N=64, 256->256, 56x56, stride 1, pad 1, "
