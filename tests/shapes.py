@@ -97,4 +97,9 @@ wide_channel_grid = [
     D(1, 300, 6, 6, 2, 1, 1, 0, 0, 1, 1, 1, 1),
     D(1, 64, 5, 40, 2, 3, 7, 1, 3, 2, 1, 1, 2),
     D(1, 48, 14, 14, 2, 3, 3, 3, 3, 2, 2, 1, 1),
+    # 3x3 at stride 1: no padding, padding 2, mixed padding, planes of whole and of ragged 8x8 patches
+    D(3, 64, 17, 8, 2, 3, 3, 0, 0, 1, 1, 1, 1),
+    D(2, 8, 16, 16, 2, 3, 3, 2, 2, 1, 1, 1, 1),
+    D(1, 16, 8, 24, 2, 3, 3, 1, 0, 1, 1, 1, 1),
+    D(2, 24, 3, 5, 2, 3, 3, 1, 1, 1, 1, 1, 1),
 ]
