@@ -39,7 +39,8 @@ typedef Tile<64, 256, 1, 4> T64x256;
 typedef Tile<256, 64, 4, 1> T256x64;
 typedef Tile<64, 64, 2, 2> T64x64;
 
-// eight MFMA blocks per wavefront, two workgroups per CU: forward / dX launches with long reductions only.
+// eight MFMA blocks per wavefront, two workgroups per CU: NCHW forward / dX launches with long reductions
+// (pick_tile_fwd) and the filter gradients whose matrix the tile covers without padding rows.
 // (The 128x256 twin measured 2-4 % slower than 128x128 on VGG16's 128-filter layers and is not built.)
 typedef Tile<256, 128, 4, 1> T256x128;
 
