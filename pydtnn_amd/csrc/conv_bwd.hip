@@ -28,8 +28,22 @@ static bool dw_tile_big(const ConvGeom& g, int nhwc)
     return nhwc ? g.k % 256 == 0 && g.kn % 128 == 0 : g.kn % 256 == 0;
 }
 
+// A multiple of 128 filters (that the 256x128 tile does not serve) and kh*kw*c a multiple of 192, at least 1152:
+// tiles of 128 filters x 192, six MFMA blocks per wavefront, also two workgroups per CU (1152 is 6 times 192: no
+// padding columns and a third fewer tiles than 9 times 128; measured +6.5 % there in both formats, but -13 % at
+// 576 = 3 x 192, which therefore stays on the 128x128 tile).
+typedef Tile<128, 192, 2, 2> T128x192;
+typedef Tile<192, 128, 2, 2> T192x128;
+
+static bool dw_tile_192x128(const ConvGeom& g, int nhwc)
+{
+    return !dw_tile_big(g, nhwc) && g.kn % 128 == 0 && g.k % 192 == 0 && g.k >= 1152;
+}
+
 SplitPlan plan_dw(const ConvGeom& g, int nhwc)
 {
+    if (dw_tile_192x128(g, nhwc))
+        return plan_pixel_split((long)(g.kn / 128) * (g.k / 192), g.n, g.howo, (long)g.kn * g.k, 512);
     if (dw_tile_big(g, nhwc)) {
         const long tiles = nhwc ? (g.k / 256) * (g.kn / 128) : (g.kn / 256) * ((g.k + 127) / 128);
         return plan_pixel_split(tiles, g.n, g.howo, (long)g.kn * g.k, 512);
@@ -54,7 +68,8 @@ int conv_dw_nchw(const ConvGeom& g, const float* dy, const float* x, const float
     // tiles (512 filters, 28x28), 3 % slower at 72, hence the tile bound.
     const long tiles = tiles_of(sel, g.kn, g.k);
     const long split_blocks = (long)sp.splits * tiles;
-    if (!cols && !accumulate && !dw_tile_big(g, 0) && sp.si.ips == g.n && tiles >= 96 && split_blocks * 100 < kTargetBlocks * 97 &&
+    if (!cols && !accumulate && !dw_tile_big(g, 0) && !dw_tile_192x128(g, 0) && sp.si.ips == g.n && tiles >= 96 &&
+        split_blocks * 100 < kTargetBlocks * 97 &&
         ws_bytes >= kBalanceBytes && g.p < (1l << 31)) {
         WITH_TILE(sel, {
             const long dy_img = (long)g.kn * g.howo;
@@ -72,6 +87,20 @@ int conv_dw_nchw(const ConvGeom& g, const float* dy, const float* x, const float
     }
     if (!cols && dw_tile_big(g, 0)) {
         typedef T256x128 T;
+        const long dy_img = (long)g.kn * g.howo;
+        if (!span_ok_k(T::BM, g.howo, sp.si.ips, dy_img)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+        auto al = plain_k<T::BM, true>(dy, g.p * g.kn, g.howo, dy_img, g.kn, g.howo);
+        al.fd_seg = group_div(g.howo, sp.si.ips);
+        Im2colNchwK<T::BN> bl;
+        bl.x = x; bl.g = g;
+        bl.g.fd_howo = group_div(g.howo, sp.si.ips);
+        rc = launch<T>(al, bl, epi_plain(ws, g.k, out_elems, g.kn, g.k, no_epilogue(), no_masks(), sp.splits), g.kn,
+                       g.k, sp.si, sp.splits, stream);
+        if (rc != PYDTNN_HIP_OK) return rc;
+        return launch_splitk_reduce(ws, dw, g.kn, g.k, out_elems, sp.splits, 0, 0, no_epilogue(), accumulate, stream);
+    }
+    if (!cols && dw_tile_192x128(g, 0)) {
+        typedef T128x192 T;
         const long dy_img = (long)g.kn * g.howo;
         if (!span_ok_k(T::BM, g.howo, sp.si.ips, dy_img)) return PYDTNN_HIP_ERR_UNSUPPORTED;
         auto al = plain_k<T::BM, true>(dy, g.p * g.kn, g.howo, dy_img, g.kn, g.howo);
@@ -132,6 +161,18 @@ int conv_dw_nhwc(const ConvGeom& g, const float* dy, const float* x, const float
     int rc = PYDTNN_HIP_OK;
     if (!rows && dw_tile_big(g, 1)) {
         typedef T256x128 T;
+        auto bl = plain_mn<T::BN>(dy, g.p * g.kn, g.kn, (long)g.howo * g.kn, g.kn);
+        Im2rowNhwcMN<T::BM> al;
+        al.x = x; al.g = g;
+        al.g.fd_howo = group_div(g.howo, sp.si.ips);
+        rc = launch<T>(al, bl, epi_plain(ws, g.kn, out_elems, g.k, g.kn, no_epilogue(), no_masks(), sp.splits), g.k,
+                       g.kn, sp.si, sp.splits, stream);
+        if (rc != PYDTNN_HIP_OK) return rc;
+        return launch_splitk_reduce(ws, dw, g.k, g.kn, out_elems, sp.splits, g.c, g.khw, no_epilogue(), accumulate,
+                                    stream);
+    }
+    if (!rows && dw_tile_192x128(g, 1)) {
+        typedef T192x128 T;
         auto bl = plain_mn<T::BN>(dy, g.p * g.kn, g.kn, (long)g.howo * g.kn, g.kn);
         Im2rowNhwcMN<T::BM> al;
         al.x = x; al.g = g;

@@ -318,7 +318,10 @@ def test_dw_of_wide_filter_sets_takes_the_256x128_tiles(cg, oracle):
     matrix at least 1152 long: 256x128 tiles, reduction split for 512 workgroups; a shape that qualifies in one
     format only, a stride, and a split that spans images included."""
     for d in [D(3, 128, 9, 9, 256, 3, 3, 1, 1, 1, 1), D(2, 256, 8, 10, 128, 3, 3, 1, 1, 1, 1),
-              D(12, 256, 6, 6, 256, 3, 3, 1, 1, 2, 2), D(2, 72, 12, 12, 512, 4, 4, 1, 1, 1, 1)]:
+              D(12, 256, 6, 6, 256, 3, 3, 1, 1, 2, 2), D(2, 72, 12, 12, 512, 4, 4, 1, 1, 1, 1),
+              # a multiple of 128 filters and kh*kw*c a multiple of 192: the 128x192 / 192x128 tiles
+              D(3, 128, 10, 9, 128, 3, 3, 1, 1, 1, 1), D(2, 128, 7, 7, 384, 3, 3, 1, 1, 1, 1),
+              D(9, 192, 6, 6, 128, 3, 3, 0, 0, 1, 1)]:
         announce("dw 256x128", d)
         x, w, _, dy = case(d)
         p = oracle.ConvParams(*d.geom())
