@@ -37,6 +37,15 @@ int conv_fwd_nchw_t(const ConvGeom& g, const float* w, const float* x, float* y,
                                             ws_bytes, stream, masks);
         }
     }
+    if (g.kn % 96 == 0 && g.kn % 64 != 0) {
+        // 96, 288, ... filters (AlexNet's first layer): 96-row tiles instead of 128-row ones that are a quarter padding
+        typedef Tile<96, 256, 1, 4> T;
+        if (!span_ok_k(T::BM, g.k, 0, 0)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+        Im2colNchwMN<T::BN, WIDE> bl;
+        bl.x = x; bl.g = g;
+        return launch_planes_forward<T>(plain_k<T::BM, false>(w, (long)g.kn * g.k, g.k, 0, g.kn, 0), bl, g, y, chan, ws,
+                                        ws_bytes, stream, masks);
+    }
     WITH_TILE(sel, {
         if (!span_ok_k(T::BM, g.k, 0, 0)) return PYDTNN_HIP_ERR_UNSUPPORTED;
         Im2colNchwMN<T::BN, WIDE> bl;
