@@ -4,7 +4,7 @@
 namespace convint {
 
 // ---------------------------------------------------------------- filter gradient
-// mat == nullptr: implicit (x gathered on the fly); otherwise the materialised x_cols / x_rows.
+// cols / rows == nullptr: implicit (x gathered on the fly); otherwise the materialised x_cols / x_rows.
 // With at most 64 filters the filter gradient is one tile wide and kh*kw*c long; where 256-long tiles would
 // be padding for a tenth or more of their length (576 = 2.25 x 256 = 3 x 192) the implicit launches use
 // 192-long tiles instead.
@@ -54,6 +54,36 @@ SplitPlan plan_dw(const ConvGeom& g, int nhwc)
     return plan_pixel_split(tiles, g.n, g.howo, (long)g.kn * g.k);
 }
 
+// One implicit NCHW launch with tile T: partial sums of the split into the workspace.
+// A(m = filter, k = (image, pixel)) = dy[image][filter][pixel]; B = the column matrix gathered from x.
+template <class T>
+static int dw_nchw_implicit(const ConvGeom& g, const SplitPlan& sp, const float* dy, const float* x, float* ws,
+                            hipStream_t stream)
+{
+    const long dy_img = (long)g.kn * g.howo;
+    if (!span_ok_k(T::BM, g.howo, sp.si.ips, dy_img)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+    auto al = plain_k<T::BM, true>(dy, g.p * g.kn, g.howo, dy_img, g.kn, g.howo);
+    al.fd_seg = group_div(g.howo, sp.si.ips);
+    Im2colNchwK<T::BN> bl;
+    bl.x = x; bl.g = g;
+    bl.g.fd_howo = group_div(g.howo, sp.si.ips);
+    const EpiPlain ep = epi_plain(ws, g.k, (long)g.kn * g.k, g.kn, g.k, no_epilogue(), no_masks(), sp.splits);
+    return launch<T>(al, bl, ep, g.kn, g.k, sp.si, sp.splits, stream);
+}
+
+// The NHWC twin: A(m = (i,j,c), k = (image, pixel)) gathered from x; B(k, n = filter) = dy[(image*howo + pixel)*kn + n].
+template <class T>
+static int dw_nhwc_implicit(const ConvGeom& g, const SplitPlan& sp, const float* dy, const float* x, float* ws,
+                            hipStream_t stream)
+{
+    auto bl = plain_mn<T::BN>(dy, g.p * g.kn, g.kn, (long)g.howo * g.kn, g.kn);
+    Im2rowNhwcMN<T::BM> al;
+    al.x = x; al.g = g;
+    al.g.fd_howo = group_div(g.howo, sp.si.ips);
+    const EpiPlain ep = epi_plain(ws, g.kn, (long)g.kn * g.k, g.k, g.kn, no_epilogue(), no_masks(), sp.splits);
+    return launch<T>(al, bl, ep, g.k, g.kn, sp.si, sp.splits, stream);
+}
+
 int conv_dw_nchw(const ConvGeom& g, const float* dy, const float* x, const float* cols, float* dw, float* ws,
                  size_t ws_bytes, hipStream_t stream, int accumulate)
 {
@@ -61,6 +91,7 @@ int conv_dw_nchw(const ConvGeom& g, const float* dy, const float* x, const float
     const long out_elems = (long)g.kn * g.k;
     if (!ws || ws_bytes < (size_t)sp.splits * out_elems * 4) return PYDTNN_HIP_ERR_WORKSPACE;
     const TileSel sel = pick_tile(g.kn, g.k);
+    const bool special_tile = dw_tile_big(g, 0) || dw_tile_192x128(g, 0) || dw_tile_192(g, 0);
     int rc = PYDTNN_HIP_OK;
     // The equal chunks of the split leave part of the chip idle when tiles * chunks misses what it holds
     // (144 tiles x 5 chunks = 720 of 768).  With all images in one reduction group the balanced launch deals
@@ -68,9 +99,8 @@ int conv_dw_nchw(const ConvGeom& g, const float* dy, const float* x, const float
     // tiles (512 filters, 28x28), 3 % slower at 72, hence the tile bound.
     const long tiles = tiles_of(sel, g.kn, g.k);
     const long split_blocks = (long)sp.splits * tiles;
-    if (!cols && !accumulate && !dw_tile_big(g, 0) && !dw_tile_192x128(g, 0) && sp.si.ips == g.n && tiles >= 96 &&
-        split_blocks * 100 < kTargetBlocks * 97 &&
-        ws_bytes >= kBalanceBytes && g.p < (1l << 31)) {
+    if (!cols && !accumulate && !special_tile && sp.si.ips == g.n && tiles >= 96 &&
+        split_blocks * 100 < kTargetBlocks * 97 && ws_bytes >= kBalanceBytes && g.p < (1l << 31)) {
         WITH_TILE(sel, {
             const long dy_img = (long)g.kn * g.howo;
             if (!span_ok_k(T::BM, g.howo, g.n, dy_img)) return PYDTNN_HIP_ERR_UNSUPPORTED;
@@ -85,68 +115,28 @@ int conv_dw_nchw(const ConvGeom& g, const float* dy, const float* x, const float
         if (rc != kNotBalanced) return rc;
         rc = PYDTNN_HIP_OK;
     }
-    if (!cols && dw_tile_big(g, 0)) {
-        typedef T256x128 T;
-        const long dy_img = (long)g.kn * g.howo;
-        if (!span_ok_k(T::BM, g.howo, sp.si.ips, dy_img)) return PYDTNN_HIP_ERR_UNSUPPORTED;
-        auto al = plain_k<T::BM, true>(dy, g.p * g.kn, g.howo, dy_img, g.kn, g.howo);
-        al.fd_seg = group_div(g.howo, sp.si.ips);
-        Im2colNchwK<T::BN> bl;
-        bl.x = x; bl.g = g;
-        bl.g.fd_howo = group_div(g.howo, sp.si.ips);
-        rc = launch<T>(al, bl, epi_plain(ws, g.k, out_elems, g.kn, g.k, no_epilogue(), no_masks(), sp.splits), g.kn,
-                       g.k, sp.si, sp.splits, stream);
-        if (rc != PYDTNN_HIP_OK) return rc;
-        return launch_splitk_reduce(ws, dw, g.kn, g.k, out_elems, sp.splits, 0, 0, no_epilogue(), accumulate, stream);
-    }
-    if (!cols && dw_tile_192x128(g, 0)) {
-        typedef T128x192 T;
-        const long dy_img = (long)g.kn * g.howo;
-        if (!span_ok_k(T::BM, g.howo, sp.si.ips, dy_img)) return PYDTNN_HIP_ERR_UNSUPPORTED;
-        auto al = plain_k<T::BM, true>(dy, g.p * g.kn, g.howo, dy_img, g.kn, g.howo);
-        al.fd_seg = group_div(g.howo, sp.si.ips);
-        Im2colNchwK<T::BN> bl;
-        bl.x = x; bl.g = g;
-        bl.g.fd_howo = group_div(g.howo, sp.si.ips);
-        rc = launch<T>(al, bl, epi_plain(ws, g.k, out_elems, g.kn, g.k, no_epilogue(), no_masks(), sp.splits), g.kn,
-                       g.k, sp.si, sp.splits, stream);
-        if (rc != PYDTNN_HIP_OK) return rc;
-        return launch_splitk_reduce(ws, dw, g.kn, g.k, out_elems, sp.splits, 0, 0, no_epilogue(), accumulate, stream);
-    }
-    if (!cols && dw_tile_192(g, 0)) {
-        typedef T64x192 T;
-        const long dy_img = (long)g.kn * g.howo;
-        if (!span_ok_k(T::BM, g.howo, sp.si.ips, dy_img)) return PYDTNN_HIP_ERR_UNSUPPORTED;
-        auto al = plain_k<T::BM, true>(dy, g.p * g.kn, g.howo, dy_img, g.kn, g.howo);
-        al.fd_seg = group_div(g.howo, sp.si.ips);
-        Im2colNchwK<T::BN> bl;
-        bl.x = x; bl.g = g;
-        bl.g.fd_howo = group_div(g.howo, sp.si.ips);
-        rc = launch<T>(al, bl, epi_plain(ws, g.k, out_elems, g.kn, g.k, no_epilogue(), no_masks(), sp.splits), g.kn,
-                       g.k, sp.si, sp.splits, stream);
-        if (rc != PYDTNN_HIP_OK) return rc;
-        return launch_splitk_reduce(ws, dw, g.kn, g.k, out_elems, sp.splits, 0, 0, no_epilogue(), accumulate, stream);
-    }
-    WITH_TILE(sel, {
-        // A(m = filter, k = (image, pixel)) = dy[image][filter][pixel]
-        const long dy_img = (long)g.kn * g.howo;
-        if (!span_ok_k(T::BM, g.howo, sp.si.ips, dy_img)) return PYDTNN_HIP_ERR_UNSUPPORTED;
-        auto al = plain_k<T::BM, true>(dy, g.p * g.kn, g.howo, dy_img, g.kn, g.howo);
-        al.fd_seg = group_div(g.howo, sp.si.ips);
-        const EpiPlain ep = epi_plain(ws, g.k, out_elems, g.kn, g.k, no_epilogue(), no_masks(), sp.splits);
-        if (cols) {
-            // B(k = (image, pixel), n = row of cols) = cols[n][image*howo + pixel]
-            if (!span_ok_k(T::BN, g.p, sp.si.ips, g.howo)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+    if (cols) {
+        WITH_TILE(sel, {
+            // A as in the implicit form; B(k = (image, pixel), n = row of cols) = cols[n][image*howo + pixel]
+            const long dy_img = (long)g.kn * g.howo;
+            if (!span_ok_k(T::BM, g.howo, sp.si.ips, dy_img) || !span_ok_k(T::BN, g.p, sp.si.ips, g.howo))
+                return PYDTNN_HIP_ERR_UNSUPPORTED;
+            auto al = plain_k<T::BM, true>(dy, g.p * g.kn, g.howo, dy_img, g.kn, g.howo);
+            al.fd_seg = group_div(g.howo, sp.si.ips);
             auto bl = plain_k<T::BN, true>(cols, (long)g.k * g.p, g.p, g.howo, g.k, g.howo);
             bl.fd_seg = group_div(g.howo, sp.si.ips);
-            rc = launch<T>(al, bl, ep, g.kn, g.k, sp.si, sp.splits, stream);
-        } else {
-            Im2colNchwK<T::BN> bl;
-            bl.x = x; bl.g = g;
-            bl.g.fd_howo = group_div(g.howo, sp.si.ips);
-            rc = launch<T>(al, bl, ep, g.kn, g.k, sp.si, sp.splits, stream);
-        }
-    })
+            rc = launch<T>(al, bl, epi_plain(ws, g.k, out_elems, g.kn, g.k, no_epilogue(), no_masks(), sp.splits), g.kn,
+                           g.k, sp.si, sp.splits, stream);
+        })
+    } else if (dw_tile_big(g, 0)) {
+        rc = dw_nchw_implicit<T256x128>(g, sp, dy, x, ws, stream);
+    } else if (dw_tile_192x128(g, 0)) {
+        rc = dw_nchw_implicit<T128x192>(g, sp, dy, x, ws, stream);
+    } else if (dw_tile_192(g, 0)) {
+        rc = dw_nchw_implicit<T64x192>(g, sp, dy, x, ws, stream);
+    } else {
+        WITH_TILE(sel, { rc = dw_nchw_implicit<T>(g, sp, dy, x, ws, stream); })
+    }
     if (rc != PYDTNN_HIP_OK) return rc;
     return launch_splitk_reduce(ws, dw, g.kn, g.k, out_elems, sp.splits, 0, 0, no_epilogue(), accumulate, stream);
 }
@@ -159,57 +149,23 @@ int conv_dw_nhwc(const ConvGeom& g, const float* dy, const float* x, const float
     if (!ws || ws_bytes < (size_t)sp.splits * out_elems * 4) return PYDTNN_HIP_ERR_WORKSPACE;
     const TileSel sel = pick_tile(g.k, g.kn);
     int rc = PYDTNN_HIP_OK;
-    if (!rows && dw_tile_big(g, 1)) {
-        typedef T256x128 T;
-        auto bl = plain_mn<T::BN>(dy, g.p * g.kn, g.kn, (long)g.howo * g.kn, g.kn);
-        Im2rowNhwcMN<T::BM> al;
-        al.x = x; al.g = g;
-        al.g.fd_howo = group_div(g.howo, sp.si.ips);
-        rc = launch<T>(al, bl, epi_plain(ws, g.kn, out_elems, g.k, g.kn, no_epilogue(), no_masks(), sp.splits), g.k,
-                       g.kn, sp.si, sp.splits, stream);
-        if (rc != PYDTNN_HIP_OK) return rc;
-        return launch_splitk_reduce(ws, dw, g.k, g.kn, out_elems, sp.splits, g.c, g.khw, no_epilogue(), accumulate,
-                                    stream);
-    }
-    if (!rows && dw_tile_192x128(g, 1)) {
-        typedef T192x128 T;
-        auto bl = plain_mn<T::BN>(dy, g.p * g.kn, g.kn, (long)g.howo * g.kn, g.kn);
-        Im2rowNhwcMN<T::BM> al;
-        al.x = x; al.g = g;
-        al.g.fd_howo = group_div(g.howo, sp.si.ips);
-        rc = launch<T>(al, bl, epi_plain(ws, g.kn, out_elems, g.k, g.kn, no_epilogue(), no_masks(), sp.splits), g.k,
-                       g.kn, sp.si, sp.splits, stream);
-        if (rc != PYDTNN_HIP_OK) return rc;
-        return launch_splitk_reduce(ws, dw, g.k, g.kn, out_elems, sp.splits, g.c, g.khw, no_epilogue(), accumulate,
-                                    stream);
-    }
-    if (!rows && dw_tile_192(g, 1)) {
-        typedef T192x64 T;
-        auto bl = plain_mn<T::BN>(dy, g.p * g.kn, g.kn, (long)g.howo * g.kn, g.kn);
-        Im2rowNhwcMN<T::BM> al;
-        al.x = x; al.g = g;
-        al.g.fd_howo = group_div(g.howo, sp.si.ips);
-        rc = launch<T>(al, bl, epi_plain(ws, g.kn, out_elems, g.k, g.kn, no_epilogue(), no_masks(), sp.splits), g.k,
-                       g.kn, sp.si, sp.splits, stream);
-        if (rc != PYDTNN_HIP_OK) return rc;
-        return launch_splitk_reduce(ws, dw, g.k, g.kn, out_elems, sp.splits, g.c, g.khw, no_epilogue(), accumulate,
-                                    stream);
-    }
-    WITH_TILE(sel, {
-        // B(k = (image, pixel), n = filter) = dy[(image*howo + pixel)*kn + n]
-        auto bl = plain_mn<T::BN>(dy, g.p * g.kn, g.kn, (long)g.howo * g.kn, g.kn);
-        const EpiPlain ep = epi_plain(ws, g.kn, out_elems, g.k, g.kn, no_epilogue(), no_masks(), sp.splits);
-        if (rows) {
-            // A(m = column of rows, k) = rows[(image*howo + pixel)*K + m]
+    if (rows) {
+        WITH_TILE(sel, {
+            // A(m = column of rows, k) = rows[(image*howo + pixel)*K + m]; B as in the implicit form
             auto al = plain_mn<T::BM>(rows, g.p * g.k, g.k, (long)g.howo * g.k, g.k);
-            rc = launch<T>(al, bl, ep, g.k, g.kn, sp.si, sp.splits, stream);
-        } else {
-            Im2rowNhwcMN<T::BM> al;
-            al.x = x; al.g = g;
-            al.g.fd_howo = group_div(g.howo, sp.si.ips);
-            rc = launch<T>(al, bl, ep, g.k, g.kn, sp.si, sp.splits, stream);
-        }
-    })
+            auto bl = plain_mn<T::BN>(dy, g.p * g.kn, g.kn, (long)g.howo * g.kn, g.kn);
+            rc = launch<T>(al, bl, epi_plain(ws, g.kn, out_elems, g.k, g.kn, no_epilogue(), no_masks(), sp.splits), g.k,
+                           g.kn, sp.si, sp.splits, stream);
+        })
+    } else if (dw_tile_big(g, 1)) {
+        rc = dw_nhwc_implicit<T256x128>(g, sp, dy, x, ws, stream);
+    } else if (dw_tile_192x128(g, 1)) {
+        rc = dw_nhwc_implicit<T192x128>(g, sp, dy, x, ws, stream);
+    } else if (dw_tile_192(g, 1)) {
+        rc = dw_nhwc_implicit<T192x64>(g, sp, dy, x, ws, stream);
+    } else {
+        WITH_TILE(sel, { rc = dw_nhwc_implicit<T>(g, sp, dy, x, ws, stream); })
+    }
     if (rc != PYDTNN_HIP_OK) return rc;
     // implicit rows come out in (i, j, c) order; materialised x_rows already has the (c, i, j) order
     const int perm_c = rows ? 0 : g.c;
