@@ -1653,7 +1653,10 @@ inline int launch_balanced(const AL& al, const BL& bl, const EP& ep, long m, lon
     sk.k = k;
     sk.partial = partial;
     const long total = (long)sk.sk_tiles * units;
-    sk.sk_blocks = (int)(total / 4 < resident ? (total / 4 > 0 ? total / 4 : 1) : resident);
+    // at least two units (four reduction steps) per piece: with few cut tiles and a short reduction the pieces
+    // of four units that this used to deal added a fifth to the longest workgroup's run
+    const long pieces = total / 2;
+    sk.sk_blocks = (int)(pieces < resident ? (pieces > 0 ? pieces : 1) : resident);
     constexpr int kPerCu = WorkgroupsPerCu<T, AL, BL>::value;
     if constexpr (kPerCu == 3)
         hipLaunchKernelGGL((gemm_streamk_kernel<T, AL, BL, EP>), dim3((unsigned)resident), dim3(kThreads), 0, stream,
