@@ -198,18 +198,27 @@ __global__ void __launch_bounds__(kThreads) bias_grad_nchw_stage1(const float* _
     const int ch = blockIdx.x, s = blockIdx.y;
     const int n0 = s * per, n1 = min(n, n0 + per);
     float acc = 0.0f;
-    for (int nn = n0; nn < n1; ++nn) {
-        const float* plane = dy + ((long)nn * c + ch) * hw;
-        if (VEC4) {
-            const float4* p4 = reinterpret_cast<const float4*>(plane);
-            float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
-            for (int i = threadIdx.x; i < hw / 4; i += kThreads) {
-                const float4 v = p4[i];
-                a0 += v.x; a1 += v.y; a2 += v.z; a3 += v.w;
+    if (!VEC4 && hw < kThreads) {
+        // planes smaller than the workgroup: its threads walk the (image, pixel) pairs of the slice together
+        const uint32_t count = (uint32_t)(n1 - n0) * (uint32_t)hw;
+        for (uint32_t e = threadIdx.x; e < count; e += kThreads) {
+            const uint32_t nn = e / (uint32_t)hw, i = e - nn * (uint32_t)hw;
+            acc += dy[((long)(n0 + (int)nn) * c + ch) * hw + i];
+        }
+    } else {
+        for (int nn = n0; nn < n1; ++nn) {
+            const float* plane = dy + ((long)nn * c + ch) * hw;
+            if (VEC4) {
+                const float4* p4 = reinterpret_cast<const float4*>(plane);
+                float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+                for (int i = threadIdx.x; i < hw / 4; i += kThreads) {
+                    const float4 v = p4[i];
+                    a0 += v.x; a1 += v.y; a2 += v.z; a3 += v.w;
+                }
+                acc += (a0 + a1) + (a2 + a3);
+            } else {
+                for (int i = threadIdx.x; i < hw; i += kThreads) acc += plane[i];
             }
-            acc += (a0 + a1) + (a2 + a3);
-        } else {
-            for (int i = threadIdx.x; i < hw; i += kThreads) acc += plane[i];
         }
     }
     const float tot = block_sum(acc);
@@ -734,10 +743,20 @@ __global__ void __launch_bounds__(kThreads) bn_reduce_nchw_stage1(const float* _
     const int n0 = s * per, n1 = min(n, n0 + per);
     const float shift = MODE == 1 ? p0[ch] : 0.0f;
     float a = 0.0f, b = 0.0f;
-    for (int nn = n0; nn < n1; ++nn) {
-        const long base = ((long)nn * c + ch) * hw;
-        for (int i = threadIdx.x; i < hw; i += kThreads)
-            bn_term<MODE>(x[base + i], MODE == 2 ? q[base + i] : 0.0f, shift, &a, &b);
+    if (hw >= kThreads) {
+        for (int nn = n0; nn < n1; ++nn) {
+            const long base = ((long)nn * c + ch) * hw;
+            for (int i = threadIdx.x; i < hw; i += kThreads)
+                bn_term<MODE>(x[base + i], MODE == 2 ? q[base + i] : 0.0f, shift, &a, &b);
+        }
+    } else {
+        // planes smaller than the workgroup: its threads walk the (image, pixel) pairs of the slice together
+        const uint32_t count = (uint32_t)(n1 - n0) * (uint32_t)hw;
+        for (uint32_t e = threadIdx.x; e < count; e += kThreads) {
+            const uint32_t nn = e / (uint32_t)hw, i = e - nn * (uint32_t)hw;
+            const long at = ((long)(n0 + (int)nn) * c + ch) * hw + i;
+            bn_term<MODE>(x[at], MODE == 2 ? q[at] : 0.0f, shift, &a, &b);
+        }
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
@@ -785,6 +804,82 @@ __global__ void __launch_bounds__(kThreads) bn_reduce_rows_stage1(const float* _
     }
 }
 
+// (rows, C) with a row of `lanes` = C/4 quads, lanes a power of two <= kThreads, 16-byte aligned tensors: as
+// bias_grad_rows_quads_stage1, whole rows per 128-bit load and several loads in flight per lane; up to
+// kBnSlices row slices.  A row beyond the slice reads as the value that adds nothing (0, or p0 for MODE 1).
+template <int MODE>
+__global__ void __launch_bounds__(kThreads) bn_reduce_rows_quads_stage1(const float4* __restrict__ x,
+                                                                       const float4* __restrict__ q,
+                                                                       const float4* __restrict__ p0,
+                                                                       float* __restrict__ partial, long rows,
+                                                                       int lanes, long per, int slices)
+{
+    constexpr int kInFlight = MODE == 2 ? 4 : 8;
+    __shared__ float4 red[MODE == 2 ? 2 : 1][kThreads];
+    const int cl = threadIdx.x & (lanes - 1);
+    const int row_lanes = kThreads / lanes, rl = threadIdx.x / lanes;
+    const long r0 = (long)blockIdx.x * per;
+    const long r1 = r0 + per < rows ? r0 + per : rows;
+    const float4 zero = float4{0.0f, 0.0f, 0.0f, 0.0f};
+    const float4 shift = MODE == 1 ? p0[cl] : zero;
+    float4 a[kInFlight], b[kInFlight];
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u) a[u] = b[u] = zero;
+    for (long r = r0 + rl; r < r1; r += (long)row_lanes * kInFlight) {
+        float4 v[kInFlight], w[kInFlight];
+#pragma unroll
+        for (int u = 0; u < kInFlight; ++u) {
+            const long rr = r + (long)u * row_lanes;
+            v[u] = rr < r1 ? x[rr * lanes + cl] : shift;
+            w[u] = MODE == 2 && rr < r1 ? q[rr * lanes + cl] : zero;
+        }
+#pragma unroll
+        for (int u = 0; u < kInFlight; ++u) {
+            bn_term<MODE>(v[u].x, w[u].x, shift.x, &a[u].x, &b[u].x);
+            bn_term<MODE>(v[u].y, w[u].y, shift.y, &a[u].y, &b[u].y);
+            bn_term<MODE>(v[u].z, w[u].z, shift.z, &a[u].z, &b[u].z);
+            bn_term<MODE>(v[u].w, w[u].w, shift.w, &a[u].w, &b[u].w);
+        }
+    }
+    float4 ta = a[0], tb = b[0];
+#pragma unroll
+    for (int u = 1; u < kInFlight; ++u) {
+        ta.x += a[u].x; ta.y += a[u].y; ta.z += a[u].z; ta.w += a[u].w;
+        tb.x += b[u].x; tb.y += b[u].y; tb.z += b[u].z; tb.w += b[u].w;
+    }
+    red[0][threadIdx.x] = ta;
+    if (MODE == 2) red[MODE == 2 ? 1 : 0][threadIdx.x] = tb;
+    __syncthreads();
+    if (rl == 0) {
+        for (int i = 1; i < row_lanes; ++i) {
+            const float4 oa = red[0][i * lanes + cl];
+            ta.x += oa.x; ta.y += oa.y; ta.z += oa.z; ta.w += oa.w;
+            if (MODE == 2) {
+                const float4 ob = red[MODE == 2 ? 1 : 0][i * lanes + cl];
+                tb.x += ob.x; tb.y += ob.y; tb.z += ob.z; tb.w += ob.w;
+            }
+        }
+        reinterpret_cast<float4*>(partial + (long)blockIdx.x * lanes * 4)[cl] = ta;
+        if (MODE == 2) reinterpret_cast<float4*>(partial + ((long)slices + blockIdx.x) * lanes * 4)[cl] = tb;
+    }
+}
+
+// Sum over slices of partial[s*c + ch] for the second stages: 16 channels x 16 slice lanes per workgroup, each
+// lane adding its slices in ascending order, then the lanes' sums in lane order (thread sl == 0 gets the total).
+__device__ __forceinline__ float bn_sum_slices(const float* __restrict__ partial, int c, int slices, int ch, int sl,
+                                               float (*red)[17])
+{
+    float acc = 0.0f;
+    if (ch < c)
+        for (int s = sl; s < slices; s += 16) acc += partial[(long)s * c + ch];
+    __syncthreads();  // red may still be read from a previous call
+    red[sl][threadIdx.x & 15] = acc;
+    __syncthreads();
+    float t = red[0][threadIdx.x & 15];
+    for (int i = 1; i < 16; ++i) t += red[i][threadIdx.x & 15];
+    return t;
+}
+
 // Second stage of the forward statistics.  PASS 0: mu = sum / count.  PASS 1: var = sum / count,
 // std = sqrt(var + eps), running statistics updated as momentum*running + (1-momentum)*new.
 template <int PASS>
@@ -795,10 +890,10 @@ __global__ void __launch_bounds__(kThreads) bn_stats_stage2(const float* __restr
                                                            float* __restrict__ running_var, float momentum,
                                                            float one_minus_momentum)
 {
-    const int ch = blockIdx.x * kThreads + threadIdx.x;
-    if (ch >= c) return;
-    float acc = 0.0f;
-    for (int s = 0; s < slices; ++s) acc += partial[(long)s * c + ch];
+    __shared__ float red[16][17];
+    const int ch = blockIdx.x * 16 + (threadIdx.x & 15), sl = threadIdx.x >> 4;
+    const float acc = bn_sum_slices(partial, c, slices, ch, sl, red);
+    if (sl != 0 || ch >= c) return;
     const float mean = acc / count;
     if (PASS == 0) {
         mu[ch] = mean;
@@ -813,13 +908,11 @@ __global__ void __launch_bounds__(kThreads) bn_stats_stage2(const float* __restr
 __global__ void __launch_bounds__(kThreads) bn_grads_stage2(const float* __restrict__ partial, int c, int slices,
                                                            float* __restrict__ dgamma, float* __restrict__ dbeta)
 {
-    const int ch = blockIdx.x * kThreads + threadIdx.x;
-    if (ch >= c) return;
-    float a = 0.0f, b = 0.0f;
-    for (int s = 0; s < slices; ++s) {
-        a += partial[(long)s * c + ch];
-        b += partial[((long)slices + s) * c + ch];
-    }
+    __shared__ float red[16][17];
+    const int ch = blockIdx.x * 16 + (threadIdx.x & 15), sl = threadIdx.x >> 4;
+    const float a = bn_sum_slices(partial, c, slices, ch, sl, red);
+    const float b = bn_sum_slices(partial + (long)slices * c, c, slices, ch, sl, red);
+    if (sl != 0 || ch >= c) return;
     dbeta[ch] = a;
     dgamma[ch] = b;
 }
@@ -1061,9 +1154,12 @@ int launch_bias_grad(const float* dy, float* db, long outer, int channels, int i
     if (inner > 1) {
         const int n = (int)outer;
         slices = n < 64 ? n : 64;
+        // small planes: a slice holds at least 2048 elements of a channel
+        const long by_size = outer * inner / 2048;
+        if (inner < kThreads && slices > by_size) slices = by_size < 1 ? 1 : (int)by_size;
         const int per = (n + slices - 1) / slices;
         slices = (n + per - 1) / per;
-        if (inner % 4 == 0 && (reinterpret_cast<uintptr_t>(dy) & 15) == 0)
+        if (inner >= kThreads && inner % 4 == 0 && (reinterpret_cast<uintptr_t>(dy) & 15) == 0)
             hipLaunchKernelGGL(bias_grad_nchw_stage1<true>, dim3(channels, slices), dim3(kThreads), 0, stream, dy,
                                workspace, n, channels, inner, per);
         else
@@ -1259,12 +1355,17 @@ int launch_cce(const float* y_pred, const float* y_targ, float* dx, float* loss,
     return PYDTNN_HIP_OK;
 }
 
-// Slices of the outer axis for a two-stage channel reduction; at most 64.
+// Slices of the outer axis for a two-stage channel reduction; at most 64 (kBnSlices for the 16-byte row kernel).
+constexpr int kBnSlices = 512;
+
 static int bn_slices(long outer, int inner, long* per)
 {
     long slices;
     if (inner > 1) {
         slices = outer < 64 ? outer : 64;
+        // small planes: a slice holds at least 2048 elements of a channel
+        const long by_size = outer * inner / 2048;
+        if (inner < kThreads && slices > by_size) slices = by_size < 1 ? 1 : by_size;
     } else {
         slices = outer < 64 * 4 ? (outer + 3) / 4 : 64;
     }
@@ -1277,18 +1378,32 @@ static void bn_reduce_stage1(const float* x, const float* q, const float* p0, fl
                              int inner, hipStream_t stream, int* slices_out)
 {
     long per;
-    const int slices = bn_slices(outer, inner, &per);
-    if (inner > 1)
+    int slices = bn_slices(outer, inner, &per);
+    const int lanes = channels / 4;
+    const auto aligned16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    if (inner > 1) {
         hipLaunchKernelGGL(bn_reduce_nchw_stage1<MODE>, dim3(channels, slices), dim3(kThreads), 0, stream, x, q, p0,
                            partial, (int)outer, channels, inner, (int)per, slices);
-    else
+    } else if (channels % 4 == 0 && lanes <= kThreads && (lanes & (lanes - 1)) == 0 && aligned16(x) &&
+               (MODE != 2 || aligned16(q)) && (MODE != 1 || aligned16(p0)) && aligned16(partial)) {
+        // a slice is at least 32 rows per row lane
+        const long rows_per_load = kThreads / lanes;
+        const long want = (outer + rows_per_load * 32 - 1) / (rows_per_load * 32);
+        slices = (int)(want < kBnSlices ? want : kBnSlices);
+        per = (outer + slices - 1) / slices;
+        slices = (int)((outer + per - 1) / per);
+        hipLaunchKernelGGL(bn_reduce_rows_quads_stage1<MODE>, dim3(slices), dim3(kThreads), 0, stream,
+                           reinterpret_cast<const float4*>(x), reinterpret_cast<const float4*>(q),
+                           reinterpret_cast<const float4*>(p0), partial, outer, lanes, per, slices);
+    } else {
         hipLaunchKernelGGL(bn_reduce_rows_stage1<MODE>, dim3(slices, (channels + 63) / 64), dim3(kThreads), 0, stream,
                            x, q, p0, partial, outer, channels, per, slices);
+    }
     *slices_out = slices;
 }
 
-// floats: two sets of 64 partial sums per channel, then mu
-size_t bn_training_workspace_floats(int channels) { return (size_t)(2 * 64 + 1) * channels; }
+// floats: two sets of kBnSlices partial sums per channel, then mu (16-byte aligned when the workspace is)
+size_t bn_training_workspace_floats(int channels) { return (size_t)(2 * kBnSlices + 4) * channels; }
 
 // Algorithmic bytes: x read three times (mean, variance, normalise), y and xn written: 20 bytes per element.
 int launch_bn_training_fwd(const float* x, float* y, float* xn, float* std_out, const float* gamma, const float* beta,
@@ -1298,18 +1413,18 @@ int launch_bn_training_fwd(const float* x, float* y, float* xn, float* std_out, 
     if (outer <= 0 || channels <= 0 || inner <= 0) return PYDTNN_HIP_ERR_INVALID;
     if (inner > 1 && outer >= (1l << 31)) return PYDTNN_HIP_ERR_UNSUPPORTED;
     float* partial = workspace;
-    float* mu = workspace + (size_t)2 * 64 * channels;
+    float* mu = workspace + (size_t)2 * kBnSlices * channels;
     const float count = (float)(outer * inner);
     const long total = outer * channels * inner;
     int slices = 0;
     bn_reduce_stage1<0>(x, nullptr, nullptr, partial, outer, channels, inner, stream, &slices);
     HIP_RETURN_IF_LAUNCH_FAILED();
-    hipLaunchKernelGGL(bn_stats_stage2<0>, dim3(blocks_for(channels)), dim3(kThreads), 0, stream, partial, channels,
+    hipLaunchKernelGGL(bn_stats_stage2<0>, dim3((channels + 15) / 16), dim3(kThreads), 0, stream, partial, channels,
                        slices, count, mu, std_out, eps, running_mean, running_var, momentum, one_minus_momentum);
     HIP_RETURN_IF_LAUNCH_FAILED();
     bn_reduce_stage1<1>(x, nullptr, mu, partial, outer, channels, inner, stream, &slices);
     HIP_RETURN_IF_LAUNCH_FAILED();
-    hipLaunchKernelGGL(bn_stats_stage2<1>, dim3(blocks_for(channels)), dim3(kThreads), 0, stream, partial, channels,
+    hipLaunchKernelGGL(bn_stats_stage2<1>, dim3((channels + 15) / 16), dim3(kThreads), 0, stream, partial, channels,
                        slices, count, mu, std_out, eps, running_mean, running_var, momentum, one_minus_momentum);
     HIP_RETURN_IF_LAUNCH_FAILED();
     hipLaunchKernelGGL(bn_train_apply_kernel, dim3(blocks_for(total)), dim3(kThreads), 0, stream, x, y, xn, total,
@@ -1329,7 +1444,7 @@ int launch_bn_training_bwd(const float* dy, const float* xn, const float* std_in
     int slices = 0;
     bn_reduce_stage1<2>(dy, xn, nullptr, workspace, outer, channels, inner, stream, &slices);
     HIP_RETURN_IF_LAUNCH_FAILED();
-    hipLaunchKernelGGL(bn_grads_stage2, dim3(blocks_for(channels)), dim3(kThreads), 0, stream, workspace, channels,
+    hipLaunchKernelGGL(bn_grads_stage2, dim3((channels + 15) / 16), dim3(kThreads), 0, stream, workspace, channels,
                        slices, dgamma, dbeta);
     HIP_RETURN_IF_LAUNCH_FAILED();
     if (dx) {

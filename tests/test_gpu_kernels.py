@@ -483,7 +483,13 @@ def test_maxpool_nhwc_matches_oracle(ops, oracle):
 
 
 @pytest.mark.parametrize("fmt,shape", [("NCHW", (8, 6, 5, 7)), ("NCHW", (70, 3, 4, 4)), ("NHWC", (8, 5, 7, 6)),
-                                       ("NHWC", (3, 9, 9, 130)), ("2D", (64, 10)), ("2D", (300, 70)), ("2D", (2, 3))])
+                                       ("NHWC", (3, 9, 9, 130)), ("2D", (64, 10)), ("2D", (300, 70)), ("2D", (2, 3)),
+                                       # row widths of a power of two of quads: the 16-byte reduction, one to many
+                                       # row slices, ragged last slice
+                                       ("NHWC", (4, 12, 12, 64)), ("NHWC", (2, 40, 41, 8)), ("NHWC", (3, 7, 7, 256)),
+                                       ("2D", (513, 128)), ("2D", (40001, 4)), ("NHWC", (1, 3, 3, 1024)),
+                                       # planes smaller than a workgroup: (image, pixel) pairs walked together
+                                       ("NCHW", (20, 5, 3, 3)), ("NCHW", (300, 4, 7, 7)), ("NCHW", (9, 2, 15, 17))])
 def test_bn_training_forward_backward(ops, oracle, fmt, shape):
     announce("bn training", (fmt, shape))
     rng = np.random.default_rng(sum(shape))
