@@ -478,6 +478,84 @@ __global__ void __launch_bounds__(kThreads) max_pool_bwd_windows_nchw_kernel(con
     }
 }
 
+// Output rows (or columns) whose window covers input coordinate `t = coord + padding`, for windows of `k` taps at
+// stride `stride` without dilation: [lo, hi], empty when lo > hi.
+__device__ __forceinline__ void pool_window_range(int t, int k, int stride, const FastDiv fd_stride, int extent,
+                                                  int* lo, int* hi)
+{
+    const int first = t - (k - 1);
+    *hi = min((int)fd_div((uint32_t)t, fd_stride), extent - 1);
+    *lo = first <= 0 ? 0 : (int)fd_div((uint32_t)(first + stride - 1), fd_stride);
+}
+
+// Backward for square windows without dilation that overlap or leave gaps (any stride and padding): the windows
+// that cover an element form a small rectangle of outputs (at most ceil(k/stride) per axis), worked out directly
+// instead of testing all k*k taps; visited in ascending (oy, ox) like the reference's scatter loop.  With
+// kh == kw the reference's decode (idx / kh, idx % kw) is the plain one, so a window's maximum lies on this
+// element exactly when its index equals ii*kw + jj.
+// PER_AXIS = 2: at most two windows per axis cover an element (k <= 2*stride): the four candidates are loaded
+// without conditions (out-of-range ones from a clamped address, masked out afterwards) so that no load waits for
+// a comparison; adding 0.0f for a window whose maximum lies elsewhere leaves the sum's bits unchanged.
+template <int PER_AXIS>
+__global__ void __launch_bounds__(kThreads) max_pool_bwd_ranges_nchw_kernel(const float* __restrict__ dy,
+                                                                           const int32_t* __restrict__ idx_max,
+                                                                           float* __restrict__ dx, ConvGeom g,
+                                                                           const int8_t* __restrict__ gate)
+{
+    const uint32_t hw = (uint32_t)(g.h * g.w);
+    const uint32_t pix = blockIdx.x * kThreads + threadIdx.x;
+    if (pix >= hw) return;
+    const int hh = (int)fd_div(pix, g.fd_w);
+    const int ww = (int)pix - hh * g.w;
+    const int ty = hh + g.vpadding, tx = ww + g.hpadding;
+    int oy0, oy1, ox0, ox1;
+    pool_window_range(ty, g.kh, g.vstride, g.fd_vs, g.ho, &oy0, &oy1);
+    pool_window_range(tx, g.kw, g.hstride, g.fd_hs, g.wo, &ox0, &ox1);
+    const uint32_t planes = (uint32_t)(g.n * g.c);
+    if (PER_AXIS == 2) {
+        int at[4], code[4];
+        bool live[4];
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                const int oy = oy0 + a, ox = ox0 + b;
+                live[a * 2 + b] = oy <= oy1 && ox <= ox1;
+                at[a * 2 + b] = live[a * 2 + b] ? oy * g.wo + ox : 0;
+                code[a * 2 + b] = (ty - oy * g.vstride) * g.kw + (tx - ox * g.hstride);
+            }
+        for (uint32_t plane = blockIdx.y; plane < planes; plane += gridDim.y) {
+            const float* gy = dy + (long)plane * g.howo;
+            const int32_t* gi = idx_max + (long)plane * g.howo;
+            int rec[4];
+            float grad[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) { rec[q] = gi[at[q]]; grad[q] = gy[at[q]]; }
+            float acc = 0.0f;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) acc += live[q] && rec[q] == code[q] ? grad[q] : 0.0f;
+            if (gate) acc *= (float)gate[(long)plane * hw + pix];
+            dx[(long)plane * hw + pix] = acc;
+        }
+        return;
+    }
+    for (uint32_t plane = blockIdx.y; plane < planes; plane += gridDim.y) {
+        const float* gy = dy + (long)plane * g.howo;
+        const int32_t* gi = idx_max + (long)plane * g.howo;
+        float acc = 0.0f;
+        for (int oy = oy0; oy <= oy1; ++oy) {
+            const int ii = ty - oy * g.vstride;
+            for (int ox = ox0; ox <= ox1; ++ox) {
+                const int jj = tx - ox * g.hstride;
+                const float grad = gy[oy * g.wo + ox];
+                acc += gi[oy * g.wo + ox] == ii * g.kw + jj ? grad : 0.0f;
+            }
+        }
+        if (gate) acc *= (float)gate[(long)plane * hw + pix];
+        dx[(long)plane * hw + pix] = acc;
+    }
+}
+
 // Backward in gather form: one thread per dx element sums dy of every window whose recorded
 // maximum decodes to this element.  The decode is the reference's own
 // (ii = idx / kh, jj = idx % kw, max_pool_2d_nchw_cython.pyx:204-205).  Windows are visited in
@@ -638,6 +716,69 @@ __global__ void __launch_bounds__(kThreads) max_pool_bwd_nhwc_kernel(const float
                 const uint32_t ri = fd_div(rec, g.fd_kh);
                 const uint32_t rj = rec - fd_div(rec, g.fd_kw) * g.kw;
                 if ((int)ri == ii && (int)rj == jj) acc += dy[at];
+            }
+        }
+        if (gate) acc *= (float)gate[(size_t)nn * per_image + e];
+        dx[(size_t)nn * per_image + e] = acc;
+    }
+}
+
+// The NHWC twin of max_pool_bwd_ranges_nchw_kernel: lanes along the channels.
+template <int PER_AXIS>
+__global__ void __launch_bounds__(kThreads) max_pool_bwd_ranges_nhwc_kernel(const float* __restrict__ dy,
+                                                                           const int32_t* __restrict__ idx_max,
+                                                                           float* __restrict__ dx, ConvGeom g,
+                                                                           int c_exact,
+                                                                           const int8_t* __restrict__ gate)
+{
+    const uint32_t per_image = (uint32_t)(g.h * g.w * g.c);
+    const uint32_t e = blockIdx.x * kThreads + threadIdx.x;
+    if (e >= per_image) return;
+    const uint32_t pix = fd_div_checked(e, g.fd_c, c_exact);
+    const uint32_t cc = e - pix * g.c;
+    const int hh = (int)fd_div(pix, g.fd_w);
+    const int ww = (int)pix - hh * g.w;
+    const int ty = hh + g.vpadding, tx = ww + g.hpadding;
+    int oy0, oy1, ox0, ox1;
+    pool_window_range(ty, g.kh, g.vstride, g.fd_vs, g.ho, &oy0, &oy1);
+    pool_window_range(tx, g.kw, g.hstride, g.fd_hs, g.wo, &ox0, &ox1);
+    if (PER_AXIS == 2) {
+        size_t at[4];
+        int code[4];
+        bool live[4];
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                const int oy = oy0 + a, ox = ox0 + b;
+                live[a * 2 + b] = oy <= oy1 && ox <= ox1;
+                at[a * 2 + b] = (live[a * 2 + b] ? (size_t)(oy * g.wo + ox) * g.c : 0) + cc;
+                code[a * 2 + b] = (ty - oy * g.vstride) * g.kw + (tx - ox * g.hstride);
+            }
+        for (uint32_t nn = blockIdx.y; nn < (uint32_t)g.n; nn += gridDim.y) {
+            const size_t base = (size_t)nn * g.howo * g.c;
+            int rec[4];
+            float grad[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) { rec[q] = idx_max[base + at[q]]; grad[q] = dy[base + at[q]]; }
+            float acc = 0.0f;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) acc += live[q] && rec[q] == code[q] ? grad[q] : 0.0f;
+            if (gate) acc *= (float)gate[(size_t)nn * per_image + e];
+            dx[(size_t)nn * per_image + e] = acc;
+        }
+        return;
+    }
+    for (uint32_t nn = blockIdx.y; nn < (uint32_t)g.n; nn += gridDim.y) {
+        const size_t base = (size_t)nn * g.howo * g.c + cc;
+        float acc = 0.0f;
+        for (int oy = oy0; oy <= oy1; ++oy) {
+            const int ii = ty - oy * g.vstride;
+            for (int ox = ox0; ox <= ox1; ++ox) {
+                const int jj = tx - ox * g.hstride;
+                const size_t at = base + (size_t)(oy * g.wo + ox) * g.c;
+                const float grad = dy[at];
+                acc += idx_max[at] == ii * g.kw + jj ? grad : 0.0f;
             }
         }
         if (gate) acc *= (float)gate[(size_t)nn * per_image + e];
@@ -1254,6 +1395,10 @@ int launch_max_pool_bwd_nchw(const float* dy, const int32_t* idx_max, float* dx,
                                g, gate);
     } else if (tiled)
         hipLaunchKernelGGL(max_pool_bwd_nchw_kernel<true>, grid, dim3(kThreads), 0, stream, dy, idx_max, dx, g, gate);
+    else if (g.kh == g.kw && g.vdilation == 1 && g.hdilation == 1 && g.kh <= 2 * g.vstride && g.kw <= 2 * g.hstride)
+        hipLaunchKernelGGL(max_pool_bwd_ranges_nchw_kernel<2>, grid, dim3(kThreads), 0, stream, dy, idx_max, dx, g, gate);
+    else if (g.kh == g.kw && g.vdilation == 1 && g.hdilation == 1)
+        hipLaunchKernelGGL(max_pool_bwd_ranges_nchw_kernel<0>, grid, dim3(kThreads), 0, stream, dy, idx_max, dx, g, gate);
     else
         hipLaunchKernelGGL(max_pool_bwd_nchw_kernel<false>, grid, dim3(kThreads), 0, stream, dy, idx_max, dx, g, gate);
     HIP_RETURN_IF_LAUNCH_FAILED();
@@ -1311,8 +1456,15 @@ int launch_max_pool_bwd_nhwc(const float* dy, const int32_t* idx_max, float* dx,
     }
     const int c_exact = (unsigned long)(per_image + kThreads) * (unsigned long)g.c < (1ul << 32);
     dim3 grid(blocks_for(per_image), (unsigned)(g.n < 65535 ? g.n : 65535));
-    hipLaunchKernelGGL(max_pool_bwd_nhwc_kernel, grid, dim3(kThreads), 0, stream, dy, idx_max, dx, g, c_exact,
-                       gate);
+    if (g.kh == g.kw && g.vdilation == 1 && g.hdilation == 1 && g.kh <= 2 * g.vstride && g.kw <= 2 * g.hstride)
+        hipLaunchKernelGGL(max_pool_bwd_ranges_nhwc_kernel<2>, grid, dim3(kThreads), 0, stream, dy, idx_max, dx, g,
+                           c_exact, gate);
+    else if (g.kh == g.kw && g.vdilation == 1 && g.hdilation == 1)
+        hipLaunchKernelGGL(max_pool_bwd_ranges_nhwc_kernel<0>, grid, dim3(kThreads), 0, stream, dy, idx_max, dx, g,
+                           c_exact, gate);
+    else
+        hipLaunchKernelGGL(max_pool_bwd_nhwc_kernel, grid, dim3(kThreads), 0, stream, dy, idx_max, dx, g, c_exact,
+                           gate);
     HIP_RETURN_IF_LAUNCH_FAILED();
     return PYDTNN_HIP_OK;
 }
