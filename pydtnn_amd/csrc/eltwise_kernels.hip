@@ -408,6 +408,85 @@ __global__ void __launch_bounds__(kThreads) max_pool_fwd_nchw_kernel(const float
     }
 }
 
+// Forward for K x K windows without dilation (any stride and padding): the K*K taps of a window are loaded
+// without conditions (taps outside the plane from a clamped address, masked out afterwards), their offsets and
+// masks worked out once per thread; the taps are then compared in the reference's order (first maximum wins).
+template <int K>
+__global__ void __launch_bounds__(kThreads) max_pool_fwd_square_nchw_kernel(const float* __restrict__ x,
+                                                                           float* __restrict__ y,
+                                                                           int32_t* __restrict__ idx_max, ConvGeom g)
+{
+    const uint32_t pix = blockIdx.x * kThreads + threadIdx.x;
+    if (pix >= (uint32_t)g.howo) return;
+    const int oy = (int)fd_div(pix, g.fd_wo);
+    const int ox = (int)pix - oy * g.wo;
+    const int y0 = g.vstride * oy - g.vpadding, x0 = g.hstride * ox - g.hpadding;
+    int off[K * K];
+    bool live[K * K];
+#pragma unroll
+    for (int ii = 0; ii < K; ++ii)
+#pragma unroll
+        for (int jj = 0; jj < K; ++jj) {
+            const bool ok = (unsigned)(y0 + ii) < (unsigned)g.h && (unsigned)(x0 + jj) < (unsigned)g.w;
+            live[ii * K + jj] = ok;
+            off[ii * K + jj] = ok ? (y0 + ii) * g.w + x0 + jj : 0;
+        }
+    const uint32_t planes = (uint32_t)(g.n * g.c);
+    for (uint32_t plane = blockIdx.y; plane < planes; plane += gridDim.y) {
+        const float* src = x + (long)plane * g.h * g.w;
+        float v[K * K];
+#pragma unroll
+        for (int t = 0; t < K * K; ++t) v[t] = src[off[t]];
+        float maxval = -3.402823466e+38f;
+        int best = 0;
+#pragma unroll
+        for (int t = 0; t < K * K; ++t)
+            if (live[t] && v[t] > maxval) { maxval = v[t]; best = t; }
+        y[(long)plane * g.howo + pix] = maxval;
+        idx_max[(long)plane * g.howo + pix] = best;
+    }
+}
+
+// The NHWC twin: lanes along the channels.
+template <int K>
+__global__ void __launch_bounds__(kThreads) max_pool_fwd_square_nhwc_kernel(const float* __restrict__ x,
+                                                                           float* __restrict__ y,
+                                                                           int32_t* __restrict__ idx_max, ConvGeom g,
+                                                                           int c_exact)
+{
+    const uint32_t per_image = (uint32_t)(g.howo * g.c);
+    const uint32_t e = blockIdx.x * kThreads + threadIdx.x;
+    if (e >= per_image) return;
+    const uint32_t pix = fd_div_checked(e, g.fd_c, c_exact);
+    const uint32_t cc = e - pix * g.c;
+    const int oy = (int)fd_div(pix, g.fd_wo);
+    const int ox = (int)pix - oy * g.wo;
+    const int y0 = g.vstride * oy - g.vpadding, x0 = g.hstride * ox - g.hpadding;
+    size_t off[K * K];
+    bool live[K * K];
+#pragma unroll
+    for (int ii = 0; ii < K; ++ii)
+#pragma unroll
+        for (int jj = 0; jj < K; ++jj) {
+            const bool ok = (unsigned)(y0 + ii) < (unsigned)g.h && (unsigned)(x0 + jj) < (unsigned)g.w;
+            live[ii * K + jj] = ok;
+            off[ii * K + jj] = (ok ? (size_t)((y0 + ii) * g.w + x0 + jj) * g.c : 0) + cc;
+        }
+    for (uint32_t nn = blockIdx.y; nn < (uint32_t)g.n; nn += gridDim.y) {
+        const float* src = x + (size_t)nn * g.h * g.w * g.c;
+        float v[K * K];
+#pragma unroll
+        for (int t = 0; t < K * K; ++t) v[t] = src[off[t]];
+        float maxval = -3.402823466e+38f;
+        int best = 0;
+#pragma unroll
+        for (int t = 0; t < K * K; ++t)
+            if (live[t] && v[t] > maxval) { maxval = v[t]; best = t; }
+        y[(size_t)nn * per_image + e] = maxval;
+        idx_max[(size_t)nn * per_image + e] = best;
+    }
+}
+
 // Forward for 2x2 windows that tile the plane exactly (stride 2, no padding or dilation, h == 2*ho, w == 2*wo,
 // 8-byte aligned x): a thread reads its window as two 64-bit loads and tests the four values in the reference's
 // order (first maximum wins).
@@ -1370,6 +1449,11 @@ int launch_max_pool_fwd_nchw(const float* x, float* y, int32_t* idx_max, const C
         HIP_RETURN_IF_LAUNCH_FAILED();
         return PYDTNN_HIP_OK;
     }
+    if (g.kh == 3 && g.kw == 3 && g.vdilation == 1 && g.hdilation == 1) {
+        hipLaunchKernelGGL(max_pool_fwd_square_nchw_kernel<3>, grid, dim3(kThreads), 0, stream, x, y, idx_max, g);
+        HIP_RETURN_IF_LAUNCH_FAILED();
+        return PYDTNN_HIP_OK;
+    }
     hipLaunchKernelGGL(max_pool_fwd_nchw_kernel, grid, dim3(kThreads), 0, stream, x, y, idx_max, g);
     HIP_RETURN_IF_LAUNCH_FAILED();
     return PYDTNN_HIP_OK;
@@ -1424,6 +1508,12 @@ int launch_max_pool_fwd_nhwc(const float* x, float* y, int32_t* idx_max, const C
     }
     const int c_exact = (unsigned long)(per_image + kThreads) * (unsigned long)g.c < (1ul << 32);
     dim3 grid(blocks_for(per_image), (unsigned)(g.n < 65535 ? g.n : 65535));
+    if (g.kh == 3 && g.kw == 3 && g.vdilation == 1 && g.hdilation == 1) {
+        hipLaunchKernelGGL(max_pool_fwd_square_nhwc_kernel<3>, grid, dim3(kThreads), 0, stream, x, y, idx_max, g,
+                           c_exact);
+        HIP_RETURN_IF_LAUNCH_FAILED();
+        return PYDTNN_HIP_OK;
+    }
     hipLaunchKernelGGL(max_pool_fwd_nhwc_kernel, grid, dim3(kThreads), 0, stream, x, y, idx_max, g, c_exact);
     HIP_RETURN_IF_LAUNCH_FAILED();
     return PYDTNN_HIP_OK;
