@@ -1183,57 +1183,65 @@ __device__ __forceinline__ void store_tile_nchw(const EpiNchwT<MASKS>& ep, const
         col_off1[j] = ok ? e : kOob;
     }
     const int lane_m0 = m0 + wm0 + 4 * frag_k;  // this lane's first row
-    [[maybe_unused]] float gate[T::TM][16][T::TN];
-    if constexpr (MASKS == kGate) {
-        const rsrc_t gate_rsrc = make_rsrc_bytes(ep.masks.gate, total);
-#pragma unroll
-        for (int i = 0; i < T::TM; ++i)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int r = i * 32 + 8 * (v / 4) + (v % 4);
-                const bool row_ok = lane_m0 + r < ep.m_extent;
-                const uint32_t soff = (uint32_t)(m0 + wm0 + r) * (uint32_t)ep.howo;
-#pragma unroll
-                for (int j = 0; j < T::TN; ++j)
-                    gate[i][v][j] = (float)(int8_t)__builtin_amdgcn_raw_buffer_load_b8(
-                        gate_rsrc, (int)(row_ok ? col_off1[j] : kOob), (int)soff, 0);
-            }
-    }
+    // The gate bytes are requested in batches of up to 64 per lane (all of a 2x2-block tile at once; row blocks
+    // of a larger tile one after the other), each batch before the stores it belongs to.
+    constexpr int kRowBlocksPerBatch = 16 * T::TN * T::TM <= 64 ? T::TM : 1;
+    [[maybe_unused]] float gate[kRowBlocksPerBatch][16][T::TN];
+    [[maybe_unused]] rsrc_t gate_rsrc;
+    if constexpr (MASKS == kGate) gate_rsrc = make_rsrc_bytes(ep.masks.gate, total);
     [[maybe_unused]] rsrc_t mask_rsrc;
     if constexpr (MASKS == kReluMask) mask_rsrc = make_rsrc_bytes(ep.masks.relu_mask, total);
 #pragma unroll
-    for (int i = 0; i < T::TM; ++i)
+    for (int i0 = 0; i0 < T::TM; i0 += kRowBlocksPerBatch) {
+        if constexpr (MASKS == kGate) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int r = i * 32 + 8 * (v / 4) + (v % 4);
-            const bool row_ok = lane_m0 + r < ep.m_extent;
-            const uint32_t soff = (uint32_t)(m0 + wm0 + r) * (uint32_t)ep.howo;
-            const int row = wm0 + 4 * frag_k + r;  // within the tile
-            float bias = 0.0f, mean = 0.0f, inv_std = 0.0f, gamma = 0.0f, beta = 0.0f;
-            if (has_bias) bias = lds[row];
-            if (has_bn) {
-                mean = lds[T::BM + row];
-                inv_std = lds[2 * T::BM + row];
-                gamma = lds[3 * T::BM + row];
-                beta = lds[4 * T::BM + row];
-            }
+            for (int ib = 0; ib < kRowBlocksPerBatch; ++ib)
 #pragma unroll
-            for (int j = 0; j < T::TN; ++j) {
-                float val = acc[i][j][v];
-                if (has_bias) val += bias;
-                if (has_bn) {
-                    const float t = (val - mean) * inv_std;
-                    val = t * gamma + beta;
+                for (int v = 0; v < 16; ++v) {
+                    const int r = (i0 + ib) * 32 + 8 * (v / 4) + (v % 4);
+                    const bool row_ok = lane_m0 + r < ep.m_extent;
+                    const uint32_t soff = (uint32_t)(m0 + wm0 + r) * (uint32_t)ep.howo;
+#pragma unroll
+                    for (int j = 0; j < T::TN; ++j)
+                        gate[ib][v][j] = (float)(int8_t)__builtin_amdgcn_raw_buffer_load_b8(
+                            gate_rsrc, (int)(row_ok ? col_off1[j] : kOob), (int)soff, 0);
                 }
-                if (ch.relu) val = val > 0.0f ? val : 0.0f;
-                if constexpr (MASKS == kGate) val *= gate[i][v][j];
-                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, val), out_rsrc,
-                                                      (int)(row_ok ? col_off4[j] : kOob), (int)(soff * 4u), 0);
-                if constexpr (MASKS == kReluMask)
-                    __builtin_amdgcn_raw_buffer_store_b8((uint8_t)(val > 0.0f ? 1 : 0), mask_rsrc,
-                                                         (int)(row_ok ? col_off1[j] : kOob), (int)soff, 0);
-            }
         }
+#pragma unroll
+        for (int ib = 0; ib < kRowBlocksPerBatch; ++ib)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int i = i0 + ib;
+                const int r = i * 32 + 8 * (v / 4) + (v % 4);
+                const bool row_ok = lane_m0 + r < ep.m_extent;
+                const uint32_t soff = (uint32_t)(m0 + wm0 + r) * (uint32_t)ep.howo;
+                const int row = wm0 + 4 * frag_k + r;  // within the tile
+                float bias = 0.0f, mean = 0.0f, inv_std = 0.0f, gamma = 0.0f, beta = 0.0f;
+                if (has_bias) bias = lds[row];
+                if (has_bn) {
+                    mean = lds[T::BM + row];
+                    inv_std = lds[2 * T::BM + row];
+                    gamma = lds[3 * T::BM + row];
+                    beta = lds[4 * T::BM + row];
+                }
+#pragma unroll
+                for (int j = 0; j < T::TN; ++j) {
+                    float val = acc[i][j][v];
+                    if (has_bias) val += bias;
+                    if (has_bn) {
+                        const float t = (val - mean) * inv_std;
+                        val = t * gamma + beta;
+                    }
+                    if (ch.relu) val = val > 0.0f ? val : 0.0f;
+                    if constexpr (MASKS == kGate) val *= gate[ib][v][j];
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, val), out_rsrc,
+                                                          (int)(row_ok ? col_off4[j] : kOob), (int)(soff * 4u), 0);
+                    if constexpr (MASKS == kReluMask)
+                        __builtin_amdgcn_raw_buffer_store_b8((uint8_t)(val > 0.0f ? 1 : 0), mask_rsrc,
+                                                             (int)(row_ok ? col_off1[j] : kOob), (int)soff, 0);
+                }
+            }
+    }
     // the staged parameters are read until here; the caller may refill LDS afterwards
     if (has_bias || has_bn) __syncthreads();
 }
