@@ -1,6 +1,7 @@
 """GPU parity at the benchmark's configurations.
 
-cfg1, cfg3 and cfg4 are small enough for the CPU oracle to run whole.  At cfg2's full size the
+cfg1, cfg3 and cfg4 are small enough for the CPU oracle to run whole, at the benchmark's batch of 64 (tile
+and launch choices depend on the problem size).  At cfg2's full size the
 outputs are checked by *sampled direct convolution in float64*: a few thousand randomly chosen
 elements of y, dw and dx are recomputed from their defining sums, which needs no column matrix and
 is independent of the kernels' tiling.  A VGG16 model (batch 8) is checked layer by layer with the
@@ -35,9 +36,9 @@ def test_cfg1_mnist_layer_nhwc(pd, oracle):
 
 def test_cfg3_alexnet_conv1_bias_relu(pd, oracle):
     announce("cfg3")
-    x, w, b = bench_configs.make_cfg3(n=16)
+    x, w, b = bench_configs.make_cfg3(n=64)
     y = pd.ConvGemm().conv_gemm_nchw(dev(w), dev(x), biases_vector=dev(b), vstride=4, hstride=4, relu=True)
-    assert tuple(y.shape) == (16, 96, 55, 55)
+    assert tuple(y.shape) == (64, 96, 55, 55)
     ref, _ = oracle.conv2d_forward_nchw_i2c(x, w, b, oracle.ConvParams(11, 11, 0, 0, 4, 4))
     ref = oracle.fused_epilogue(ref, "NCHW", relu_flag=True)
     assert_close(host(y), ref, what="cfg3 y")
@@ -46,7 +47,7 @@ def test_cfg3_alexnet_conv1_bias_relu(pd, oracle):
 
 def test_cfg4_resnet_bottleneck_fused_nhwc(pd, oracle):
     announce("cfg4")
-    x, ws, bns = bench_configs.make_cfg4(n=8)
+    x, ws, bns = bench_configs.make_cfg4(n=64)
     model = bench_configs.build_cfg4_model(pd, torch, ws, bns, fused=True)
     y = model.evaluate_dataset_batch(dev(x))
     block = model.layers[1]

@@ -634,7 +634,10 @@ def test_large_batches_run_as_image_groups(oracle, fmt, d):
 
 fold_grid = [D(2, 16, 30, 30, 130, 3, 3, 1, 1, 1, 1, 1, 1), D(5, 8, 19, 23, 20, 5, 3, 2, 1, 2, 1, 1, 1),
              D(2, 33, 14, 14, 257, 1, 1, 0, 0, 1, 1, 1, 1), D(3, 1, 28, 28, 32, 3, 3, 1, 1, 1, 1, 1, 1),
-             D(16, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1, 1, 1)]  # the last one takes the balanced launch and its fixup
+             D(16, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1, 1, 1),   # takes the balanced launch and its fixup
+             # tiles whose gated / masked store runs in several batches of rows: 512 tiles of 256x128 with a long
+             # reduction, and the 96-row tile of filter counts that are multiples of 96
+             D(64, 256, 32, 32, 256, 3, 3, 1, 1, 1, 1, 1, 1), D(8, 16, 35, 35, 96, 3, 3, 1, 1, 1, 1, 1, 1)]
 
 
 @pytest.mark.parametrize("d", fold_grid, ids=repr)
