@@ -74,12 +74,27 @@ int pydtnn_hip_row2im_nhwc(const float *rows, float *dx, int b, int h, int w, in
  *                                op(B) = B (k x n, ldb) or B^T (B stored n x k, ldb) when transb != 0.
  * Optional fused epilogue on C: + bias[n] (FC forward, pydtnn/backends/cpu/layers/fc_cpu.py:63), then ReLU.
  * Small m*n with long k is split along k; then `workspace` must hold
- * pydtnn_hip_sgemm_workspace_bytes(m, n, k) bytes (0 means none needed).
+ * pydtnn_hip_sgemm_workspace_bytes(m, n, k) bytes (0 means none needed) and C must be dense
+ * (ldc == n; PYDTNN_HIP_ERR_UNSUPPORTED otherwise, before anything is launched).
  * ---------------------------------------------------------------------------------------- */
 size_t pydtnn_hip_sgemm_workspace_bytes(long m, long n, long k);
 int pydtnn_hip_sgemm(int transa, int transb, long m, long n, long k, const float *a, long lda, const float *b,
                      long ldb, float *c, long ldc, const float *bias, int relu, void *workspace,
                      size_t workspace_bytes, void *stream);
+
+/* pydtnn_hip_sgemm for callers that cannot allocate device memory or hold a workspace of their own (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart
+ * in PyDTNN.  Same arguments, meaning and results (bit for bit) as pydtnn_hip_sgemm minus the workspace:
+ * the partial sums of a split along k go to an array that is part of the library's device image,
+ * pydtnn_hip_sgemm_static_scratch_bytes() = 64 MiB on every GPU the library has run on, held until the
+ * process ends.  A problem whose pydtnn_hip_sgemm_workspace_bytes(m, n, k) exceeds that returns
+ * PYDTNN_HIP_ERR_WORKSPACE and launches nothing.  The call allocates and frees nothing; the first call on a
+ * device asks the runtime for the array's address there (make that call before starting a capture).
+ * All calls on one GPU share the array: calls that may overlap there (different streams, different
+ * threads) race; order them on one stream. */
+size_t pydtnn_hip_sgemm_static_scratch_bytes(void);
+int pydtnn_hip_sgemm_static(int transa, int transb, long m, long n, long k, const float *a, long lda, const float *b,
+                            long ldb, float *c, long ldc, const float *bias, int relu, void *stream);
 
 /* ------------------------------------------------------------------------------------------
  * Implicit-im2col convolution GEMMs: the column matrix is never materialised.

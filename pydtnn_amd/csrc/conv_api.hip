@@ -1,6 +1,7 @@
 // Device-pointer C ABI: argument checks, batching over image groups, and the launches that are not
 // convolutions (GEMM, explicit-path GEMMs, streaming kernels).
 #include "conv_internal.h"
+#include <mutex>
 
 namespace {
 
@@ -139,6 +140,83 @@ int conv_dx_batched(int nhwc, long b, long c, long h, long w, long kn, long kh, 
     return PYDTNN_HIP_OK;
 }
 
+// ---------------------------------------------------------------- GEMM (shared by the two entry points)
+int sgemm_impl(int transa, int transb, long m, long n, long k, const float* a, long lda, const float* b, long ldb,
+               float* c, long ldc, const float* bias, int relu, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (!a || !b || !c || m <= 0 || n <= 0 || k <= 0) return PYDTNN_HIP_ERR_INVALID;
+    const long lim = 1l << 31;
+    if (m >= lim || n >= lim || k >= lim) return PYDTNN_HIP_ERR_UNSUPPORTED;
+    if (lda < (transa ? m : k) || ldb < (transb ? k : n) || ldc < n) return PYDTNN_HIP_ERR_INVALID;
+    const TileSel sel = pick_tile(m, n);
+    const SplitPlan sp = plan_plain_split(tiles_of(sel, m, n), k, m * n);
+    const ChanEpilogue chan = make_chan(bias, nullptr, nullptr, nullptr, nullptr, relu);
+    float* dst = c;
+    long dst_ld = ldc;
+    ChanEpilogue gemm_chan = chan;
+    if (sp.splits > 1) {
+        if (ldc != n) return PYDTNN_HIP_ERR_UNSUPPORTED;  // the sum over the split writes a dense C
+        if (!workspace || workspace_bytes < (size_t)sp.splits * m * n * 4) return PYDTNN_HIP_ERR_WORKSPACE;
+        dst = (float*)workspace;
+        dst_ld = n;
+        gemm_chan = no_epilogue();
+    }
+    const hipStream_t st = as_stream(stream);
+    int rc = PYDTNN_HIP_OK;
+    // floats reachable from each base pointer (last row may be shorter than its leading dimension)
+    const long a_total = transa ? (k - 1) * lda + m : (m - 1) * lda + k;
+    const long b_total = transb ? (n - 1) * ldb + k : (k - 1) * ldb + n;
+    WITH_TILE(sel, {
+        const EpiPlain ep = epi_plain(dst, dst_ld, m * n, m, n, gemm_chan, no_masks(), sp.splits);
+        if ((!transa && !span_ok_k(T::BM, lda, 0, 0)) || (transa && !span_ok_mn(lda)) ||
+            (transb && !span_ok_k(T::BN, ldb, 0, 0)) || (!transb && !span_ok_mn(ldb)))
+            return PYDTNN_HIP_ERR_UNSUPPORTED;
+        if (!transa && !transb)
+            rc = launch<T>(plain_k<T::BM, false>(a, a_total, lda, 0, m, 0), plain_mn<T::BN>(b, b_total, ldb, 0, n), ep,
+                           m, n, sp.si, sp.splits, st);
+        else if (!transa && transb)
+            rc = launch<T>(plain_k<T::BM, false>(a, a_total, lda, 0, m, 0),
+                           plain_k<T::BN, false>(b, b_total, ldb, 0, n, 0), ep, m, n, sp.si, sp.splits, st);
+        else if (transa && !transb)
+            rc = launch<T>(plain_mn<T::BM>(a, a_total, lda, 0, m), plain_mn<T::BN>(b, b_total, ldb, 0, n), ep, m, n,
+                           sp.si, sp.splits, st);
+        else
+            rc = launch<T>(plain_mn<T::BM>(a, a_total, lda, 0, m), plain_k<T::BN, false>(b, b_total, ldb, 0, n, 0), ep,
+                           m, n, sp.si, sp.splits, st);
+    })
+    if (rc != PYDTNN_HIP_OK || sp.splits == 1) return rc;
+    return launch_splitk_reduce((const float*)workspace, c, m, (int)n, m * n, sp.splits, 0, 0, chan, 0, st);
+}
+
+// ---------------------------------------------------------------- scratch that no call allocates
+// Partial sums of pydtnn_hip_sgemm_static's split along k.  Every GPU the library runs on holds its own
+// copy of this array, at its own address, until the process ends.  In host code the name `scratch` is
+// only a handle for hipGetSymbolAddress: kernels get the address that call returns for the current
+// device.  Nothing in it has to start at zero: a split GEMM writes every partial sum it later reads.
+constexpr size_t kStaticScratchBytes = (size_t)64 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_lock;
+void* g_scratch_address[kMaxDevices] = {};
+
+// Address of `scratch` on the current device, asked once per device (the first call on a device loads
+// the library's code object there, which is the only set-up work).
+int static_scratch_address(void** out)
+{
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) return PYDTNN_HIP_ERR_LAUNCH;
+    if (dev < 0 || dev >= kMaxDevices) return PYDTNN_HIP_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> hold(g_scratch_lock);
+    if (!g_scratch_address[dev]) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return PYDTNN_HIP_ERR_LAUNCH;
+        g_scratch_address[dev] = p;
+    }
+    *out = g_scratch_address[dev];
+    return PYDTNN_HIP_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -218,48 +296,23 @@ int pydtnn_hip_sgemm(int transa, int transb, long m, long n, long k, const float
                      long ldb, float* c, long ldc, const float* bias, int relu, void* workspace,
                      size_t workspace_bytes, void* stream)
 {
-    if (!a || !b || !c || m <= 0 || n <= 0 || k <= 0) return PYDTNN_HIP_ERR_INVALID;
-    const long lim = 1l << 31;
-    if (m >= lim || n >= lim || k >= lim) return PYDTNN_HIP_ERR_UNSUPPORTED;
-    if (lda < (transa ? m : k) || ldb < (transb ? k : n) || ldc < n) return PYDTNN_HIP_ERR_INVALID;
-    const TileSel sel = pick_tile(m, n);
-    const SplitPlan sp = plan_plain_split(tiles_of(sel, m, n), k, m * n);
-    const ChanEpilogue chan = make_chan(bias, nullptr, nullptr, nullptr, nullptr, relu);
-    float* dst = c;
-    long dst_ld = ldc;
-    ChanEpilogue gemm_chan = chan;
-    if (sp.splits > 1) {
-        if (!workspace || workspace_bytes < (size_t)sp.splits * m * n * 4) return PYDTNN_HIP_ERR_WORKSPACE;
-        dst = (float*)workspace;
-        dst_ld = n;
-        gemm_chan = no_epilogue();
+    return sgemm_impl(transa, transb, m, n, k, a, lda, b, ldb, c, ldc, bias, relu, workspace, workspace_bytes, stream);
+}
+
+size_t pydtnn_hip_sgemm_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+int pydtnn_hip_sgemm_static(int transa, int transb, long m, long n, long k, const float* a, long lda, const float* b,
+                            long ldb, float* c, long ldc, const float* bias, int relu, void* stream)
+{
+    const size_t need = pydtnn_hip_sgemm_workspace_bytes(m, n, k);
+    if (need > kStaticScratchBytes) return PYDTNN_HIP_ERR_WORKSPACE;
+    void* ws = nullptr;
+    if (need > 0) {
+        const int rc = static_scratch_address(&ws);
+        if (rc != PYDTNN_HIP_OK) return rc;
     }
-    const hipStream_t st = as_stream(stream);
-    int rc = PYDTNN_HIP_OK;
-    // floats reachable from each base pointer (last row may be shorter than its leading dimension)
-    const long a_total = transa ? (k - 1) * lda + m : (m - 1) * lda + k;
-    const long b_total = transb ? (n - 1) * ldb + k : (k - 1) * ldb + n;
-    WITH_TILE(sel, {
-        const EpiPlain ep = epi_plain(dst, dst_ld, m * n, m, n, gemm_chan, no_masks(), sp.splits);
-        if ((!transa && !span_ok_k(T::BM, lda, 0, 0)) || (transa && !span_ok_mn(lda)) ||
-            (transb && !span_ok_k(T::BN, ldb, 0, 0)) || (!transb && !span_ok_mn(ldb)))
-            return PYDTNN_HIP_ERR_UNSUPPORTED;
-        if (!transa && !transb)
-            rc = launch<T>(plain_k<T::BM, false>(a, a_total, lda, 0, m, 0), plain_mn<T::BN>(b, b_total, ldb, 0, n), ep,
-                           m, n, sp.si, sp.splits, st);
-        else if (!transa && transb)
-            rc = launch<T>(plain_k<T::BM, false>(a, a_total, lda, 0, m, 0),
-                           plain_k<T::BN, false>(b, b_total, ldb, 0, n, 0), ep, m, n, sp.si, sp.splits, st);
-        else if (transa && !transb)
-            rc = launch<T>(plain_mn<T::BM>(a, a_total, lda, 0, m), plain_mn<T::BN>(b, b_total, ldb, 0, n), ep, m, n,
-                           sp.si, sp.splits, st);
-        else
-            rc = launch<T>(plain_mn<T::BM>(a, a_total, lda, 0, m), plain_k<T::BN, false>(b, b_total, ldb, 0, n, 0), ep,
-                           m, n, sp.si, sp.splits, st);
-    })
-    if (rc != PYDTNN_HIP_OK || sp.splits == 1) return rc;
-    if (ldc != n) return PYDTNN_HIP_ERR_UNSUPPORTED;  // the split reduction writes a dense C
-    return launch_splitk_reduce((const float*)workspace, c, m, (int)n, m * n, sp.splits, 0, 0, chan, 0, st);
+    return sgemm_impl(transa, transb, m, n, k, a, lda, b, ldb, c, ldc, bias, relu, ws, need ? kStaticScratchBytes : 0,
+                      stream);
 }
 
 // ---------------------------------------------------------------- convolution

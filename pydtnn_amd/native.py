@@ -33,6 +33,9 @@ SIGNATURES = {
     "pydtnn_hip_sgemm_workspace_bytes": (_c.c_size_t, [_c.c_long] * 3),
     "pydtnn_hip_sgemm": (_c.c_int, [_c.c_int, _c.c_int, _c.c_long, _c.c_long, _c.c_long, _f32p, _c.c_long, _f32p,
                                     _c.c_long, _f32p, _c.c_long, _f32p, _c.c_int, _vp, _c.c_size_t, _vp]),
+    "pydtnn_hip_sgemm_static_scratch_bytes": (_c.c_size_t, []),
+    "pydtnn_hip_sgemm_static": (_c.c_int, [_c.c_int, _c.c_int, _c.c_long, _c.c_long, _c.c_long, _f32p, _c.c_long, _f32p,
+                                           _c.c_long, _f32p, _c.c_long, _f32p, _c.c_int, _vp]),
     "pydtnn_hip_conv_workspace_bytes": (_c.c_size_t, [_c.c_int, _c.c_int] + _geom13_i),
     "pydtnn_hip_sconvGemmNCHW": (_c.c_int, [_c.c_char] + _geom13_u + [_f32p] * 8 + [_c.c_bool, _vp, _c.c_size_t, _vp]),
     "pydtnn_hip_sconvGemmNHWC": (_c.c_int, [_c.c_char] + _geom13_u + [_f32p] * 8 + [_c.c_bool, _vp, _c.c_size_t, _vp]),
