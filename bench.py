@@ -29,6 +29,8 @@ HBM_PEAK_GBS = 8000.0
 # scaled by what the same counter reads for a 256 MiB copy (factors 2.000 and 1.000):
 # main launch (166125.0 * 2.0 + 262144.0) KiB plus the fixup launch of its cut tiles (32822.9 * 2.0 + 4096.0) KiB.
 # The summary of those runs is profiles/cfg2_conv3x3_pmc_counters.md.
+TRAFFIC_SOURCE = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in profiles/cfg2_conv3x3_pmc_counters.md "
+                  "(a constant read off that profile, not measured by this run)")
 MEASURED_TRAFFIC_BYTES = {"cfg2": int((166125.0 * 2.0 + 262144.0 + 32822.9 * 2.0 + 4096.0) * 1024)}
 
 
@@ -40,6 +42,8 @@ def parse_args():
     ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-vgg16", action="store_true", help="skip the VGG16 training-step extra of the default run")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip cfg1, cfg3 and cfg4 (GPU and CPU legs) in the default run's extra")
     ap.add_argument("--no-folding-extra", action="store_true",
                     help="skip the extra VGG16 runs (enable_relu_folding=True; NHWC) that are reported beside the headline one")
     ap.add_argument("--conv-layers", action="store_true",
@@ -151,6 +155,7 @@ def run_cfg2(torch, pd, args):
     }
     # explicit-path streams: bytes(x) + bytes(cols) and bytes(cols) + bytes(dx).  The C ABI is called on buffers
     # allocated once, so that no allocation falls between a pair of timing events.
+    from pydtnn_amd import native
     from pydtnn_amd.native import check, f32, lib, stream_ptr
     geom = (3, 3, 1, 1, 1, 1, 1, 1)
     mat = torch.empty(256 * 9 * n * 56 * 56, device="cuda")   # x_cols (K x P) or x_rows (P x K)
@@ -177,6 +182,32 @@ def run_cfg2(torch, pd, args):
         extra[second + "_gbs"] = round(stream_bytes / (t2.median_ms() * 1e-3) / 1e9, 1)
     extra["im2col_pct_hbm_peak"] = round(100 * extra["im2col_gbs"] / HBM_PEAK_GBS, 1)
     extra["col2im_pct_hbm_peak"] = round(100 * extra["col2im_gbs"] / HBM_PEAK_GBS, 1)
+    # the explicit route on the same layer (Conv2D with enable_conv_gemm=False): the three GEMMs over the
+    # materialised column matrix, (co,K)@(K,P) forward, (co,P)@(P,K) for dw and (K,co)@(co,P) + col2im for dx,
+    # each 236.76 GFLOP, with the buffers of the gather timings above
+    kxp = torch.empty(256 * 9 * n * 56 * 56, device="cuda")   # the (K x P) product of the explicit dx
+    g13 = (n, 256, 56, 56, 256, 3, 3, 1, 1, 1, 1, 1, 1)
+    calls["im2col"]()
+    y_i2c, dw_i2c = torch.empty_like(xd), torch.empty_like(conv.weights)
+    dw_ws, dw_ws_bytes = native.conv_workspace(native.OP_DW, False, g13)
+    i2c = {
+        "i2c_fwd": lambda: check(lib().pydtnn_hip_conv_i2c_forward(0, *g13, f32(conv.weights), f32(mat), f32(y_i2c),
+                                                                   f32(conv.biases), stream_ptr()), "i2c forward"),
+        "i2c_dw": lambda: check(lib().pydtnn_hip_conv_i2c_dw(0, *g13, f32(dyd), f32(mat), f32(dw_i2c), dw_ws,
+                                                             dw_ws_bytes, stream_ptr()), "i2c dw"),
+        "i2c_dx": lambda: check(lib().pydtnn_hip_conv_i2c_dx(0, *g13, f32(conv.weights), f32(dyd), f32(back), f32(kxp),
+                                                             kxp.numel() * 4, stream_ptr()), "i2c dx"),
+    }
+    for name, fn in i2c.items():
+        t = Timer(torch)
+        for i in range(5):
+            fn() if i == 0 else t(fn)
+        torch.cuda.synchronize()
+        extra[name + "_ms"] = round(t.median_ms(), 4)
+        extra[name + "_tflops"] = round(gemm_flop / (t.median_ms() * 1e-3) / 1e12, 2)
+    extra["i2c_note"] = ("explicit route at cfg2: GEMMs over the materialised (K x P) matrix; i2c_fwd excludes the "
+                         "im2col pass (im2col_gbs), i2c_dx includes the col2im pass")
+    del kxp, y_i2c
     # the bias -> BN(inference) -> ReLU epilogue as a stand-alone pass over y (2 * bytes(y)); fused into the
     # GEMM's store it costs no traffic at all
     ch = [torch.rand(256, device="cuda") + 0.5 for _ in range(5)]
@@ -191,7 +222,8 @@ def run_cfg2(torch, pd, args):
     del mat, back
     roofline = {"bound": "mfma", "kernel": "gemm_streamk_kernel_big_tile<256x128, PlainK4, Im2colNchwMN, EpiNchw> + streamk_fixup_kernel (forward)",
                 "achieved": round(achieved, 3), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES["cfg2"]}
+                "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES["cfg2"],
+                "traffic_source": TRAFFIC_SOURCE}
     workload = ("cfg2: VGG16-style 3x3 conv layer fwd+dW+db+dX, fp32 NCHW, N=64, 256->256, 56x56, stride 1, pad 1, "
                 "implicit GEMM")
     return ms, step_flop / (ms * 1e-3) / 1e9, workload, roofline, extra
@@ -203,7 +235,8 @@ def cpu_baseline_cfg2(sample_images=64, reps=30):
     import numpy as np
     from threadpoolctl import threadpool_limits
     from oracle import cpu_ref
-    cores = int(os.environ.get("OMP_NUM_THREADS", min(16, os.cpu_count() or 1)))
+    from bench_configs import _cpu_cores, host_cpus
+    cores = _cpu_cores()
     x, w, b, dy = make_cfg2(sample_images)
     p = cpu_ref.ConvParams(3, 3, 1, 1)
     times = []
@@ -220,7 +253,8 @@ def cpu_baseline_cfg2(sample_images=64, reps=30):
                 break
     best = min(times)
     flop = 3 * 2.0 * 256 * 2304 * sample_images * 56 * 56
-    return {"value": round(flop / best / 1e9, 1), "unit": "GFLOP/s", "cores": cores, "kind": "port",
+    return {"value": round(flop / best / 1e9, 1), "unit": "GFLOP/s", "cores": cores, "host_logical_cpus": host_cpus(),
+            "kind": "port",
             "sample": f"{sample_images} of 64 images of cfg2, fwd+dW+db+dX, 1 warm-up then best of {len(times)} "
                       f"({best:.2f} s each, {sum(times):.1f} s in all); C/OpenMP im2col+col2im and NumPy(OpenBLAS) "
                       f"matmul limited to {cores} threads"}
@@ -352,6 +386,9 @@ def main():
         if not args.no_vgg16:
             _, vgg = run_cfg5(torch, pd, args, steps=3, warmup=1)
             extra.update(vgg)
+        if not args.no_other_configs:
+            from bench_configs import other_configs_extra
+            extra.update(other_configs_extra(torch, pd, timed_steps, cpu=not args.no_cpu_baseline))
     elif args.workload == "cfg5":
         ms, extra = run_cfg5(torch, pd, args)
         if args.conv_layers:

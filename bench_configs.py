@@ -71,8 +71,19 @@ def build_cfg4_model(pd, torch, ws, bns, fused=True):
 # as restated by the oracle, timed on this host.  Reported beside the GPU figure, never a target.
 
 def _cpu_cores():
+    """Threads of the CPU legs: the process's share of the host (OMP_NUM_THREADS where the launcher sets it,
+    otherwise every CPU the process may run on)."""
     import os
-    return int(os.environ.get("OMP_NUM_THREADS", min(16, os.cpu_count() or 1)))
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = os.cpu_count() or 1
+    return int(os.environ.get("OMP_NUM_THREADS", usable))
+
+
+def host_cpus():
+    import os
+    return os.cpu_count() or 1
 
 
 def _time_cpu(fn, budget_s, max_reps):
@@ -91,17 +102,18 @@ def _time_cpu(fn, budget_s, max_reps):
 
 
 def _cpu_report(value, unit, what, best, reps, total):
-    return {"value": round(value, 1), "unit": unit, "cores": _cpu_cores(), "kind": "port",
+    return {"value": round(value, 1), "unit": unit, "cores": _cpu_cores(), "host_logical_cpus": host_cpus(),
+            "kind": "port",
             "sample": f"{what}, 1 warm-up then best of {reps} ({best:.3g} s each, {total:.1f} s in all); C/OpenMP "
                       f"gathers and NumPy(OpenBLAS) matmul limited to {_cpu_cores()} threads"}
 
 
-def cpu_baseline_other(workload):
+def cpu_baseline_other(workload, budget_s=12.0):
     from oracle import cpu_ref
     if workload == "cfg1":
         x, w, b = make_cfg1()
         p = cpu_ref.ConvParams(3, 3, 1, 1)
-        best, reps, total = _time_cpu(lambda: cpu_ref.conv2d_forward_nhwc_i2c(x, w, b, p), 10.0, 2000)
+        best, reps, total = _time_cpu(lambda: cpu_ref.conv2d_forward_nhwc_i2c(x, w, b, p), min(budget_s, 10.0), 2000)
         return _cpu_report(2.0 * 32 * 9 * 64 * 28 * 28 / best / 1e9, "GFLOP/s", "all 64 images of cfg1, forward", best,
                            reps, total)
     if workload == "cfg3":
@@ -112,7 +124,7 @@ def cpu_baseline_other(workload):
             y, _ = cpu_ref.conv2d_forward_nchw_i2c(x, w, b, p)
             cpu_ref.relu(y)
 
-        best, reps, total = _time_cpu(fwd, 12.0, 100)
+        best, reps, total = _time_cpu(fwd, budget_s, 100)
         return _cpu_report(2.0 * 96 * 363 * 64 * 55 * 55 / best / 1e9, "GFLOP/s",
                            "all 64 images of cfg3, forward + bias + ReLU as separate passes", best, reps, total)
     if workload == "cfg4":
@@ -129,7 +141,7 @@ def cpu_baseline_other(workload):
             cur = cpu_ref.eltw_sum(cur, x)
             cpu_ref.relu(cur)
 
-        best, reps, total = _time_cpu(block, 12.0, 100)
+        best, reps, total = _time_cpu(block, budget_s, 100)
         flop = 2.0 * 64 * 56 * 56 * (256 * 64 + 576 * 64 + 64 * 256)
         return _cpu_report(flop / best / 1e9, "GFLOP/s",
                            "all 64 images of cfg4, unfused layers (conv, BN, ReLU, add as separate passes)", best, reps,
@@ -217,43 +229,53 @@ def cpu_baseline_vgg16(sample_images=16, budget_s=14.0):
                        best, reps, total)
 
 
-def run_other(torch, pd, args, Timer, timed_steps):
+def run_cfg1(torch, pd, timed_steps, steps, warmup):
     from pydtnn_amd.conv_gemm import ConvGemm
     cg = ConvGemm()
-    if args.workload == "cfg1":
-        x, w, b = make_cfg1()
-        xd, wd, bd = (torch.from_numpy(a).cuda() for a in (x, w, b))
+    x, w, b = make_cfg1()
+    xd, wd, bd = (torch.from_numpy(a).cuda() for a in (x, w, b))
 
-        def step(timers):
-            cg.conv_gemm_nhwc(wd, xd, biases_vector=bd, vpadding=1, hpadding=1)
+    def step(timers):
+        cg.conv_gemm_nhwc(wd, xd, biases_vector=bd, vpadding=1, hpadding=1)
 
-        ms, _ = timed_steps(torch, step, args.steps, args.warmup)
-        flop = 2.0 * 32 * 9 * 64 * 28 * 28
-        nbytes = x.nbytes + w.nbytes + 64 * 28 * 28 * 32 * 4
-        gbs = nbytes / (ms * 1e-3) / 1e9
-        roofline = {"bound": "hbm", "kernel": "gemm_kernel<64x64, Im2rowNhwcK, FilterNhwcMN, EpiPlain>",
-                    "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
-                    "traffic": None}
-        workload = "cfg1: Conv2D forward, fp32 NHWC, N=64, 28x28x1 -> 32, 3x3, stride 1, pad 1 (launch-latency bound)"
-        return ms, flop / (ms * 1e-3) / 1e9, "GFLOP/s", workload, roofline, {"bytes": nbytes, "gbs": round(gbs, 1)}
+    ms, _ = timed_steps(torch, step, steps, warmup)
+    flop = 2.0 * 32 * 9 * 64 * 28 * 28
+    nbytes = x.nbytes + w.nbytes + 64 * 28 * 28 * 32 * 4
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "kernel": "gemm_kernel<64x64, Im2colNchwMN<NHWC>, PlainMN, EpiPlain>",
+                "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                "traffic": None}
+    workload = "cfg1: Conv2D forward, fp32 NHWC, N=64, 28x28x1 -> 32, 3x3, stride 1, pad 1 (launch-latency bound)"
+    return ms, flop / (ms * 1e-3) / 1e9, "GFLOP/s", workload, roofline, {"bytes": nbytes, "gbs": round(gbs, 1)}
 
-    if args.workload == "cfg3":
-        x, w, b = make_cfg3()
-        xd, wd, bd = (torch.from_numpy(a).cuda() for a in (x, w, b))
 
-        def step(timers):
-            cg.conv_gemm_nchw(wd, xd, biases_vector=bd, vstride=4, hstride=4, relu=True)
+def run_cfg3(torch, pd, timed_steps, steps, warmup):
+    from pydtnn_amd.conv_gemm import ConvGemm
+    cg = ConvGemm()
+    x, w, b = make_cfg3()
+    xd, wd, bd = (torch.from_numpy(a).cuda() for a in (x, w, b))
 
-        ms, _ = timed_steps(torch, step, args.steps, args.warmup)
-        flop = 2.0 * 96 * 363 * 64 * 55 * 55
-        tf = flop / (ms * 1e-3) / 1e12
-        roofline = {"bound": "mfma", "kernel": "gemm_kernel<128x128, PlainK, Im2colNchwMN, EpiNchw>",
-                    "achieved": round(tf, 3), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                    "frac": round(tf / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": None}
-        workload = ("cfg3: AlexNet conv1 forward + fused bias + ReLU, fp32 NCHW, N=64, 3x227x227 -> 96, 11x11, "
-                    "stride 4, pad 0 (M=96 fills 75 % of a 128-row tile, K=363)")
-        return ms, flop / (ms * 1e-3) / 1e9, "GFLOP/s", workload, roofline, {}
+    def step(timers):
+        cg.conv_gemm_nchw(wd, xd, biases_vector=bd, vstride=4, hstride=4, relu=True)
 
+    ms, _ = timed_steps(torch, step, steps, warmup)
+    flop = 2.0 * 96 * 363 * 64 * 55 * 55
+    tf = flop / (ms * 1e-3) / 1e12
+    roofline = {"bound": "mfma", "kernel": "implicit GEMM on 96-row tiles, Im2colNchwMN, EpiNchw (bias + ReLU)",
+                "achieved": round(tf, 3), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(tf / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": None}
+    workload = ("cfg3: AlexNet conv1 forward + fused bias + ReLU, fp32 NCHW, N=64, 3x227x227 -> 96, 11x11, "
+                "stride 4, pad 0 (K=363)")
+    return ms, flop / (ms * 1e-3) / 1e9, "GFLOP/s", workload, roofline, {}
+
+
+CFG4_FLOP = 2.0 * 64 * 56 * 56 * (256 * 64 + 576 * 64 + 64 * 256)
+# what the fused block cannot avoid moving: x read by the first convolution and again as the residual, the two
+# 64-channel intermediates written and read, the output written
+CFG4_MIN_BYTES = 4.0 * 64 * 56 * 56 * (256 + 64 + 64 + 64 + 64 + 256 + 256)
+
+
+def run_cfg4(torch, pd, timed_steps, steps, warmup):
     x, ws, bns = make_cfg4()
     model = build_cfg4_model(pd, torch, ws, bns, fused=True)
     plain = build_cfg4_model(pd, torch, ws, bns, fused=False)
@@ -263,21 +285,40 @@ def run_other(torch, pd, args, Timer, timed_steps):
     def step(timers):
         model.evaluate_batch(xd)
 
-    ms, _ = timed_steps(torch, step, args.steps, args.warmup)
+    ms, _ = timed_steps(torch, step, steps, warmup)
 
     def step_plain(timers):
         plain.evaluate_batch(xd)
 
-    ms_plain, _ = timed_steps(torch, step_plain, args.steps, args.warmup)
-    flop = 2.0 * 64 * 56 * 56 * (256 * 64 + 576 * 64 + 64 * 256)
-    tf = flop / (ms * 1e-3) / 1e12
-    nbytes = 4.0 * 64 * 56 * 56 * (256 + 64 + 64 + 64 + 64 + 256 + 256 + 256 + 256 + 256)
-    roofline = {"bound": "mfma", "kernel": "3 fused conv+BN(+ReLU) implicit GEMMs + residual add + ReLU",
+    ms_plain, _ = timed_steps(torch, step_plain, steps, warmup)
+    tf = CFG4_FLOP / (ms * 1e-3) / 1e12
+    roofline = {"bound": "mfma", "kernel": "the block's fused conv+BN(+ReLU)(+residual) implicit GEMMs",
                 "achieved": round(tf, 3), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(tf / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": None}
     extra = {"unfused_ms": round(ms_plain, 4), "fused_ms": round(ms, 4),
-             "block_gbs_vs_8TBs": round(nbytes / (ms * 1e-3) / 1e9, 1),
+             "block_gbs_vs_8TBs": round(CFG4_MIN_BYTES / (ms * 1e-3) / 1e9, 1),
              "layers": [l.canonical_name for l in model.get_all_layers()]}
     workload = ("cfg4: ResNet-50 bottleneck inference, fp32 NHWC, N=64, 56x56x256: fused Conv+BN+ReLU 1x1 256->64, "
                 "3x3 64->64, Conv+BN 1x1 64->256, residual add, ReLU")
-    return ms, flop / (ms * 1e-3) / 1e9, "GFLOP/s", workload, roofline, extra
+    return ms, CFG4_FLOP / (ms * 1e-3) / 1e9, "GFLOP/s", workload, roofline, extra
+
+
+def run_other(torch, pd, args, Timer, timed_steps):
+    fn = {"cfg1": run_cfg1, "cfg3": run_cfg3, "cfg4": run_cfg4}[args.workload]
+    return fn(torch, pd, timed_steps, args.steps, args.warmup)
+
+
+def other_configs_extra(torch, pd, timed_steps, cpu=True, steps=20, warmup=3):
+    """cfg1, cfg3 and cfg4 for the default run's `extra`: GPU time and rate of each beside its CPU route."""
+    out = {}
+    for name, fn, budget in (("cfg1", run_cfg1, 2.0), ("cfg3", run_cfg3, 5.0), ("cfg4", run_cfg4, 5.0)):
+        ms, value, unit, _, roofline, extra = fn(torch, pd, timed_steps, steps, warmup)
+        out[f"{name}_ms"] = round(ms, 4)
+        out[f"{name}_gflops"] = round(value, 1)
+        out[f"{name}_roofline"] = {k: roofline[k] for k in ("bound", "achieved", "peak", "unit", "frac")}
+        if name == "cfg4":
+            out["cfg4_unfused_ms"] = extra["unfused_ms"]
+            out["cfg4_gbs_of_min_traffic"] = extra["block_gbs_vs_8TBs"]
+        if cpu:
+            out[f"{name}_cpu_baseline"] = cpu_baseline_other(name, budget)
+    return out

@@ -243,6 +243,23 @@ int pydtnn_hip_max_pool_2d_bwd_gated(int nhwc, const float *dy, const int32_t *i
                                      int b, int c, int h, int w, int kh, int kw, int vpadding, int hpadding,
                                      int vstride, int hstride, int vdilation, int hdilation, void *stream);
 
+/* The sum of an addition block done by the store of the convolution that ends one of its two paths
+ * (inference).  The forward of pydtnn_hip_sconvGemmNCHW / NHWC (nhwc = 0 / 1; b, c, h, w name the input's
+ * batch, channels, height, width in either format) followed by
+ *     y = y + residual                      eltw_sum_cython (pydtnn/cython_modules/eltw_sum_cython.pyx:25-36) as
+ *                                           AdditionBlockCPU.forward applies it
+ *                                           (pydtnn/backends/cpu/layers/addition_block_cpu.py:41-45)
+ *     y = y > 0 ? y : 0                     when relu_after_add: the Relu layer that follows the block
+ * with `residual` shaped like y.  Results equal the separate calls bit for bit.  residual may alias neither x
+ * nor y.  Same optional workspace as the forward. */
+int pydtnn_hip_sconvGemm_residual(int nhwc, unsigned b, unsigned c, unsigned h, unsigned w, unsigned kn, unsigned kh,
+                                  unsigned kw, unsigned vpadding, unsigned hpadding, unsigned vstride,
+                                  unsigned hstride, unsigned vdilation, unsigned hdilation, const float *weights,
+                                  const float *x, float *y, const float *bias_vector, const float *bn_running_mean,
+                                  const float *bn_inv_std, const float *bn_gamma, const float *bn_beta, bool relu,
+                                  const float *residual, bool relu_after_add, void *workspace, size_t workspace_bytes,
+                                  void *stream);
+
 /* BatchNormalization in training mode (pydtnn/backends/cpu/layers/batch_normalization_cpu.py:59-82 and
  * :108-129; dx as pydtnn/cython_modules/bn_training_cython.pyx:236-243).  Tensors are viewed as
  * (outer, channels, inner): NCHW = (N, C, H*W); NHWC and 2-D = (rows, C, 1).  With n = outer * inner:

@@ -40,11 +40,15 @@ class ConvGemm:
     # ------------------------------------------------------------------ forward / dW
     def conv_gemm_nchw(self, weights, x, biases=None, vpadding=0, hpadding=0, vstride=1, hstride=1,
                        vdilation=1, hdilation=1, biases_vector=None, trans=False, bn_running_mean=None,
-                       bn_inv_std=None, bn_gamma=None, bn_beta=None, relu=False, relu_mask=None):
+                       bn_inv_std=None, bn_gamma=None, bn_beta=None, relu=False, relu_mask=None, residual=None,
+                       relu_after_residual=False):
         """``weights * im2col(x)`` (+ fused bias / BN / ReLU), or with ``trans`` the filter gradient
         ``dy_cols * im2col(x)^T`` written into ``biases`` (pydtnn/backends/cpu/libs/conv_gemm.py:117-207).
         ``relu_mask`` (not in the reference; forward with ``relu`` and no BN only): an int8 tensor shaped
-        like the output that receives the mask a separate ReLU layer would keep for its backward."""
+        like the output that receives the mask a separate ReLU layer would keep for its backward.
+        ``residual`` (not in the reference; forward only): a tensor shaped like the output that is added
+        after the bias / BN / ReLU chain, i.e. the sum an addition block makes of its paths; with
+        ``relu_after_residual`` the sum is rectified (the Relu layer that follows the block)."""
         b, c, h, w = x.shape
         if not trans:
             kn, ck, kh, kw = weights.shape
@@ -76,6 +80,14 @@ class ConvGemm:
                 f32(x), f32(biases), f32(biases_vector), ptr(relu_mask), ws, ws_bytes, stream_ptr()),
                 "sconvGemm_relu_mask")
             return biases
+        if residual is not None:
+            self._check_residual(residual, biases, trans, relu_mask)
+            check(lib().pydtnn_hip_sconvGemm_residual(
+                0, b, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation, f32(weights),
+                f32(x), f32(biases), f32(biases_vector), f32(bn_running_mean), f32(bn_inv_std), f32(bn_gamma),
+                f32(bn_beta), bool(relu), f32(residual), bool(relu_after_residual), ws, ws_bytes, stream_ptr()),
+                "sconvGemm_residual")
+            return biases
         check(lib().pydtnn_hip_sconvGemmNCHW(
             b'Y' if trans else b'N', b, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation,
             hdilation, f32(weights), f32(x), f32(biases), f32(biases_vector), f32(bn_running_mean), f32(bn_inv_std),
@@ -84,7 +96,8 @@ class ConvGemm:
 
     def conv_gemm_nhwc(self, weights, x, biases=None, vpadding=0, hpadding=0, vstride=1, hstride=1,
                        vdilation=1, hdilation=1, biases_vector=None, trans=False, bn_running_mean=None,
-                       bn_inv_std=None, bn_gamma=None, bn_beta=None, relu=False, relu_mask=None):
+                       bn_inv_std=None, bn_gamma=None, bn_beta=None, relu=False, relu_mask=None, residual=None,
+                       relu_after_residual=False):
         """NHWC twin (pydtnn/backends/cpu/libs/conv_gemm.py:209-250): weights (c, kh, kw, kn)."""
         b, h, w, c = x.shape
         if not trans:
@@ -114,6 +127,14 @@ class ConvGemm:
                 f32(x), f32(biases), f32(biases_vector), ptr(relu_mask), ws, ws_bytes, stream_ptr()),
                 "sconvGemm_relu_mask")
             return biases
+        if residual is not None:
+            self._check_residual(residual, biases, trans, relu_mask)
+            check(lib().pydtnn_hip_sconvGemm_residual(
+                1, b, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation, f32(weights),
+                f32(x), f32(biases), f32(biases_vector), f32(bn_running_mean), f32(bn_inv_std), f32(bn_gamma),
+                f32(bn_beta), bool(relu), f32(residual), bool(relu_after_residual), ws, ws_bytes, stream_ptr()),
+                "sconvGemm_residual")
+            return biases
         check(lib().pydtnn_hip_sconvGemmNHWC(
             b'Y' if trans else b'N', b, h, w, c, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation,
             hdilation, f32(weights), f32(x), f32(biases), f32(biases_vector), f32(bn_running_mean), f32(bn_inv_std),
@@ -126,6 +147,13 @@ class ConvGemm:
             "relu_mask goes with a forward call that applies ReLU and no batch normalization"
         assert relu_mask.dtype == torch.int8 and relu_mask.shape == out.shape and relu_mask.is_contiguous(), \
             "relu_mask must be a contiguous int8 tensor shaped like the output"
+
+    @staticmethod
+    def _check_residual(residual, out, trans, relu_mask):
+        assert not trans and relu_mask is None, "residual goes with a forward call without relu_mask"
+        assert residual.dtype == out.dtype and residual.shape == out.shape and residual.is_contiguous(), \
+            "residual must be a contiguous tensor shaped like the output"
+        assert residual.data_ptr() != out.data_ptr(), "residual must not be the output tensor"
 
     @staticmethod
     def _check_gate(gate, dx):

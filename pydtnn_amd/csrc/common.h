@@ -94,30 +94,39 @@ static inline ChanEpilogue no_epilogue()
     return e;
 }
 
-// Per-element byte masks a GEMM store can read or write beside its output, both indexed like the output:
+// Per-element companions a GEMM store can read or write beside its output, all indexed like the output:
 //   gate      (input)  the value is stored as v * gate[i], i.e. ReLU's backward dx = dy * mask
 //                      (pydtnn/backends/cpu/activations/relu_cpu.py:38-40) applied by the producer of dy;
 //   relu_mask (output) relu_mask[i] = v > 0, the mask ReLU's forward keeps for its backward
-//                      (pydtnn/cython_modules/relu_cython.pyx:25-59), written by a store that also rectifies.
+//                      (pydtnn/cython_modules/relu_cython.pyx:25-59), written by a store that also rectifies;
+//   residual  (input)  the value is stored as v + residual[i], the sum an addition block makes of its paths
+//                      (pydtnn/backends/cpu/layers/addition_block_cpu.py:41-45, eltw_sum_cython.pyx:25-36),
+//                      then rectified when relu_after_add is set (the Relu layer that follows the block).
 struct ElemMasks {
     const int8_t* gate;
     int8_t* relu_mask;
+    const float* residual;
+    int relu_after_add;
 };
 
 static inline ElemMasks no_masks()
 {
-    ElemMasks m = {nullptr, nullptr};
+    ElemMasks m = {nullptr, nullptr, nullptr, 0};
     return m;
 }
 
-// Which of the two a store handles is a compile-time choice, so that no store tests a pointer per element.
-constexpr int kNoMasks = 0, kGate = 1, kReluMask = 2;
+// Which of them a store handles is a compile-time choice, so that no store tests a pointer per element.
+constexpr int kNoMasks = 0, kGate = 1, kReluMask = 2, kResidual = 3;
 
 template <int MASKS>
 __device__ __forceinline__ float elem_masks_apply(const ElemMasks& mk, long i, float v)
 {
     if (MASKS == kGate) v *= (float)mk.gate[i];
     if (MASKS == kReluMask) mk.relu_mask[i] = v > 0.0f ? 1 : 0;
+    if (MASKS == kResidual) {
+        v += mk.residual[i];
+        if (mk.relu_after_add) v = v > 0.0f ? v : 0.0f;
+    }
     return v;
 }
 

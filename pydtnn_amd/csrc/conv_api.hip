@@ -24,7 +24,7 @@ int conv_dx(const ConvGeom& g, int nhwc, const float* w, const float* dy, float*
     const size_t used = (need + 255) & ~(size_t)255;
     float* rest = ws_bytes > used ? ws + used / 4 : nullptr;
     const size_t rest_bytes = ws_bytes > used ? ws_bytes - used : 0;
-    const ElemMasks masks = {gate, nullptr};
+    const ElemMasks masks = {gate, nullptr, nullptr, 0};
     return nhwc ? conv_fwd_nhwc(gb, ws, dy, dx, no_epilogue(), rest, rest_bytes, stream, masks)
                 : conv_fwd_nchw(gb, ws, dy, dx, no_epilogue(), rest, rest_bytes, stream, masks);
 }
@@ -43,14 +43,15 @@ int geom_from_args(ConvGeom* g, long b, long c, long h, long w, long kn, long kh
 int sconv_gemm(int nhwc, char trans, const ConvGeom& g, const float* in1, const float* x, float* out,
                const float* bias, const float* mean, const float* inv_std, const float* gamma, const float* beta,
                bool relu, void* ws, size_t ws_bytes, hipStream_t stream, int accumulate = 0,
-               int8_t* relu_mask = nullptr)
+               int8_t* relu_mask = nullptr, const float* residual = nullptr, int relu_after_add = 0)
 {
     if (!in1 || !x || !out) return PYDTNN_HIP_ERR_INVALID;
     if (relu_mask && !relu) return PYDTNN_HIP_ERR_INVALID;
+    if (residual && (relu_mask || trans != 'N')) return PYDTNN_HIP_ERR_INVALID;
     if (trans == 'N') {
         if (!bn_args_consistent(mean, inv_std, gamma, beta)) return PYDTNN_HIP_ERR_INVALID;
         const ChanEpilogue chan = make_chan(bias, mean, inv_std, gamma, beta, relu ? 1 : 0);
-        const ElemMasks masks = {nullptr, relu_mask};
+        const ElemMasks masks = {nullptr, relu_mask, residual, relu_after_add};
         return nhwc ? conv_fwd_nhwc(g, in1, x, out, chan, (float*)ws, ws_bytes, stream, masks)
                     : conv_fwd_nchw(g, in1, x, out, chan, (float*)ws, ws_bytes, stream, masks);
     }
@@ -97,7 +98,7 @@ int sconv_gemm_batched(int nhwc, char trans, long b, long c, long h, long w, lon
                        long hpadding, long vstride, long hstride, long vdilation, long hdilation, const float* in1,
                        const float* x, float* out, const float* bias, const float* mean, const float* inv_std,
                        const float* gamma, const float* beta, bool relu, void* ws, size_t ws_bytes, hipStream_t stream,
-                       int8_t* relu_mask = nullptr)
+                       int8_t* relu_mask = nullptr, const float* residual = nullptr, int relu_after_add = 0)
 {
     if (!in1 || !x || !out) return PYDTNN_HIP_ERR_INVALID;
     ImageGroups ig;
@@ -114,7 +115,8 @@ int sconv_gemm_batched(int nhwc, char trans, long b, long c, long h, long w, lon
                             relu, ws, ws_bytes, stream, n0 > 0);
         else               // in1 = weights, out = y
             rc = sconv_gemm(nhwc, trans, g, in1, xg, out + n0 * ig.per_image_out, bias, mean, inv_std, gamma, beta,
-                            relu, ws, ws_bytes, stream, 0, relu_mask ? relu_mask + n0 * ig.per_image_out : nullptr);
+                            relu, ws, ws_bytes, stream, 0, relu_mask ? relu_mask + n0 * ig.per_image_out : nullptr,
+                            residual ? residual + n0 * ig.per_image_out : nullptr, relu_after_add);
         if (rc != PYDTNN_HIP_OK) return rc;
     }
     return PYDTNN_HIP_OK;
@@ -535,6 +537,20 @@ int pydtnn_hip_sconvGemm_relu_mask(int nhwc, unsigned b, unsigned c, unsigned h,
     if (!mask) return PYDTNN_HIP_ERR_INVALID;
     return sconv_gemm_batched(nhwc, 'N', GEOM_ARGS, weights, x, y, bias_vector, nullptr, nullptr, nullptr, nullptr,
                               true, workspace, workspace_bytes, as_stream(stream), mask);
+}
+
+int pydtnn_hip_sconvGemm_residual(int nhwc, unsigned b, unsigned c, unsigned h, unsigned w, unsigned kn, unsigned kh,
+                                  unsigned kw, unsigned vpadding, unsigned hpadding, unsigned vstride,
+                                  unsigned hstride, unsigned vdilation, unsigned hdilation, const float* weights,
+                                  const float* x, float* y, const float* bias_vector, const float* bn_running_mean,
+                                  const float* bn_inv_std, const float* bn_gamma, const float* bn_beta, bool relu,
+                                  const float* residual, bool relu_after_add, void* workspace, size_t workspace_bytes,
+                                  void* stream)
+{
+    if (!residual) return PYDTNN_HIP_ERR_INVALID;
+    return sconv_gemm_batched(nhwc, 'N', GEOM_ARGS, weights, x, y, bias_vector, bn_running_mean, bn_inv_std, bn_gamma,
+                              bn_beta, relu, workspace, workspace_bytes, as_stream(stream), nullptr, residual,
+                              relu_after_add ? 1 : 0);
 }
 
 int pydtnn_hip_sconvGemm_back_gated(int nhwc, unsigned b, unsigned c, unsigned h, unsigned w, unsigned kn, unsigned kh,

@@ -14,6 +14,9 @@ int launch_planes_forward(const AL& al, const BL& bl, const ConvGeom& g, float* 
     case kReluMask:
         return launch_balanced<T>(al, bl, epi_nchw<kReluMask>(y, g.kn, g.howo, g.p, chan, masks), g.kn, g.p, g.k, ws,
                                   ws_bytes, stream);
+    case kResidual:
+        return launch_balanced<T>(al, bl, epi_nchw<kResidual>(y, g.kn, g.howo, g.p, chan, masks), g.kn, g.p, g.k, ws,
+                                  ws_bytes, stream);
     default:
         return launch_balanced<T>(al, bl, epi_nchw(y, g.kn, g.howo, g.p, chan), g.kn, g.p, g.k, ws, ws_bytes, stream);
     }

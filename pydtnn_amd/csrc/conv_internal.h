@@ -246,8 +246,12 @@ inline EpiNchwT<MASKS> epi_nchw(float* out, int channels, int howo, long p, cons
     return e;
 }
 
-// at most one of the two is ever set: the forward writes a ReLU mask, dX reads a gate
-inline int mask_kind(const ElemMasks& m) { return m.gate ? kGate : m.relu_mask ? kReluMask : kNoMasks; }
+// at most one of them is ever set: a training forward writes a ReLU mask, dX reads a gate, an inference
+// forward at the end of an addition block's path adds the other path
+inline int mask_kind(const ElemMasks& m)
+{
+    return m.gate ? kGate : m.relu_mask ? kReluMask : m.residual ? kResidual : kNoMasks;
+}
 
 // ---------------------------------------------------------------- forward (implicit)
 // The padding test works on tap masks of 31 usable bits: one word over i*kw + j when kh*kw <= 31,
@@ -289,6 +293,9 @@ inline int launch_rows_forward(const AL& al, const BL& bl, const ConvGeom& g, fl
                                         ws_bytes, stream);
     case kReluMask:
         return gemm::launch_balanced<T>(al, bl, epi_plain<kReluMask>(y, g.kn, 0, g.p, g.kn, chan, masks), g.p, g.kn,
+                                        g.k, ws, ws_bytes, stream);
+    case kResidual:
+        return gemm::launch_balanced<T>(al, bl, epi_plain<kResidual>(y, g.kn, 0, g.p, g.kn, chan, masks), g.p, g.kn,
                                         g.k, ws, ws_bytes, stream);
     default:
         return gemm::launch_balanced<T>(al, bl, epi_plain(y, g.kn, 0, g.p, g.kn, chan), g.p, g.kn, g.k, ws, ws_bytes,

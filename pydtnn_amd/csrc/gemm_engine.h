@@ -854,8 +854,8 @@ struct Im2rowNhwcMN {
 // ---------------------------------------------------------------- epilogues
 // Row-major store C[split*split_stride + m*ldc + n]; the per-channel chain uses the column index
 // (NHWC convolution, FC forward).
-// MASKS (kNoMasks, kGate, kReluMask): the store also applies the gate or writes the ReLU mask (separate
-// instantiations, so that no case carries a test per stored element).
+// MASKS (kNoMasks, kGate, kReluMask, kResidual): the store also applies the gate, writes the ReLU mask or adds
+// the residual (separate instantiations, so that no case carries a test per stored element).
 template <int MASKS>
 struct EpiPlainT {
     using Unmasked = EpiPlainT<kNoMasks>;
@@ -1191,8 +1191,22 @@ __device__ __forceinline__ void store_tile_nchw(const EpiNchwT<MASKS>& ep, const
     if constexpr (MASKS == kGate) gate_rsrc = make_rsrc_bytes(ep.masks.gate, total);
     [[maybe_unused]] rsrc_t mask_rsrc;
     if constexpr (MASKS == kReluMask) mask_rsrc = make_rsrc_bytes(ep.masks.relu_mask, total);
+    if constexpr (MASKS == kResidual) gate_rsrc = make_rsrc(ep.masks.residual, total);
 #pragma unroll
     for (int i0 = 0; i0 < T::TM; i0 += kRowBlocksPerBatch) {
+        if constexpr (MASKS == kResidual) {  // the residual values of the batch, like the gate bytes below
+#pragma unroll
+            for (int ib = 0; ib < kRowBlocksPerBatch; ++ib)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int r = (i0 + ib) * 32 + 8 * (v / 4) + (v % 4);
+                    const bool row_ok = lane_m0 + r < ep.m_extent;
+                    const uint32_t soff = (uint32_t)(m0 + wm0 + r) * (uint32_t)ep.howo;
+#pragma unroll
+                    for (int j = 0; j < T::TN; ++j)
+                        gate[ib][v][j] = buf_load(gate_rsrc, row_ok ? col_off4[j] : kOob, soff * 4u);
+                }
+        }
         if constexpr (MASKS == kGate) {
 #pragma unroll
             for (int ib = 0; ib < kRowBlocksPerBatch; ++ib)
@@ -1234,6 +1248,10 @@ __device__ __forceinline__ void store_tile_nchw(const EpiNchwT<MASKS>& ep, const
                     }
                     if (ch.relu) val = val > 0.0f ? val : 0.0f;
                     if constexpr (MASKS == kGate) val *= gate[ib][v][j];
+                    if constexpr (MASKS == kResidual) {
+                        val += gate[ib][v][j];
+                        if (ep.masks.relu_after_add) val = val > 0.0f ? val : 0.0f;
+                    }
                     __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, val), out_rsrc,
                                                           (int)(row_ok ? col_off4[j] : kOob), (int)(soff * 4u), 0);
                     if constexpr (MASKS == kReluMask)
@@ -1267,6 +1285,7 @@ __device__ __forceinline__ void store_tile_plain(const EpiPlainT<MASKS>& ep, con
     [[maybe_unused]] rsrc_t mask_rsrc;
     if constexpr (MASKS == kGate) mask_rsrc = make_rsrc_bytes(ep.masks.gate, ep.span);
     if constexpr (MASKS == kReluMask) mask_rsrc = make_rsrc_bytes(ep.masks.relu_mask, ep.span);
+    if constexpr (MASKS == kResidual) mask_rsrc = make_rsrc(ep.masks.residual, ep.span);
     const int lane_m0 = m0 + wm0 + 4 * frag_k;  // this lane's first row
     const uint32_t ldc = (uint32_t)ep.ldc;
 #pragma unroll
@@ -1297,6 +1316,16 @@ __device__ __forceinline__ void store_tile_plain(const EpiPlainT<MASKS>& ep, con
                         mask_rsrc, (int)(row_ok ? off1 : kOob), (int)((uint32_t)(m0 + wm0 + r) * ldc), 0);
                 }
         }
+        if constexpr (MASKS == kResidual) {
+#pragma unroll
+            for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int r = i * 32 + 8 * (v / 4) + (v % 4);
+                    const bool row_ok = lane_m0 + r < ep.m_extent;
+                    gate[i][v] = buf_load(mask_rsrc, row_ok ? off4 : kOob, (uint32_t)(m0 + wm0 + r) * ldc * 4u);
+                }
+        }
 #pragma unroll
         for (int i = 0; i < T::TM; ++i)
 #pragma unroll
@@ -1312,6 +1341,10 @@ __device__ __forceinline__ void store_tile_plain(const EpiPlainT<MASKS>& ep, con
                 }
                 if (ch.relu) val = val > 0.0f ? val : 0.0f;
                 if constexpr (MASKS == kGate) val *= gate[i][v];
+                if constexpr (MASKS == kResidual) {
+                    val += gate[i][v];
+                    if (ep.masks.relu_after_add) val = val > 0.0f ? val : 0.0f;
+                }
                 __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, val), out_rsrc,
                                                       (int)(row_ok ? off4 : kOob), (int)(soff * 4u), 0);
                 if constexpr (MASKS == kReluMask)

@@ -783,15 +783,20 @@ class _FusedConv(Conv2D, _FromParents):
                       bn_beta=self.beta)
         return kw
 
-    def _forward_nchw_cg(self, x):
+    def _forward_nchw_cg(self, x, residual=None, relu_after_residual=False):
         if self.model.mode == TRAIN_MODE:
             raise RuntimeError("Fused layers cannot be used in training mode!")
-        return self.cg.conv_gemm_nchw(self.weights, x, biases=None, **self._epilogue_kwargs())
+        return self.cg.conv_gemm_nchw(self.weights, x, biases=None, residual=residual,
+                                      relu_after_residual=relu_after_residual, **self._epilogue_kwargs())
 
-    def _forward_nhwc_cg(self, x):
+    def _forward_nhwc_cg(self, x, residual=None, relu_after_residual=False):
         if self.model.mode == TRAIN_MODE:
             raise RuntimeError("Fused layers cannot be used in training mode!")
-        return self.cg.conv_gemm_nhwc(self.weights, x, biases=None, **self._epilogue_kwargs())
+        return self.cg.conv_gemm_nhwc(self.weights, x, biases=None, residual=residual,
+                                      relu_after_residual=relu_after_residual, **self._epilogue_kwargs())
+
+    # the sum of an addition block (and the Relu after it) can ride in this layer's store
+    accepts_residual = True
 
     def backward(self, x):
         raise RuntimeError(f"Backward method of {self.__class__.__name__} should not be called")
@@ -834,7 +839,31 @@ class AdditionBlock(Layer):
         assert all([o == self.out_shapes[0] for o in self.out_shapes])
         self.shape = self.out_shapes[0]
 
+    def _folded_sum_path(self):
+        """Index of the path whose last layer can add the other path's result in its own store, or None.
+        Only after the model's fusion pass, in EVALUATE_MODE, for blocks of two paths (a sum of two is the
+        same bits in either order; three or more would fix an order)."""
+        if not getattr(self.model, "_fused", False) or self.model.mode != EVALUATE_MODE or len(self.paths) != 2:
+            return None
+        for i, p in enumerate(self.paths):
+            if p and getattr(p[-1], "accepts_residual", False):
+                return i
+        return None
+
     def forward(self, x):
+        k = self._folded_sum_path()
+        if k is not None:
+            other = x
+            for layer in self.paths[1 - k]:
+                other = layer.forward(other)
+            cur = x
+            for layer in self.paths[k][:-1]:
+                cur = layer.forward(cur)
+            relu = self.relu_above is not None
+            y = self.paths[k][-1].forward(cur, residual=other, relu_after_residual=relu)
+            if relu:
+                self.relu_above.take_folded(y, None)
+            return y
         xs = [x] * len(self.paths)
         for i, p in enumerate(self.paths):
             for layer in p:

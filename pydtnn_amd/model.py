@@ -160,9 +160,21 @@ class Model:
                 fused.append(curr)
             return fused
 
+        def link_blocks(layers):
+            # an addition block whose sum is made by the last convolution of a path (AdditionBlock.forward)
+            # can also do the Relu layer that consumes its output
+            for i, layer in enumerate(layers):
+                if layer.is_block_layer:
+                    nxt = layers[i + 1] if i + 1 < len(layers) else None
+                    layer.relu_above = nxt if type(nxt) is L.Relu else None
+                    for p in layer.paths:
+                        link_blocks(p)
+
         if bn_relu or conv_relu or conv_bn or conv_bn_relu:
             self.layers = fuse(self.layers)
             self._fused = True
+            if conv_relu or conv_bn or conv_bn_relu:
+                link_blocks(self.layers)
 
     # ------------------------------------------------------------------ loops
     def train_batch(self, x, y_targ, loss_func, optimizer, global_batch_size=None):

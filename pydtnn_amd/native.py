@@ -42,6 +42,8 @@ SIGNATURES = {
     "pydtnn_hip_sconvGemmNCHW_back": (_c.c_int, _geom13_u + [_f32p] * 3 + [_vp, _c.c_size_t, _vp]),
     "pydtnn_hip_sconvGemmNHWC_back": (_c.c_int, _geom13_u + [_f32p] * 3 + [_vp, _c.c_size_t, _vp]),
     "pydtnn_hip_sconvGemm_relu_mask": (_c.c_int, [_c.c_int] + _geom13_u + [_f32p] * 4 + [_i8p, _vp, _c.c_size_t, _vp]),
+    "pydtnn_hip_sconvGemm_residual": (_c.c_int, [_c.c_int] + _geom13_u + [_f32p] * 8 + [_c.c_bool, _f32p, _c.c_bool, _vp,
+                                                 _c.c_size_t, _vp]),
     "pydtnn_hip_sconvGemm_back_gated": (_c.c_int, [_c.c_int] + _geom13_u + [_f32p] * 3 + [_i8p, _vp, _c.c_size_t, _vp]),
     "pydtnn_hip_max_pool_2d_bwd_gated": (_c.c_int, [_c.c_int, _f32p, _i32p, _f32p, _i8p] + [_c.c_int] * 12 + [_vp]),
     "pydtnn_hip_conv_i2c_forward": (_c.c_int, [_c.c_int] + _geom13_i + [_f32p] * 4 + [_vp]),

@@ -660,6 +660,37 @@ def test_conv_forward_with_relu_mask_equals_conv_then_relu(ops, cg, fmt, d):
     assert 0 < int(mask.sum()) < mask.numel()
 
 
+# shapes of the bottleneck's last convolution (1x1, few reduction steps, 256 filters) join the grid here
+residual_grid = fold_grid + [D(4, 64, 28, 28, 256, 1, 1, 0, 0, 1, 1, 1, 1), D(2, 256, 14, 14, 64, 1, 1, 0, 0, 1, 1, 1, 1)]
+
+
+@pytest.mark.parametrize("d", residual_grid, ids=repr)
+@pytest.mark.parametrize("fmt", ["NCHW", "NHWC"])
+@pytest.mark.parametrize("relu_after", [False, True], ids=["sum", "sum_relu"])
+def test_conv_forward_with_residual_equals_conv_then_sum_then_relu(ops, cg, fmt, d, relu_after):
+    """The addition block's sum (and the Relu after it) done by the convolution's store: bit for bit what
+    eltw_sum and relu make of the plain fused call's output."""
+    announce("conv+residual", fmt, d, relu_after)
+    x, w, b, dy = case(d)
+    rng = np.random.default_rng(11)
+    bn = [rng.uniform(0.5, 1.5, d.kn).astype(np.float32) for _ in range(4)]
+    res_np = rng.standard_normal(dy.shape).astype(np.float32)
+    if fmt == "NCHW":
+        conv, xs, ws, res = cg.conv_gemm_nchw, dev(x), dev(w), dev(res_np)
+    else:
+        conv, xs, ws, res = cg.conv_gemm_nhwc, dev(nhwc(x)), dev(w_nhwc(w)), dev(nhwc(res_np))
+    epi = dict(biases_vector=dev(b), bn_running_mean=dev(bn[0]), bn_inv_std=dev(bn[1]), bn_gamma=dev(bn[2]),
+               bn_beta=dev(bn[3]), **_kw(d))
+    ref = conv(ws, xs, **epi)
+    ops.eltw_sum(ref, res)
+    if relu_after:
+        ref, _ = ops.relu(ref, with_mask=False)
+    y = torch.full(ref.shape, np.nan, device="cuda")
+    conv(ws, xs, biases=y, residual=res, relu_after_residual=relu_after, **epi)
+    assert torch.equal(y, ref)
+    assert torch.equal(res, dev(res_np if fmt == "NCHW" else nhwc(res_np))), "the residual must stay untouched"
+
+
 @pytest.mark.parametrize("d", fold_grid, ids=repr)
 @pytest.mark.parametrize("fmt", ["NCHW", "NHWC"])
 def test_conv_dx_with_gate_equals_dx_then_relu_backward(ops, cg, fmt, d):

@@ -233,6 +233,16 @@ def test_residual_block_with_fusion(pd, oracle):
         ["Conv2DBatchNormalizationRelu", "Conv2DBatchNormalizationRelu", "Conv2DBatchNormalization"]
     assert np.array_equal(host(xd), x), "the block must not add into its input"
     assert_close(host(y_fused), host(y_plain), tol=1e-6, what="bottleneck fused vs plain")
+    # the fused model's block lets its last convolution add the shortcut and do the Relu that follows; the
+    # same layers with that hand-over switched off (separate eltw_sum and relu passes) give the same bits
+    assert block.relu_above is fused.layers[2] and block._folded_sum_path() == 0
+    fused._fused = False
+    try:
+        assert block._folded_sum_path() is None
+        y_separate = fused.evaluate_batch(xd)
+    finally:
+        fused._fused = True
+    assert torch.equal(y_fused, y_separate)
     # oracle: relu(x + bn3(conv3(relu(bn2(conv2(relu(bn1(conv1(x)))))))))
     convs = [l for l in plain.get_all_layers() if l.canonical_name == "Conv2D"]
     bns = [l for l in plain.get_all_layers() if l.canonical_name == "BatchNormalization"]
