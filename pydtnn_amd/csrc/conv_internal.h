@@ -313,6 +313,10 @@ int conv_fwd_nhwc(const ConvGeom& g, const float* w, const float* x, float* y, c
 // conv_fwd_nhwc_pointwise.hip
 int conv_fwd_nhwc_pointwise(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan,
                             float* ws, size_t ws_bytes, hipStream_t stream, const ElemMasks& masks);
+// conv_stream.hip: small filter matrices (whole in LDS), activations straight from memory into MFMA operands
+bool conv_stream_nhwc_eligible(const ConvGeom& g, const float* w, const float* x);
+int conv_stream_nhwc(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan,
+                     hipStream_t stream, const ElemMasks& masks);
 // conv_bwd.hip
 SplitPlan plan_dw(const ConvGeom& g, int nhwc);
 int conv_dw_nchw(const ConvGeom& g, const float* dy, const float* x, const float* cols, float* dw, float* ws,

@@ -27,6 +27,19 @@ mid_grid = [
 ]
 all_grid = small_grid + mid_grid
 
+# NHWC shapes that take the streaming kernel (filter matrix resident in LDS, at most 36864 floats, channels in
+# chunks of 64, at least 32768 output pixels): the three convolutions of a ResNet bottleneck, a strided
+# 1x1 shortcut, a dilated 3x3, 128 filters
+stream_grid = [
+    D(16, 256, 56, 56, 64, 1, 1, 0, 0, 1, 1, 1, 1),
+    D(16, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1, 1, 1),
+    D(16, 64, 56, 56, 256, 1, 1, 0, 0, 1, 1, 1, 1),
+    D(48, 128, 56, 56, 256, 1, 1, 0, 0, 2, 2, 1, 1),
+    D(16, 64, 48, 48, 64, 3, 3, 2, 2, 1, 1, 2, 2),
+    D(11, 128, 64, 64, 128, 1, 1, 0, 0, 1, 1, 1, 1),
+    D(40, 64, 31, 33, 128, 2, 2, 1, 0, 1, 1, 1, 1),
+]
+
 
 @pytest.fixture(scope="module")
 def ops():
@@ -176,6 +189,31 @@ def test_conv_gemm_forward_both_formats(cg, oracle, d):
     y2 = cg.conv_gemm_nhwc(dev(w_nhwc(w)), dev(nhwc(x)), biases_vector=dev(b), **_kw(d))
     ref_nhwc, _ = oracle.conv2d_forward_nhwc_i2c(nhwc(x), w_nhwc(w), b, oracle.ConvParams(*d.geom()))
     assert_close(host(y2), ref_nhwc, what="nhwc")
+
+
+@pytest.mark.parametrize("d", stream_grid, ids=repr)
+def test_streaming_kernel_shapes_nhwc(cg, oracle, d):
+    """Forward (with bias, BN and ReLU), filter gradient and input gradient of the shapes above, NHWC."""
+    announce("stream shapes", d)
+    assert (d.b * d.ho * d.wo) % 32 == 0 and d.b * d.ho * d.wo >= 32768
+    x, w, b, dy = case(d)
+    rng = np.random.default_rng(9)
+    bn = [rng.uniform(0.5, 1.5, d.kn).astype(np.float32) for _ in range(4)]
+    xr, wr, dyr = nhwc(x), w_nhwc(w), nhwc(dy)
+    p = oracle.ConvParams(*d.geom())
+    y_ref, rows = oracle.conv2d_forward_nhwc_i2c(xr, wr, b, p)
+    y = cg.conv_gemm_nhwc(dev(wr), dev(xr), biases_vector=dev(b), **_kw(d))
+    assert_close(host(y), y_ref, what="y")
+    y = cg.conv_gemm_nhwc(dev(wr), dev(xr), biases_vector=dev(b), bn_running_mean=dev(bn[0]), bn_inv_std=dev(bn[1]),
+                          bn_gamma=dev(bn[2]), bn_beta=dev(bn[3]), relu=True, **_kw(d))
+    assert_close(host(y), oracle.fused_epilogue(y_ref, "NHWC", bn=bn, relu_flag=True), what="fused y")
+    dw_ref, _, dx_ref = oracle.conv2d_backward_nhwc_i2c(dyr, rows, wr, xr.shape, p)
+    dx = torch.full(xr.shape, np.nan, device="cuda")
+    cg.deconv_gemm_nhwc(dev(wr), dev(dyr), dx, **_kw(d))
+    assert_close(host(dx), dx_ref, what="dx")
+    dw = torch.empty_like(dev(wr))
+    cg.conv_gemm_nhwc(dev(dyr), dev(xr), biases=dw, trans=True, **_kw(d))
+    assert_close(host(dw), dw_ref, what="dw")
 
 
 @pytest.mark.parametrize("x,w,stride", [
@@ -661,7 +699,8 @@ def test_conv_forward_with_relu_mask_equals_conv_then_relu(ops, cg, fmt, d):
 
 
 # shapes of the bottleneck's last convolution (1x1, few reduction steps, 256 filters) join the grid here
-residual_grid = fold_grid + [D(4, 64, 28, 28, 256, 1, 1, 0, 0, 1, 1, 1, 1), D(2, 256, 14, 14, 64, 1, 1, 0, 0, 1, 1, 1, 1)]
+residual_grid = fold_grid + [D(4, 64, 28, 28, 256, 1, 1, 0, 0, 1, 1, 1, 1), D(2, 256, 14, 14, 64, 1, 1, 0, 0, 1, 1, 1, 1),
+                             stream_grid[0], stream_grid[2], stream_grid[3]]
 
 
 @pytest.mark.parametrize("d", residual_grid, ids=repr)
