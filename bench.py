@@ -261,19 +261,9 @@ def cpu_baseline_cfg2(sample_images=64, reps=30):
 
 
 def build_vgg16(pd, n=64, tensor_format="NCHW", **flags):
+    """pydtnn/models/vgg16.py without its two Dropout(0.5) layers (the configuration has none)."""
     model = pd.Model(tensor_format=tensor_format, batch_size=n, **flags)
-    model.add(pd.Input(shape=(224, 224, 3)))
-    for nlayers, nfilters in [[2, 64], [2, 128], [3, 256], [3, 512], [3, 512]]:
-        for _ in range(nlayers):
-            model.add(pd.Conv2D(nfilters=nfilters, filter_shape=(3, 3), padding=1, stride=1, activation="relu",
-                                weights_initializer="he_normal"))
-        model.add(pd.MaxPool2D(pool_shape=(2, 2), stride=2))
-    model.add(pd.Flatten())
-    # pydtnn/models/vgg16.py:34-38 without the two Dropout(0.5) layers (the configuration has none)
-    model.add(pd.FC(shape=(4096,), activation="relu", weights_initializer="he_normal"))
-    model.add(pd.FC(shape=(4096,), activation="relu", weights_initializer="he_normal"))
-    model.add(pd.FC(shape=(1000,), activation="softmax", weights_initializer="he_normal"))
-    return model
+    return pd.models.create_vgg16_imagenet(model, dropout=False)
 
 
 def run_cfg5(torch, pd, args, steps=None, warmup=None):

@@ -217,6 +217,17 @@ int pydtnn_hip_max_pool_2d_bwd_nhwc(const float *dy, const int32_t *idx_max, flo
                                     int kh, int kw, int vpadding, int hpadding, int vstride, int hstride,
                                     int vdilation, int hdilation, void *stream);
 
+/* AveragePool2D in either format (nhwc = 0: pydtnn/cython_modules/average_pool_2d_nchw_cython.pyx:25-52 and
+ * :135-160; nhwc = 1: average_pool_2d_nhwc_cython.pyx, same lines): the mean over the window's taps that lie
+ * inside the image (padding is not counted); backward gives every such tap dy / count.  b, c, h, w name the
+ * input's batch, channels, height, width; dx is fully written. */
+int pydtnn_hip_average_pool_2d_fwd(int nhwc, const float *x, float *y, int b, int c, int h, int w, int kh, int kw,
+                                   int vpadding, int hpadding, int vstride, int hstride, int vdilation,
+                                   int hdilation, void *stream);
+int pydtnn_hip_average_pool_2d_bwd(int nhwc, const float *dy, float *dx, int b, int c, int h, int w, int kh, int kw,
+                                   int vpadding, int hpadding, int vstride, int hstride, int vdilation,
+                                   int hdilation, void *stream);
+
 /* ------------------------------------------------------------------------------------------
  * The ReLU layer between two layers of a training step, done by its neighbours' stores instead of
  * two passes of its own.  Results are those of the separate calls, bit for bit.

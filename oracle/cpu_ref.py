@@ -234,6 +234,33 @@ def max_pool_2d_bwd_nchw(dy, idx_max, n, c, h, w, kh, kw, vpadding, hpadding, vs
     return dx
 
 
+def average_pool_2d_fwd(x, tensor_format, kh, kw, vpadding, hpadding, vstride, hstride, vdilation=1, hdilation=1):
+    """pydtnn/cython_modules/average_pool_2d_nchw_cython.pyx:25-52 / average_pool_2d_nhwc_cython.pyx:25-52.
+    ``kh`` / ``kw`` of 0 mean the whole extent (pydtnn/layers/abstract_pool_2d_layer.py:44-47)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    if tensor_format == "NCHW":
+        n, c, h, w = x.shape
+    else:
+        n, h, w, c = x.shape
+    kh, kw = kh or h, kw or w
+    hh, ww = out_hw(h, w, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
+    y = np.zeros((n, c, hh, ww) if tensor_format == "NCHW" else (n, hh, ww, c), dtype=np.float32)
+    fn = getattr(lib(), f"oracle_average_pool_2d_{tensor_format.lower()}_fwd_f32")
+    fn(_p(x), _p(y), n, c, h, w, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
+    return y
+
+
+def average_pool_2d_bwd(dy, tensor_format, n, c, h, w, kh, kw, vpadding, hpadding, vstride, hstride,
+                        vdilation=1, hdilation=1):
+    """pydtnn/cython_modules/average_pool_2d_nchw_cython.pyx:135-160 / average_pool_2d_nhwc_cython.pyx:135-160"""
+    dy = np.ascontiguousarray(dy, dtype=np.float32)
+    kh, kw = kh or h, kw or w
+    dx = np.zeros((n, c, h, w) if tensor_format == "NCHW" else (n, h, w, c), dtype=np.float32)
+    fn = getattr(lib(), f"oracle_average_pool_2d_{tensor_format.lower()}_bwd_f32")
+    fn(_p(dy), _p(dx), n, c, h, w, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
+    return dx
+
+
 def max_pool_2d_fwd_nhwc(x, kh, kw, vpadding, hpadding, vstride, hstride, vdilation=1, hdilation=1):
     """pydtnn/cython_modules/max_pool_2d_nhwc_cython.pyx:25-52"""
     x = np.ascontiguousarray(x, dtype=np.float32)

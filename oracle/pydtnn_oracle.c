@@ -388,3 +388,76 @@ void oracle_max_pool_2d_bwd_nhwc_f32(const float *dy, const int32_t *idx_max, fl
                         dx[IDX_NHWC(nn, x_x, x_y, cc, h, w, c)] += dy[IDX_NHWC(nn, xx, yy, cc, hh, ww, c)];
                 }
 }
+
+/* ---------------------------------------------------------------------------
+ * AveragePool2D forward / backward, both tensor formats.
+ * pydtnn/cython_modules/average_pool_2d_nchw_cython.pyx:83-108 and :198-227,
+ * average_pool_2d_nhwc_cython.pyx:83-108 and :198-227: the window's taps that
+ * lie inside the image are summed in (ii, jj) order and divided by their
+ * number (padding is not counted); backward adds dy / items to every such
+ * tap, windows visited in ascending (xx, yy) order.
+ * ------------------------------------------------------------------------- */
+#define DEF_AVG_POOL(NAME, NHWC)                                                                         \
+void NAME##_fwd_f32(const float *x, float *y, int n, int c, int h, int w, int kh, int kw,               \
+                    int vpadding, int hpadding, int vstride, int hstride, int vdilation, int hdilation) \
+{                                                                                                        \
+    const int hh = out_dim(h, vpadding, vdilation, kh, vstride);                                         \
+    const int ww = out_dim(w, hpadding, hdilation, kw, hstride);                                         \
+    _Pragma("omp parallel for")                                                                          \
+    for (int nn = 0; nn < n; nn++)                                                                       \
+        for (int cc = 0; cc < c; cc++)                                                                   \
+            for (int xx = 0; xx < hh; xx++)                                                              \
+                for (int yy = 0; yy < ww; yy++) {                                                        \
+                    float accum = 0;                                                                     \
+                    int items = 0;                                                                       \
+                    for (int ii = 0; ii < kh; ii++) {                                                    \
+                        const int x_x = vstride * xx + vdilation * ii - vpadding;                        \
+                        if (0 <= x_x && x_x < h)                                                         \
+                            for (int jj = 0; jj < kw; jj++) {                                            \
+                                const int x_y = hstride * yy + hdilation * jj - hpadding;                \
+                                if (0 <= x_y && x_y < w) {                                               \
+                                    accum = accum + (NHWC ? x[IDX4(nn, x_x, x_y, cc, h, w, c)]           \
+                                                          : x[IDX4(nn, cc, x_x, x_y, c, h, w)]);         \
+                                    items = items + 1;                                                   \
+                                }                                                                        \
+                            }                                                                            \
+                    }                                                                                    \
+                    y[NHWC ? IDX4(nn, xx, yy, cc, hh, ww, c) : IDX4(nn, cc, xx, yy, c, hh, ww)] =        \
+                        accum / items;                                                                   \
+                }                                                                                        \
+}                                                                                                        \
+void NAME##_bwd_f32(const float *dy, float *dx, int n, int c, int h, int w, int kh, int kw,             \
+                    int vpadding, int hpadding, int vstride, int hstride, int vdilation, int hdilation) \
+{                                                                                                        \
+    const int hh = out_dim(h, vpadding, vdilation, kh, vstride);                                         \
+    const int ww = out_dim(w, hpadding, hdilation, kw, hstride);                                         \
+    _Pragma("omp parallel for")                                                                          \
+    for (int nn = 0; nn < n; nn++)                                                                       \
+        for (int cc = 0; cc < c; cc++)                                                                   \
+            for (int xx = 0; xx < hh; xx++)                                                              \
+                for (int yy = 0; yy < ww; yy++) {                                                        \
+                    int items = 0;                                                                       \
+                    for (int ii = 0; ii < kh; ii++) {                                                    \
+                        const int x_x = vstride * xx + vdilation * ii - vpadding;                        \
+                        if (0 <= x_x && x_x < h)                                                         \
+                            for (int jj = 0; jj < kw; jj++) {                                            \
+                                const int x_y = hstride * yy + hdilation * jj - hpadding;                \
+                                if (0 <= x_y && x_y < w) items = items + 1;                              \
+                            }                                                                            \
+                    }                                                                                    \
+                    const float avgval =                                                                 \
+                        dy[NHWC ? IDX4(nn, xx, yy, cc, hh, ww, c) : IDX4(nn, cc, xx, yy, c, hh, ww)] / items; \
+                    for (int ii = 0; ii < kh; ii++) {                                                    \
+                        const int x_x = vstride * xx + vdilation * ii - vpadding;                        \
+                        if (0 <= x_x && x_x < h)                                                         \
+                            for (int jj = 0; jj < kw; jj++) {                                            \
+                                const int x_y = hstride * yy + hdilation * jj - hpadding;                \
+                                if (0 <= x_y && x_y < w)                                                 \
+                                    dx[NHWC ? IDX4(nn, x_x, x_y, cc, h, w, c)                            \
+                                            : IDX4(nn, cc, x_x, x_y, c, h, w)] += avgval;                \
+                            }                                                                            \
+                    }                                                                                    \
+                }                                                                                        \
+}
+DEF_AVG_POOL(oracle_average_pool_2d_nchw, 0)
+DEF_AVG_POOL(oracle_average_pool_2d_nhwc, 1)

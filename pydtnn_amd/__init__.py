@@ -5,11 +5,11 @@ Conv2D / FC ``forward()`` / ``backward()`` behind PyDTNN's layer protocol, the N
 kernels (``csrc/``) through a thin C ABI (``include/pydtnn_hip.h``).  There is no CPU fallback:
 importing the layers works anywhere, running them needs the built library and a GPU.
 """
-from .layers import (EVALUATE_MODE, TRAIN_MODE, UNSPECIFIED_MODE, AdditionBlock, BatchNormalization,
+from .layers import (EVALUATE_MODE, TRAIN_MODE, UNSPECIFIED_MODE, AdditionBlock, AveragePool2D, BatchNormalization,
                      BatchNormalizationRelu, Conv2D, Conv2DBatchNormalization, Conv2DBatchNormalizationRelu,
                      Conv2DRelu, Dropout, FC, Flatten, Input, Layer, MaxPool2D, Relu, Softmax)
 from .model import SGD, CategoricalCrossEntropy, Model
-from . import tracers
+from . import models, tracers
 from .best_of import BestOf
 from .conv_gemm import ConvGemm
 from .utils import (PYDTNN_TENSOR_FORMAT_NCHW, PYDTNN_TENSOR_FORMAT_NHWC, decode_tensor, encode_tensor, to_device,

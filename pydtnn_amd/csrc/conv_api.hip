@@ -515,6 +515,28 @@ int pydtnn_hip_max_pool_2d_bwd_nhwc(const float* dy, const int32_t* idx_max, flo
     return rc != PYDTNN_HIP_OK ? rc : launch_max_pool_bwd_nhwc(dy, idx_max, dx, g, as_stream(stream), nullptr);
 }
 
+int pydtnn_hip_average_pool_2d_fwd(int nhwc, const float* x, float* y, int b, int c, int h, int w, int kh, int kw,
+                                   int vpadding, int hpadding, int vstride, int hstride, int vdilation, int hdilation,
+                                   void* stream)
+{
+    if (!x || !y) return PYDTNN_HIP_ERR_INVALID;
+    ConvGeom g;
+    const int kn = 1;
+    const int rc = geom_from_args(&g, GEOM_ARGS);
+    return rc != PYDTNN_HIP_OK ? rc : launch_avg_pool_fwd(nhwc, x, y, g, as_stream(stream));
+}
+
+int pydtnn_hip_average_pool_2d_bwd(int nhwc, const float* dy, float* dx, int b, int c, int h, int w, int kh, int kw,
+                                   int vpadding, int hpadding, int vstride, int hstride, int vdilation, int hdilation,
+                                   void* stream)
+{
+    if (!dy || !dx) return PYDTNN_HIP_ERR_INVALID;
+    ConvGeom g;
+    const int kn = 1;
+    const int rc = geom_from_args(&g, GEOM_ARGS);
+    return rc != PYDTNN_HIP_OK ? rc : launch_avg_pool_bwd(nhwc, dy, dx, g, as_stream(stream));
+}
+
 int pydtnn_hip_max_pool_2d_bwd_gated(int nhwc, const float* dy, const int32_t* idx_max, float* dx, const int8_t* gate,
                                      int b, int c, int h, int w, int kh, int kw, int vpadding, int hpadding,
                                      int vstride, int hstride, int vdilation, int hdilation, void* stream)

@@ -27,6 +27,8 @@ int launch_max_pool_fwd_nchw(const float*, float*, int32_t*, const ConvGeom&, hi
 int launch_max_pool_bwd_nchw(const float*, const int32_t*, float*, const ConvGeom&, hipStream_t, const int8_t* gate);
 int launch_max_pool_fwd_nhwc(const float*, float*, int32_t*, const ConvGeom&, hipStream_t);
 int launch_max_pool_bwd_nhwc(const float*, const int32_t*, float*, const ConvGeom&, hipStream_t, const int8_t* gate);
+int launch_avg_pool_fwd(int nhwc, const float*, float*, const ConvGeom&, hipStream_t);
+int launch_avg_pool_bwd(int nhwc, const float*, float*, const ConvGeom&, hipStream_t);
 int launch_sgd_momentum(float*, const float*, float*, long, float, float, float, int, hipStream_t);
 
 namespace convint {

@@ -600,6 +600,20 @@ class MaxPool2D(Layer):
             return dx
 
 
+class AveragePool2D(MaxPool2D):
+    """pydtnn/layers/abstract_pool_2d_layer.py:28-57 + pydtnn/backends/cpu/layers/average_pool_2d_cpu.py:30-108.
+    ``pool_shape=(0, 0)`` pools each whole plane (global average pooling)."""
+
+    def forward(self, x):
+        nhwc = self.model.tensor_format != PYDTNN_TENSOR_FORMAT_NCHW
+        return ops.average_pool_2d_fwd(x, nhwc, *self._geom())
+
+    def backward(self, dy):
+        if self.need_dx:
+            nhwc = self.model.tensor_format != PYDTNN_TENSOR_FORMAT_NCHW
+            return ops.average_pool_2d_bwd(dy, nhwc, dy.shape[0], self.ci, self.hi, self.wi, *self._geom())
+
+
 class Flatten(Layer):
     """pydtnn/layers/flatten.py:26-30 + pydtnn/backends/cpu/layers/flatten_cpu.py"""
 

@@ -224,19 +224,64 @@ class Model:
 
 
     # ------------------------------------------------------------------ weights on disk (pydtnn/model.py:351-387)
-    def load_store_path(self, layers, d, mode):
-        """Walks the layers (and the paths of block layers) and moves every trainable tensor, plus the
-        running statistics of BatchNormalization, between the layers and the dictionary ``d`` under
-        the reference's key ``"{layer.id}_{canonical_name}_{variable}"``.  Arrays keep the in-memory
-        layout of the model's tensor format, as in the reference."""
+    def _walk_trainable(self, layers, prev=None):
+        """Yields (layer, variable names, layer before it in its sequence) in the reference's order: block
+        layers are entered path by path, and only their children carry variables."""
         for layer in layers:
             name = layer.canonical_name
             if name in ["AdditionBlock", "ConcatenationBlock"]:
                 for path in layer.paths:
-                    self.load_store_path(path, d, mode)
+                    yield from self._walk_trainable(path, prev)
+            else:
+                keys = [g for g in layer.grad_vars] + \
+                       (["running_var", "running_mean"] if name == "BatchNormalization" else [])
+                yield layer, keys, prev
+            prev = layer
+
+    @staticmethod
+    def _file_tensor_format(pairs, d):
+        """The tensor format of the model that wrote ``d``, read off the first convolution whose filter shape
+        tells the two layouts apart ((co,ci,kh,kw) against (ci,kh,kw,co)); None if no filter does."""
+        for layer, keys, _ in pairs:
+            base = f"{layer.id}_{layer.canonical_name}_weights"
+            if layer.canonical_name != "Conv2D" or base not in d:
                 continue
-            keys = [g for g in layer.grad_vars] + \
-                   (["running_var", "running_mean"] if name == "BatchNormalization" else [])
+            co, ci, kh, kw = layer.co, layer.ci, layer.kh, layer.kw
+            nchw, nhwc = (co, ci, kh, kw), (ci, kh, kw, co)
+            if nchw != nhwc and tuple(d[base].shape) in (nchw, nhwc):
+                return "NCHW" if tuple(d[base].shape) == nchw else "NHWC"
+        return None
+
+    def _to_model_format(self, layer, key, ary, prev, file_format):
+        """An array written by a model in ``file_format`` as this model's layout wants it.  Filters go between
+        (ci,kh,kw,co) and (co,ci,kh,kw) as pydtnn/tests/check_tensor_format_models.py:70-71 does
+        (``transpose(3, 0, 1, 2)`` towards NCHW); the rows of an FC layer that follows the Flatten of an image
+        follow the flattening order of that image, (h,w,c) or (c,h,w)."""
+        mine = "NCHW" if self.tensor_format == PYDTNN_TENSOR_FORMAT_NCHW else "NHWC"
+        if file_format is None or file_format == mine or key != "weights":
+            return ary
+        if layer.canonical_name == "Conv2D":
+            return ary.transpose(3, 0, 1, 2) if mine == "NCHW" else ary.transpose(1, 2, 3, 0)
+        if layer.canonical_name == "FC" and prev is not None and prev.canonical_name == "Flatten" and \
+                len(prev.prev_shape) == 3:
+            from .utils import decode_tensor
+            h, w, c = decode_tensor(prev.prev_shape, self.tensor_format)
+            if mine == "NCHW":   # rows (h,w,c) -> (c,h,w)
+                return ary.reshape(h, w, c, -1).transpose(2, 0, 1, 3).reshape(ary.shape)
+            return ary.reshape(c, h, w, -1).transpose(1, 2, 0, 3).reshape(ary.shape)
+        return ary
+
+    def load_store_path(self, layers, d, mode, tensor_format=None):
+        """Moves every trainable tensor, plus the running statistics of BatchNormalization, between the
+        layers and the dictionary ``d`` under the reference's key ``"{layer.id}_{canonical_name}_{variable}"``
+        (block layers are walked path by path).  Stored arrays keep the in-memory layout of the model's
+        tensor format, as in the reference.  On load, ``tensor_format`` names the format of the model that
+        wrote ``d`` when it differs from this model's; without it the format is read off the filter shapes."""
+        pairs = list(self._walk_trainable(layers))
+        if mode == "load" and tensor_format is None:
+            tensor_format = self._file_tensor_format(pairs, d)
+        for layer, keys, prev in pairs:
+            name = layer.canonical_name
             if name == "BatchNormalization":
                 layer.updated_running_var = True
             for key in keys:
@@ -245,14 +290,18 @@ class Model:
                     if base not in d:
                         print(f"Could not find '{base}' for layer '{name}' in file!")
                         continue
-                    ary = np.ascontiguousarray(d[base], dtype=np.float32)
-                    setattr(layer, key, torch.from_numpy(ary).cuda())
+                    ary = self._to_model_format(layer, key, np.asarray(d[base]), prev, tensor_format)
+                    current = getattr(layer, key, None)
+                    if current is not None and tuple(ary.shape) != tuple(current.shape):
+                        raise ValueError(f"'{base}' has shape {tuple(ary.shape)}, the layer expects "
+                                         f"{tuple(current.shape)}")
+                    setattr(layer, key, torch.from_numpy(np.ascontiguousarray(ary, dtype=np.float32)).cuda())
                 elif mode == "store":
                     d[base] = getattr(layer, key).detach().cpu().numpy()
 
-    def load_weights_and_bias(self, filename):
+    def load_weights_and_bias(self, filename, tensor_format=None):
         d = np.load(filename)
-        self.load_store_path(self.layers, d, "load")
+        self.load_store_path(self.layers, d, "load", tensor_format)
 
     def store_weights_and_bias(self, filename):
         d = {}

@@ -58,6 +58,8 @@ SIGNATURES = {
     "pydtnn_hip_max_pool_2d_bwd_nchw": (_c.c_int, [_f32p, _i32p, _f32p] + [_c.c_int] * 12 + [_vp]),
     "pydtnn_hip_max_pool_2d_fwd_nhwc": (_c.c_int, [_f32p, _f32p, _i32p] + [_c.c_int] * 12 + [_vp]),
     "pydtnn_hip_max_pool_2d_bwd_nhwc": (_c.c_int, [_f32p, _i32p, _f32p] + [_c.c_int] * 12 + [_vp]),
+    "pydtnn_hip_average_pool_2d_fwd": (_c.c_int, [_c.c_int, _f32p, _f32p] + [_c.c_int] * 12 + [_vp]),
+    "pydtnn_hip_average_pool_2d_bwd": (_c.c_int, [_c.c_int, _f32p, _f32p] + [_c.c_int] * 12 + [_vp]),
     "pydtnn_hip_bn_training_workspace_bytes": (_c.c_size_t, [_c.c_int]),
     "pydtnn_hip_bn_training_fwd": (_c.c_int, [_f32p] * 8 + [_c.c_double, _c.c_double, _c.c_long, _c.c_int, _c.c_int,
                                                         _vp, _c.c_size_t, _vp]),

@@ -189,6 +189,26 @@ def bias_grad(dy, channels, inner):
     return db
 
 
+def average_pool_2d_fwd(x, nhwc, kh, kw, vpadding, hpadding, vstride, hstride, vdilation=1, hdilation=1):
+    """pydtnn/cython_modules/average_pool_2d_nchw_cython.pyx:25-52 / average_pool_2d_nhwc_cython.pyx:25-52"""
+    _need_f32(x)
+    n, c, h, w = (x.shape[0], x.shape[3], x.shape[1], x.shape[2]) if nhwc else x.shape
+    hh, ww = _out_hw(h, w, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
+    y = torch.empty((n, hh, ww, c) if nhwc else (n, c, hh, ww), dtype=x.dtype, device=x.device)
+    check(lib().pydtnn_hip_average_pool_2d_fwd(int(nhwc), f32(x), f32(y), n, c, h, w, kh, kw, vpadding, hpadding,
+                                               vstride, hstride, vdilation, hdilation, stream_ptr()), "avg_pool_fwd")
+    return y
+
+
+def average_pool_2d_bwd(dy, nhwc, n, c, h, w, kh, kw, vpadding, hpadding, vstride, hstride, vdilation=1, hdilation=1):
+    """pydtnn/cython_modules/average_pool_2d_nchw_cython.pyx:135-160 / average_pool_2d_nhwc_cython.pyx:135-160"""
+    _need_f32(dy)
+    dx = torch.empty((n, h, w, c) if nhwc else (n, c, h, w), dtype=dy.dtype, device=dy.device)
+    check(lib().pydtnn_hip_average_pool_2d_bwd(int(nhwc), f32(dy), f32(dx), n, c, h, w, kh, kw, vpadding, hpadding,
+                                               vstride, hstride, vdilation, hdilation, stream_ptr()), "avg_pool_bwd")
+    return dx
+
+
 def max_pool_2d_fwd_nchw(x, kh, kw, vpadding, hpadding, vstride, hstride, vdilation=1, hdilation=1):
     """pydtnn/cython_modules/max_pool_2d_nchw_cython.pyx:25-52 -> (y, idx_max int32)"""
     _need_f32(x)

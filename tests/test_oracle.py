@@ -465,6 +465,77 @@ def test_maxpool_nhwc_is_the_nchw_pool_in_the_other_layout(oracle):
         assert np.array_equal(dxh, dx.transpose(0, 2, 3, 1))
 
 
+POOL_GEOMS = [  # (n, c, h, w, kh, kw, pv, ph, sv, sh, dv, dh)
+    (2, 3, 8, 10, 2, 2, 0, 0, 2, 2, 1, 1),
+    (2, 4, 9, 9, 3, 3, 1, 1, 2, 2, 1, 1),      # ResNet's 3x3 / stride 2 / pad 1
+    (1, 5, 7, 11, 3, 2, 1, 0, 1, 2, 1, 1),     # rectangular window, padding on one axis, mixed strides
+    (1, 2, 9, 9, 2, 2, 1, 1, 1, 1, 2, 2),      # dilated
+    (2, 3, 12, 12, 3, 3, 1, 1, 1, 1, 1, 1),    # overlapping windows at stride 1
+]
+
+
+@pytest.mark.parametrize("geom", POOL_GEOMS, ids=str)
+def test_maxpool_padded_strided_dilated_against_torch(oracle, geom):
+    """torch.nn.functional.max_pool2d pads with -inf, i.e. ignores padding taps like the reference's bound
+    tests; distinct random values leave no ties, so values and gradients must agree exactly.  Square windows
+    only go through backward: the reference decodes the stored index with kh where kw belongs."""
+    n, c, h, w, kh, kw, pv, ph, sv, sh, dv, dh = geom
+    rng = np.random.default_rng(21)
+    x = rng.permutation(n * c * h * w).astype(np.float32).reshape(n, c, h, w) / 7.0
+    y, idx = oracle.max_pool_2d_fwd_nchw(x, kh, kw, pv, ph, sv, sh, dv, dh)
+    xt = torch.from_numpy(x).requires_grad_(True)
+    yt = F.max_pool2d(xt, (kh, kw), (sv, sh), (pv, ph), (dv, dh))
+    assert np.array_equal(y, yt.detach().numpy())
+    if kh == kw:
+        dy = rng.standard_normal(y.shape).astype(np.float32)
+        yt.backward(torch.from_numpy(dy))
+        dx = oracle.max_pool_2d_bwd_nchw(dy, idx, n, c, h, w, kh, kw, pv, ph, sv, sh, dv, dh)
+        np.testing.assert_allclose(dx, xt.grad.numpy(), rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("fmt", ["NCHW", "NHWC"])
+@pytest.mark.parametrize("geom", [g for g in POOL_GEOMS if g[10] == 1 and g[11] == 1] + [(2, 6, 7, 7, 0, 0, 0, 0, 1, 1, 1, 1)],
+                         ids=str)
+def test_average_pool_against_torch(oracle, fmt, geom):
+    """avg_pool2d(count_include_pad=False) divides by the taps inside the image, as the reference does; the
+    last geometry is the global pooling of a 7x7 plane (pool_shape (0, 0))."""
+    n, c, h, w, kh, kw, pv, ph, sv, sh, dv, dh = geom
+    rng = np.random.default_rng(22)
+    x = rng.standard_normal((n, c, h, w))
+    xt = torch.from_numpy(x).requires_grad_(True)
+    yt = F.avg_pool2d(xt, (kh or h, kw or w), (sv, sh), (pv, ph), count_include_pad=False)
+    dy = rng.standard_normal(tuple(yt.shape))
+    yt.backward(torch.from_numpy(dy))
+    to_fmt = (lambda a: a) if fmt == "NCHW" else (lambda a: np.ascontiguousarray(a.transpose(0, 2, 3, 1)))
+    y = oracle.average_pool_2d_fwd(to_fmt(x.astype(np.float32)), fmt, kh, kw, pv, ph, sv, sh)
+    dx = oracle.average_pool_2d_bwd(to_fmt(dy.astype(np.float32)), fmt, n, c, h, w, kh, kw, pv, ph, sv, sh)
+    np.testing.assert_allclose(y, to_fmt(yt.detach().numpy()), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(dx, to_fmt(xt.grad.numpy()), rtol=1e-5, atol=1e-6)
+
+
+def test_average_pool_closed_forms(oracle):
+    # ones stay ones whatever the padding (the divisor counts inside taps only) ...
+    y = oracle.average_pool_2d_fwd(np.ones((1, 2, 5, 5), np.float32), "NCHW", 3, 3, 1, 1, 2, 2)
+    assert np.array_equal(y, np.ones_like(y))
+    # ... and backward of ones is the sum over covering windows of 1 / (taps inside): corner of a 3x3 / pad 1 /
+    # stride 1 pooling of a 3x3 image is covered by the windows at (0,0) [4 taps], (0,1), (1,0) [6] and (1,1) [9]
+    dx = oracle.average_pool_2d_bwd(np.ones((1, 1, 3, 3), np.float32), "NCHW", 1, 1, 3, 3, 3, 3, 1, 1, 1, 1)
+    assert abs(dx[0, 0, 0, 0] - (1 / 4 + 2 / 6 + 1 / 9)) < 1e-6
+
+
+def test_sgd_decay_and_nesterov_closed_forms(oracle):
+    """pydtnn/backends/cpu/optimizers/sgd_cpu.py:28-41 with every term switched on, by hand:
+    v' = m v + g;  plain: w' = w - lr (d w + v');  nesterov: w' = w - lr (d w + g + m v')."""
+    w0, g, v0, lr, m, d = 2.0, 0.5, 1.0, 0.1, 0.9, 0.01
+    w, v = oracle.sgd_update(np.array([w0]), np.array([g]), np.array([v0]), lr=lr, momentum=m, decay=d)
+    assert np.allclose(v, 1.4) and np.allclose(w, 2.0 - 0.1 * (0.02 + 1.4))
+    w, v = oracle.sgd_update(np.array([w0]), np.array([g]), np.array([v0]), lr=lr, momentum=m, decay=d, nesterov=True)
+    assert np.allclose(v, 1.4) and np.allclose(w, 2.0 - 0.1 * (0.02 + 0.5 + 0.9 * 1.4))
+    # decay alone shrinks the weight geometrically when there is no gradient and no momentum
+    w, v = oracle.sgd_update(np.array([3.0]), np.array([0.0]), np.array([0.0]), lr=0.5, momentum=0.0, decay=0.2)
+    assert np.allclose(w, 3.0 * (1 - 0.5 * 0.2))
+
+
 # ------------------------------------------------------------------ larger library cross-check
 
 @pytest.mark.parametrize("layer", [0, 1, 4, 7], ids=lambda i: f"alexnet{i}")
