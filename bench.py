@@ -220,6 +220,7 @@ def run_cfg2(torch, pd, args):
     extra["epilogue_gbs"] = round(2 * x.nbytes / (t3.median_ms() * 1e-3) / 1e9, 1)
     extra["epilogue_pct_hbm_peak"] = round(100 * extra["epilogue_gbs"] / HBM_PEAK_GBS, 1)
     del mat, back
+    extra.update(compat_route(x, w, b, gemm_flop))
     roofline = {"bound": "mfma", "kernel": "gemm_streamk_kernel_big_tile<256x128, PlainK4, Im2colNchwMN, EpiNchw> + streamk_fixup_kernel (forward)",
                 "achieved": round(achieved, 3), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES["cfg2"],
@@ -227,6 +228,40 @@ def run_cfg2(torch, pd, args):
     workload = ("cfg2: VGG16-style 3x3 conv layer fwd+dW+db+dX, fp32 NCHW, N=64, 256->256, 56x56, stride 1, pad 1, "
                 "implicit GEMM")
     return ms, step_flop / (ms * 1e-3) / 1e9, workload, roofline, extra
+
+
+def compat_route(x, w, b, gemm_flop, reps=3):
+    """cfg2's forward through libconvGemm.so with host pointers, exactly as the reference's shim calls it
+    (pydtnn/backends/cpu/libs/conv_gemm.py:191-205): 205 MB in and 205 MB out over PCIe per call, so the rate
+    is that of the copies.  Reported beside the device-resident numbers, never as `value`."""
+    import ctypes
+    import numpy as np
+    from pydtnn_amd import native
+    lib = ctypes.CDLL(native.COMPAT_LIB_PATH)
+    ac, bc = ctypes.POINTER(ctypes.c_float)(), ctypes.POINTER(ctypes.c_float)()
+    lib.alloc_pack_buffs.restype = ctypes.c_int
+    if lib.alloc_pack_buffs(ctypes.byref(ac), ctypes.byref(bc)) != 0:
+        return {}
+    n, c, h, wd = x.shape
+    y = np.empty((n, 256, h, wd), np.float32)
+    u, vp, none = ctypes.c_uint, (lambda a: ctypes.c_void_p(a.ctypes.data)), ctypes.c_void_p(None)
+
+    def call():
+        lib.sconvGemmNCHW(ctypes.c_char(b'N'), u(n), u(c), u(h), u(wd), u(256), u(3), u(3), u(1), u(1), u(1), u(1),
+                          u(1), u(1), vp(w), vp(x), vp(y), vp(b), none, none, none, none, ctypes.c_bool(False), ac, bc)
+
+    call()  # allocates the library's device buffers
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        call()
+        times.append(time.perf_counter() - t0)
+    libc = ctypes.CDLL("libc.so.6")
+    libc.free(ac)
+    libc.free(bc)
+    best = min(times)
+    return {"compat_hostptr_fwd_ms": round(best * 1e3, 2), "compat_hostptr_fwd_tflops": round(gemm_flop / best / 1e12, 2),
+            "compat_hostptr_pcie_gbs": round((x.nbytes + y.nbytes) / best / 1e9, 1)}
 
 
 def cpu_baseline_cfg2(sample_images=64, reps=30):

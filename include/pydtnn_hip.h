@@ -42,10 +42,7 @@ int pydtnn_hip_version(void);
 const char *pydtnn_hip_status_string(int status);
 /* One launch addresses a tensor with 32-bit byte offsets: at most 2^29 floats.  The implicit
  * convolution entry points (sconvGemm*, *_back) run a larger batch as consecutive groups of whole
- * images, each below that limit; the filter gradient is summed over the groups in order.  For tests
- * only: lowers the limit (1 .. 2^29 floats) so that small tensors take that route; returns the
- * previous value.  Process-wide, not synchronised with running calls. */
-long pydtnn_hip_debug_set_tensor_floats_limit(long floats);
+ * images, each below that limit; the filter gradient is summed over the groups in order. */
 
 /* ------------------------------------------------------------------------------------------
  * Explicit im2col / col2im.  Replace the Cython modules

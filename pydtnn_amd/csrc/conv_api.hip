@@ -1,6 +1,7 @@
 // Device-pointer C ABI: argument checks, batching over image groups, and the launches that are not
 // convolutions (GEMM, explicit-path GEMMs, streaming kernels).
 #include "conv_internal.h"
+#include "../../include/pydtnn_hip_test.h"
 #include <mutex>
 
 namespace {
@@ -218,6 +219,29 @@ int static_scratch_address(void** out)
     *out = g_scratch_address[dev];
     return PYDTNN_HIP_OK;
 }
+
+// Pooling layers work plane by plane, so a batch whose tensors exceed the addressing limit of one launch runs
+// as consecutive groups of whole images, like the convolutions.  `launch(geometry of the group, first image)`.
+template <class Launch>
+int pool_batched(long b, long c, long h, long w, long kh, long kw, long vpadding, long hpadding, long vstride,
+                 long hstride, long vdilation, long hdilation, Launch launch)
+{
+    ImageGroups ig;
+    const long kn = c;  // the output has the input's channels
+    int rc = plan_image_groups(&ig, GEOM_ARGS);
+    if (rc != PYDTNN_HIP_OK) return rc;
+    for (long n0 = 0; n0 < b; n0 += ig.images) {
+        ConvGeom g;
+        const long nb = b - n0 < ig.images ? b - n0 : ig.images;
+        rc = geom_from_args(&g, nb, c, h, w, 1, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation);
+        if (rc != PYDTNN_HIP_OK) return rc;
+        rc = launch(g, n0 * ig.per_image_in, n0 * ig.per_image_out);
+        if (rc != PYDTNN_HIP_OK) return rc;
+    }
+    return PYDTNN_HIP_OK;
+}
+
+#define POOL_ARGS b, c, h, w, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation
 
 }  // namespace
 
@@ -476,10 +500,9 @@ int pydtnn_hip_max_pool_2d_fwd_nchw(const float* x, float* y, int32_t* idx_max, 
                                     int hdilation, void* stream)
 {
     if (!x || !y || !idx_max) return PYDTNN_HIP_ERR_INVALID;
-    ConvGeom g;
-    const int kn = 1;
-    const int rc = geom_from_args(&g, GEOM_ARGS);
-    return rc != PYDTNN_HIP_OK ? rc : launch_max_pool_fwd_nchw(x, y, idx_max, g, as_stream(stream));
+    return pool_batched(POOL_ARGS, [&](const ConvGeom& g, long in0, long out0) {
+        return launch_max_pool_fwd_nchw(x + in0, y + out0, idx_max + out0, g, as_stream(stream));
+    });
 }
 
 int pydtnn_hip_max_pool_2d_bwd_nchw(const float* dy, const int32_t* idx_max, float* dx, int b, int c, int h, int w,
@@ -487,10 +510,9 @@ int pydtnn_hip_max_pool_2d_bwd_nchw(const float* dy, const int32_t* idx_max, flo
                                     int vdilation, int hdilation, void* stream)
 {
     if (!dy || !dx || !idx_max) return PYDTNN_HIP_ERR_INVALID;
-    ConvGeom g;
-    const int kn = 1;
-    const int rc = geom_from_args(&g, GEOM_ARGS);
-    return rc != PYDTNN_HIP_OK ? rc : launch_max_pool_bwd_nchw(dy, idx_max, dx, g, as_stream(stream), nullptr);
+    return pool_batched(POOL_ARGS, [&](const ConvGeom& g, long in0, long out0) {
+        return launch_max_pool_bwd_nchw(dy + out0, idx_max + out0, dx + in0, g, as_stream(stream), nullptr);
+    });
 }
 
 int pydtnn_hip_max_pool_2d_fwd_nhwc(const float* x, float* y, int32_t* idx_max, int b, int h, int w, int c, int kh,
@@ -498,10 +520,9 @@ int pydtnn_hip_max_pool_2d_fwd_nhwc(const float* x, float* y, int32_t* idx_max, 
                                     int hdilation, void* stream)
 {
     if (!x || !y || !idx_max) return PYDTNN_HIP_ERR_INVALID;
-    ConvGeom g;
-    const int kn = 1;
-    const int rc = geom_from_args(&g, GEOM_ARGS);
-    return rc != PYDTNN_HIP_OK ? rc : launch_max_pool_fwd_nhwc(x, y, idx_max, g, as_stream(stream));
+    return pool_batched(POOL_ARGS, [&](const ConvGeom& g, long in0, long out0) {
+        return launch_max_pool_fwd_nhwc(x + in0, y + out0, idx_max + out0, g, as_stream(stream));
+    });
 }
 
 int pydtnn_hip_max_pool_2d_bwd_nhwc(const float* dy, const int32_t* idx_max, float* dx, int b, int h, int w, int c,
@@ -509,10 +530,9 @@ int pydtnn_hip_max_pool_2d_bwd_nhwc(const float* dy, const int32_t* idx_max, flo
                                     int vdilation, int hdilation, void* stream)
 {
     if (!dy || !dx || !idx_max) return PYDTNN_HIP_ERR_INVALID;
-    ConvGeom g;
-    const int kn = 1;
-    const int rc = geom_from_args(&g, GEOM_ARGS);
-    return rc != PYDTNN_HIP_OK ? rc : launch_max_pool_bwd_nhwc(dy, idx_max, dx, g, as_stream(stream), nullptr);
+    return pool_batched(POOL_ARGS, [&](const ConvGeom& g, long in0, long out0) {
+        return launch_max_pool_bwd_nhwc(dy + out0, idx_max + out0, dx + in0, g, as_stream(stream), nullptr);
+    });
 }
 
 int pydtnn_hip_average_pool_2d_fwd(int nhwc, const float* x, float* y, int b, int c, int h, int w, int kh, int kw,
@@ -520,10 +540,9 @@ int pydtnn_hip_average_pool_2d_fwd(int nhwc, const float* x, float* y, int b, in
                                    void* stream)
 {
     if (!x || !y) return PYDTNN_HIP_ERR_INVALID;
-    ConvGeom g;
-    const int kn = 1;
-    const int rc = geom_from_args(&g, GEOM_ARGS);
-    return rc != PYDTNN_HIP_OK ? rc : launch_avg_pool_fwd(nhwc, x, y, g, as_stream(stream));
+    return pool_batched(POOL_ARGS, [&](const ConvGeom& g, long in0, long out0) {
+        return launch_avg_pool_fwd(nhwc, x + in0, y + out0, g, as_stream(stream));
+    });
 }
 
 int pydtnn_hip_average_pool_2d_bwd(int nhwc, const float* dy, float* dx, int b, int c, int h, int w, int kh, int kw,
@@ -531,10 +550,9 @@ int pydtnn_hip_average_pool_2d_bwd(int nhwc, const float* dy, float* dx, int b, 
                                    void* stream)
 {
     if (!dy || !dx) return PYDTNN_HIP_ERR_INVALID;
-    ConvGeom g;
-    const int kn = 1;
-    const int rc = geom_from_args(&g, GEOM_ARGS);
-    return rc != PYDTNN_HIP_OK ? rc : launch_avg_pool_bwd(nhwc, dy, dx, g, as_stream(stream));
+    return pool_batched(POOL_ARGS, [&](const ConvGeom& g, long in0, long out0) {
+        return launch_avg_pool_bwd(nhwc, dy + out0, dx + in0, g, as_stream(stream));
+    });
 }
 
 int pydtnn_hip_max_pool_2d_bwd_gated(int nhwc, const float* dy, const int32_t* idx_max, float* dx, const int8_t* gate,
@@ -542,12 +560,10 @@ int pydtnn_hip_max_pool_2d_bwd_gated(int nhwc, const float* dy, const int32_t* i
                                      int vstride, int hstride, int vdilation, int hdilation, void* stream)
 {
     if (!dy || !dx || !idx_max || !gate) return PYDTNN_HIP_ERR_INVALID;
-    ConvGeom g;
-    const int kn = 1;
-    const int rc = geom_from_args(&g, GEOM_ARGS);
-    if (rc != PYDTNN_HIP_OK) return rc;
-    return nhwc ? launch_max_pool_bwd_nhwc(dy, idx_max, dx, g, as_stream(stream), gate)
-                : launch_max_pool_bwd_nchw(dy, idx_max, dx, g, as_stream(stream), gate);
+    return pool_batched(POOL_ARGS, [&](const ConvGeom& g, long in0, long out0) {
+        return nhwc ? launch_max_pool_bwd_nhwc(dy + out0, idx_max + out0, dx + in0, g, as_stream(stream), gate + in0)
+                    : launch_max_pool_bwd_nchw(dy + out0, idx_max + out0, dx + in0, g, as_stream(stream), gate + in0);
+    });
 }
 
 int pydtnn_hip_sconvGemm_relu_mask(int nhwc, unsigned b, unsigned c, unsigned h, unsigned w, unsigned kn, unsigned kh,

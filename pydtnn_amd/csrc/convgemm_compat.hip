@@ -1,11 +1,14 @@
 // Host-pointer flavour of the convolution entry points, with the names and signatures of the
 // external libconvGemm that PyDTNN binds through ctypes
 // (pydtnn/backends/cpu/libs/conv_gemm.py:85-107).  Operands are copied to the GPU, the
-// device-pointer entry points do the work, and the result is copied back.
+// device-pointer entry points do the work, and the result is copied back.  The reference's ABI has no error
+// channel (void functions): a failure is reported on stderr and the process aborts instead of continuing with
+// numbers that were never computed.
 #include "../../include/pydtnn_hip.h"
 #include <hip/hip_runtime.h>
 #include <stdio.h>
 #include <stdlib.h>
+#include <mutex>
 
 namespace {
 
@@ -25,29 +28,52 @@ void check_rc(int rc, const char* what)
     if (rc != PYDTNN_HIP_OK) die(what, pydtnn_hip_status_string(rc));
 }
 
-struct DeviceBuf {
-    void* p = nullptr;
-    size_t bytes = 0;
-    explicit DeviceBuf(size_t n) : bytes(n)
-    {
-        if (n) check_hip(hipMalloc(&p, n), "hipMalloc");
-    }
-    ~DeviceBuf()
-    {
-        if (p) (void)hipFree(p);
-    }
-    float* f() const { return static_cast<float*>(p); }
-    void upload(const void* src) const
-    {
-        if (src && bytes) check_hip(hipMemcpy(p, src, bytes, hipMemcpyHostToDevice), "hipMemcpy H2D");
-    }
-    void download(void* dst) const
-    {
-        if (dst && bytes) check_hip(hipMemcpy(dst, p, bytes, hipMemcpyDeviceToHost), "hipMemcpy D2H");
-    }
-    DeviceBuf(const DeviceBuf&) = delete;
-    DeviceBuf& operator=(const DeviceBuf&) = delete;
+// Device buffers live in a grow-only cache, one slot per role, kept for the life of the process: a layer
+// calls with the same shapes again and again, and a hipMalloc / hipFree pair per operand and call costs more
+// than a small kernel.  The slots are never freed explicitly (at process exit the HIP runtime may already be
+// gone when static destructors run; the driver reclaims the memory).  One call at a time: the reference calls
+// from a single thread, but ctypes releases the GIL, so a mutex keeps two callers from sharing the slots.
+enum Slot { SLOT_IN1, SLOT_X, SLOT_OUT, SLOT_WS, SLOT_BIAS, SLOT_MEAN, SLOT_ISTD, SLOT_GAMMA, SLOT_BETA, SLOT_COUNT };
+
+struct Cache {
+    void* p[SLOT_COUNT] = {};
+    size_t bytes[SLOT_COUNT] = {};
+    int device = -1;
+    std::mutex lock;
 };
+Cache g_cache;
+
+void* slot(Slot s, size_t n)
+{
+    if (n == 0) return nullptr;
+    int dev = 0;
+    check_hip(hipGetDevice(&dev), "hipGetDevice");
+    if (dev != g_cache.device) {  // buffers belong to the device they were allocated on
+        for (int i = 0; i < SLOT_COUNT; ++i) {
+            if (g_cache.p[i]) (void)hipFree(g_cache.p[i]);
+            g_cache.p[i] = nullptr;
+            g_cache.bytes[i] = 0;
+        }
+        g_cache.device = dev;
+    }
+    if (g_cache.bytes[s] < n) {
+        if (g_cache.p[s]) check_hip(hipFree(g_cache.p[s]), "hipFree");
+        g_cache.p[s] = nullptr;
+        g_cache.bytes[s] = 0;
+        const size_t want = n + n / 8;  // a little head room: batch sizes wobble
+        check_hip(hipMalloc(&g_cache.p[s], want), "hipMalloc");
+        g_cache.bytes[s] = want;
+    }
+    return g_cache.p[s];
+}
+
+float* upload(Slot s, const void* src, size_t n)
+{
+    if (!src || n == 0) return nullptr;
+    void* d = slot(s, n);
+    check_hip(hipMemcpy(d, src, n, hipMemcpyHostToDevice), "hipMemcpy H2D");
+    return static_cast<float*>(d);
+}
 
 inline unsigned out_dim(unsigned in, unsigned pad, unsigned dil, unsigned k, unsigned stride)
 {
@@ -63,34 +89,34 @@ void conv_host(int nhwc, char trans, unsigned b, unsigned c, unsigned h, unsigne
     const size_t ho = out_dim(h, vpadding, vdilation, kh, vstride), wo = out_dim(w, hpadding, hdilation, kw, hstride);
     const size_t x_elems = (size_t)b * c * h * w, y_elems = (size_t)b * kn * ho * wo, w_elems = (size_t)kn * c * kh * kw;
     const bool fwd = trans == 'N';
-    DeviceBuf d_in1((fwd ? w_elems : y_elems) * 4), d_x(x_elems * 4), d_out((fwd ? y_elems : w_elems) * 4);
-    d_in1.upload(in1);
-    d_x.upload(x);
+    std::lock_guard<std::mutex> hold(g_cache.lock);
+    float* d_in1 = upload(SLOT_IN1, in1, (fwd ? w_elems : y_elems) * 4);
+    float* d_x = upload(SLOT_X, x, x_elems * 4);
+    const size_t out_bytes = (fwd ? y_elems : w_elems) * 4;
+    float* d_out = static_cast<float*>(slot(SLOT_OUT, out_bytes));
     const size_t vec = (size_t)kn * 4;
-    DeviceBuf d_bias(bias_vector ? vec : 0), d_mean(mean ? vec : 0), d_istd(inv_std ? vec : 0),
-        d_gamma(gamma ? vec : 0), d_beta(beta ? vec : 0);
-    d_bias.upload(bias_vector);
-    d_mean.upload(mean);
-    d_istd.upload(inv_std);
-    d_gamma.upload(gamma);
-    d_beta.upload(beta);
-    const size_t ws_bytes =
-        fwd ? 0
-            : pydtnn_hip_conv_workspace_bytes(PYDTNN_HIP_OP_DW, nhwc, b, c, h, w, kn, kh, kw, vpadding, hpadding,
-                                              vstride, hstride, vdilation, hdilation);
-    DeviceBuf d_ws(ws_bytes);
+    float* d_bias = upload(SLOT_BIAS, bias_vector, vec);
+    float* d_mean = upload(SLOT_MEAN, mean, vec);
+    float* d_istd = upload(SLOT_ISTD, inv_std, vec);
+    float* d_gamma = upload(SLOT_GAMMA, gamma, vec);
+    float* d_beta = upload(SLOT_BETA, beta, vec);
+    // forward: the optional workspace that balances the launch; filter gradient: the partial sums of its split
+    const size_t ws_bytes = pydtnn_hip_conv_workspace_bytes(fwd ? PYDTNN_HIP_OP_FWD : PYDTNN_HIP_OP_DW, nhwc, b, c, h, w,
+                                                            kn, kh, kw, vpadding, hpadding, vstride, hstride,
+                                                            vdilation, hdilation);
+    void* d_ws = slot(SLOT_WS, ws_bytes);
     int rc;
     if (nhwc)
         rc = pydtnn_hip_sconvGemmNHWC(trans, b, h, w, c, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation,
-                                      hdilation, d_in1.f(), d_x.f(), d_out.f(), d_bias.f(), d_mean.f(), d_istd.f(),
-                                      d_gamma.f(), d_beta.f(), relu, d_ws.p, ws_bytes, nullptr);
+                                      hdilation, d_in1, d_x, d_out, d_bias, d_mean, d_istd, d_gamma, d_beta, relu,
+                                      d_ws, ws_bytes, nullptr);
     else
         rc = pydtnn_hip_sconvGemmNCHW(trans, b, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation,
-                                      hdilation, d_in1.f(), d_x.f(), d_out.f(), d_bias.f(), d_mean.f(), d_istd.f(),
-                                      d_gamma.f(), d_beta.f(), relu, d_ws.p, ws_bytes, nullptr);
+                                      hdilation, d_in1, d_x, d_out, d_bias, d_mean, d_istd, d_gamma, d_beta, relu,
+                                      d_ws, ws_bytes, nullptr);
     check_rc(rc, nhwc ? "sconvGemmNHWC" : "sconvGemmNCHW");
-    check_hip(hipDeviceSynchronize(), "kernel execution");
-    d_out.download(out);
+    // the copy back is ordered after the kernels on the null stream and returns when the data is on the host
+    check_hip(hipMemcpy(out, d_out, out_bytes, hipMemcpyDeviceToHost), "hipMemcpy D2H");
 }
 
 void deconv_host(int nhwc, unsigned b, unsigned c, unsigned h, unsigned w, unsigned kn, unsigned kh, unsigned kw,
@@ -99,22 +125,22 @@ void deconv_host(int nhwc, unsigned b, unsigned c, unsigned h, unsigned w, unsig
 {
     const size_t ho = out_dim(h, vpadding, vdilation, kh, vstride), wo = out_dim(w, hpadding, hdilation, kw, hstride);
     const size_t x_elems = (size_t)b * c * h * w, y_elems = (size_t)b * kn * ho * wo, w_elems = (size_t)kn * c * kh * kw;
-    DeviceBuf d_w(w_elems * 4), d_dy(y_elems * 4), d_dx(x_elems * 4);
-    d_w.upload(weights);
-    d_dy.upload(dy);
+    std::lock_guard<std::mutex> hold(g_cache.lock);
+    float* d_w = upload(SLOT_IN1, weights, w_elems * 4);
+    float* d_dy = upload(SLOT_X, dy, y_elems * 4);
+    float* d_dx = static_cast<float*>(slot(SLOT_OUT, x_elems * 4));
     const size_t ws_bytes = pydtnn_hip_conv_workspace_bytes(PYDTNN_HIP_OP_DX, nhwc, b, c, h, w, kn, kh, kw, vpadding,
                                                             hpadding, vstride, hstride, vdilation, hdilation);
-    DeviceBuf d_ws(ws_bytes);
+    void* d_ws = slot(SLOT_WS, ws_bytes);
     int rc;
     if (nhwc)
         rc = pydtnn_hip_sconvGemmNHWC_back(b, h, w, c, kn, kh, kw, vstride, hstride, vpadding, hpadding, vdilation,
-                                           hdilation, d_w.f(), d_dy.f(), d_dx.f(), d_ws.p, ws_bytes, nullptr);
+                                           hdilation, d_w, d_dy, d_dx, d_ws, ws_bytes, nullptr);
     else
         rc = pydtnn_hip_sconvGemmNCHW_back(b, c, h, w, kn, kh, kw, vstride, hstride, vpadding, hpadding, vdilation,
-                                           hdilation, d_w.f(), d_dy.f(), d_dx.f(), d_ws.p, ws_bytes, nullptr);
+                                           hdilation, d_w, d_dy, d_dx, d_ws, ws_bytes, nullptr);
     check_rc(rc, nhwc ? "sconvGemmNHWC_back" : "sconvGemmNCHW_back");
-    check_hip(hipDeviceSynchronize(), "kernel execution");
-    d_dx.download(dx);
+    check_hip(hipMemcpy(dx, d_dx, x_elems * 4, hipMemcpyDeviceToHost), "hipMemcpy D2H");
 }
 
 }  // namespace

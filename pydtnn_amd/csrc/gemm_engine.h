@@ -37,6 +37,7 @@
 // along k spread over all banks, and loaders whose lanes run along m / n store two rows at once.
 #pragma once
 #include "common.h"
+#include <atomic>
 
 namespace gemm {
 
@@ -1640,21 +1641,27 @@ inline hipError_t streamk_blocks_per_cu(int* per_cu)
                                                             kThreads, 0);
 }
 
+// Asked from the runtime once per device and kernel; the answer is two ints, so a race between two first
+// callers only repeats the query.
 template <class T, class AL, class BL, class EP>
 inline Residency resident_workgroups()
 {
-    static Residency cached = {0, 0};
-    if (cached.workgroups == 0) {
-        int dev = 0, cus = 0, per_cu = 0;
-        if (hipGetDevice(&dev) != hipSuccess ||
-            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-            streamk_blocks_per_cu<T, AL, BL, EP>(&per_cu) != hipSuccess ||
-            cus <= 0 || per_cu <= 0)
-            return cached;
-        cached.workgroups = cus * per_cu;
-        cached.cus = cus;
+    constexpr int kDevices = 64;
+    static std::atomic<int> workgroups[kDevices], compute_units[kDevices];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kDevices) return Residency{0, 0};
+    Residency r = {workgroups[dev].load(std::memory_order_acquire), compute_units[dev].load(std::memory_order_relaxed)};
+    if (r.workgroups == 0) {
+        int cus = 0, per_cu = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+            streamk_blocks_per_cu<T, AL, BL, EP>(&per_cu) != hipSuccess || cus <= 0 || per_cu <= 0)
+            return Residency{0, 0};
+        r.workgroups = cus * per_cu;
+        r.cus = cus;
+        compute_units[dev].store(cus, std::memory_order_relaxed);
+        workgroups[dev].store(r.workgroups, std::memory_order_release);
     }
-    return cached;
+    return r;
 }
 
 inline size_t streamk_workspace_bytes(int resident, int bm, int bn) { return (size_t)2 * resident * bm * bn * 4; }

@@ -25,7 +25,7 @@ _geom13_u = [_c.c_uint] * 13
 SIGNATURES = {
     "pydtnn_hip_version": (_c.c_int, []),
     "pydtnn_hip_status_string": (_c.c_char_p, [_c.c_int]),
-    "pydtnn_hip_debug_set_tensor_floats_limit": (_c.c_long, [_c.c_long]),
+    "pydtnn_hip_debug_set_tensor_floats_limit": (_c.c_long, [_c.c_long]),  # test-only (include/pydtnn_hip_test.h)
     "pydtnn_hip_im2col_nchw": (_c.c_int, [_f32p, _f32p] + [_c.c_int] * 12 + [_vp]),
     "pydtnn_hip_col2im_nchw": (_c.c_int, [_f32p, _f32p] + [_c.c_int] * 12 + [_vp]),
     "pydtnn_hip_im2row_nhwc": (_c.c_int, [_f32p, _f32p] + [_c.c_int] * 12 + [_vp]),
@@ -130,8 +130,10 @@ def f32(t, name="tensor"):
 
 
 # --------------------------------------------------------------------------- workspace
-# One grow-only scratch buffer per device.  All work is enqueued on the caller's current stream,
-# so consecutive calls use it strictly one after the other.
+# One grow-only scratch buffer per (device, stream): work is enqueued on the caller's current stream, so
+# consecutive calls on a stream use its buffer strictly one after the other, and calls on different streams
+# never share one.  A buffer that is outgrown is released to torch's caching allocator, which keeps a block
+# away from other streams until the work queued on its own stream has passed.
 _WORKSPACE = {}
 
 
@@ -140,13 +142,14 @@ def workspace(nbytes):
     if nbytes == 0:
         return None, 0
     dev = torch.cuda.current_device()
-    buf = _WORKSPACE.get(dev)
+    key = (dev, torch.cuda.current_stream().cuda_stream)
+    buf = _WORKSPACE.get(key)
     if buf is None or buf.numel() < nbytes:
         if buf is not None:
-            del _WORKSPACE[dev]
+            del _WORKSPACE[key]
             del buf
         buf = torch.empty(int(nbytes * 1.25) + 256, dtype=torch.uint8, device=f"cuda:{dev}")
-        _WORKSPACE[dev] = buf
+        _WORKSPACE[key] = buf
     return ctypes.c_void_p(buf.data_ptr()), buf.numel()
 
 

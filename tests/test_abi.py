@@ -8,11 +8,11 @@ import pytest
 import torch
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADER = os.path.join(ROOT, "include", "pydtnn_hip.h")
+HEADERS = [os.path.join(ROOT, "include", "pydtnn_hip.h"), os.path.join(ROOT, "include", "pydtnn_hip_test.h")]
 
 
 def declared_functions():
-    text = open(HEADER).read()
+    text = "".join(open(h).read() for h in HEADERS)
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     names = re.findall(r"\b([A-Za-z_][A-Za-z0-9_]*)\s*\(", text)
     keep = [n for n in names if n.startswith("pydtnn_hip_") or n.startswith("sconvGemm") or n == "alloc_pack_buffs"]

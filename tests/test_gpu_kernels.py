@@ -786,6 +786,40 @@ def test_relu_mask_and_gate_arguments_are_checked(cg):
                             gate=torch.ones(x.shape, device="cuda"), **_kw(d))
 
 
+@pytest.mark.parametrize("fmt", ["NCHW", "NHWC"])
+def test_pooling_batches_beyond_the_addressing_limit_run_as_image_groups(ops, fmt):
+    """Pooling works plane by plane; with the per-launch limit lowered so that 7 images need 3 launches the
+    results equal the single launch bit for bit (max and average pooling, forward, backward and gated)."""
+    from pydtnn_amd import native
+    n, c, h, w = 7, 5, 12, 10
+    announce("pooling in image groups", fmt)
+    rng = np.random.default_rng(17)
+    nh = fmt == "NHWC"
+    x = dev(rng.standard_normal((n, h, w, c) if nh else (n, c, h, w)).astype(np.float32))
+    g = (3, 3, 1, 1, 2, 2)
+    fwd, bwd = (ops.max_pool_2d_fwd_nhwc, ops.max_pool_2d_bwd_nhwc) if nh else (ops.max_pool_2d_fwd_nchw, ops.max_pool_2d_bwd_nchw)
+    dims = (n, h, w, c) if nh else (n, c, h, w)
+
+    def run():
+        y, idx = fwd(x, *g)
+        dy = torch.arange(y.numel(), device="cuda", dtype=torch.float32).reshape(y.shape) / 16.0
+        gate = (x > 0).to(torch.int8)
+        out = [y, idx, bwd(dy, idx, *dims, *g), bwd(dy, idx, *dims, *g, gate=gate)]
+        ya = ops.average_pool_2d_fwd(x, nh, *g)
+        out += [ya, ops.average_pool_2d_bwd(dy, nh, n, c, h, w, *g)]
+        return out
+
+    whole = run()
+    lib = native.lib()
+    before = lib.pydtnn_hip_debug_set_tensor_floats_limit(3 * c * h * w + 1)
+    try:
+        grouped = run()
+    finally:
+        lib.pydtnn_hip_debug_set_tensor_floats_limit(before)
+    for a, b in zip(whole, grouped):
+        assert torch.equal(a, b)
+
+
 def test_maxpool_backward_with_gate_equals_backward_then_relu_backward(ops):
     rng = np.random.default_rng(12)
     for (shape, kh, kw, s, p) in [((2, 3, 8, 10), 2, 2, 2, 0), ((2, 4, 9, 9), 3, 3, 2, 1), ((2, 3, 9, 11), 2, 2, 2, 0),
@@ -845,6 +879,34 @@ def test_libconvgemm_compat_abi_runs_like_the_reference_shim(oracle):
                            ctypes.c_void_p(w.ctypes.data), ctypes.c_void_p(dy.ctypes.data),
                            ctypes.c_void_p(dx.ctypes.data), ac, bc)
     assert_close(dx, dx_ref, what="compat dx")
+    # the NHWC entry points and the batch-normalisation arguments (pydtnn/backends/cpu/libs/conv_gemm.py:234-248,
+    # :321-328), on a larger and then a smaller problem so that the library's cached device buffers are reused
+    # at a different size
+    vp = lambda a: ctypes.c_void_p(a.ctypes.data)
+    rng = np.random.default_rng(12)
+    for d2 in (mid_grid[6], small_grid[1]):
+        announce("compat abi nhwc", d2)
+        x2, w2, b2, dy2 = case(d2)
+        xr, wr, dyr = nhwc(x2), w_nhwc(w2), nhwc(dy2)
+        g = [u(v) for v in (d2.b, d2.h, d2.w, d2.c, d2.kn, d2.kh, d2.kw)]
+        pads = [u(d2.vpadding), u(d2.hpadding)]
+        strides = [u(d2.vstride), u(d2.hstride)]
+        dils = [u(d2.vdilation), u(d2.hdilation)]
+        bn = [rng.uniform(0.5, 1.5, d2.kn).astype(np.float32) for _ in range(4)]
+        y2 = np.full((d2.b, d2.ho, d2.wo, d2.kn), np.nan, np.float32)
+        lib.sconvGemmNHWC(ctypes.c_char(b'N'), *g, *pads, *strides, *dils, vp(wr), vp(xr), vp(y2), vp(b2), vp(bn[0]),
+                          vp(bn[1]), vp(bn[2]), vp(bn[3]), ctypes.c_bool(True), ac, bc)
+        p2 = oracle.ConvParams(*d2.geom())
+        ref2, rows = oracle.conv2d_forward_nhwc_i2c(xr, wr, b2, p2)
+        assert_close(y2, oracle.fused_epilogue(ref2, "NHWC", bn=bn, relu_flag=True), what="compat nhwc fused fwd")
+        dw2 = np.full(wr.shape, np.nan, np.float32)
+        lib.sconvGemmNHWC(ctypes.c_char(b'Y'), *g, *pads, *strides, *dils, vp(dyr), vp(xr), vp(dw2), none, none, none,
+                          none, none, ctypes.c_bool(False), ac, bc)
+        dw_ref2, _, dx_ref2 = oracle.conv2d_backward_nhwc_i2c(dyr, rows, wr, xr.shape, p2)
+        assert_close(dw2, dw_ref2, what="compat nhwc dw")
+        dx2 = np.zeros(xr.shape, np.float32)
+        lib.sconvGemmNHWC_back(*g, *strides, *pads, *dils, vp(wr), vp(dyr), vp(dx2), ac, bc)   # stride before padding
+        assert_close(dx2, dx_ref2, what="compat nhwc dx")
     libc = ctypes.CDLL("libc.so.6")
     libc.free(ac)
     libc.free(bc)
