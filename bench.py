@@ -221,6 +221,8 @@ def run_cfg2(torch, pd, args):
     extra["epilogue_pct_hbm_peak"] = round(100 * extra["epilogue_gbs"] / HBM_PEAK_GBS, 1)
     del mat, back
     extra.update(compat_route(x, w, b, gemm_flop))
+    del xd, dyd
+    extra.update(f64_route(torch, gemm_flop))
     roofline = {"bound": "mfma", "kernel": "gemm_streamk_kernel_big_tile<256x128, PlainK4, Im2colNchwMN, EpiNchw> + streamk_fixup_kernel (forward)",
                 "achieved": round(achieved, 3), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES["cfg2"],
@@ -228,6 +230,36 @@ def run_cfg2(torch, pd, args):
     workload = ("cfg2: VGG16-style 3x3 conv layer fwd+dW+db+dX, fp32 NCHW, N=64, 256->256, 56x56, stride 1, pad 1, "
                 "implicit GEMM")
     return ms, step_flop / (ms * 1e-3) / 1e9, workload, roofline, extra
+
+
+FP64_MFMA_PEAK_TFLOPS = 78.6
+
+
+def f64_route(torch, gemm_flop, n=64):
+    """The explicit route's three GEMMs of cfg2 in float64 (the reference's float64 path is im2col + a @ b),
+    on the v_mfma_f64_16x16x4_f64 engine, against the 78.6 TFLOP/s float64 matrix peak."""
+    from pydtnn_amd import ops
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    p = n * 56 * 56
+    w2d = torch.randn((256, 2304), device="cuda", dtype=torch.float64, generator=gen)
+    cols = torch.randn((2304, p), device="cuda", dtype=torch.float64, generator=gen)
+    dy_cols = torch.randn((256, p), device="cuda", dtype=torch.float64, generator=gen)
+    y = torch.empty((256, p), device="cuda", dtype=torch.float64)
+    dw = torch.empty((256, 2304), device="cuda", dtype=torch.float64)
+    calls = {"f64_i2c_fwd": lambda: ops.matmul(w2d, cols, c=y),            # (co,K) @ (K,P)
+             "f64_i2c_dw": lambda: ops.matmul(dy_cols, cols.t(), c=dw),    # (co,P) @ (P,K)
+             "f64_i2c_dx_gemm": lambda: ops.matmul(w2d.t(), dy_cols, c=cols)}  # (K,co) @ (co,P)
+    out = {}
+    for name, fn in calls.items():
+        t = Timer(torch)
+        for i in range(4):
+            fn() if i == 0 else t(fn)
+        torch.cuda.synchronize()
+        ms = t.median_ms()
+        out[name + "_ms"] = round(ms, 3)
+        out[name + "_tflops"] = round(gemm_flop / (ms * 1e-3) / 1e12, 2)
+        out[name + "_pct_fp64_mfma_peak"] = round(100 * gemm_flop / (ms * 1e-3) / 1e12 / FP64_MFMA_PEAK_TFLOPS, 1)
+    return out
 
 
 def compat_route(x, w, b, gemm_flop, reps=3):

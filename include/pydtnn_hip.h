@@ -307,6 +307,44 @@ int pydtnn_hip_sgd_momentum(float *w, const float *dw, float *velocity, long tot
                             float decay, int nesterov, void *stream);
 
 /* ------------------------------------------------------------------------------------------
+ * The float64 route.  The reference computes in float64 through its explicit path only: the im2col / im2row /
+ * col2im / row2im, add, ReLU and BN-inference modules dispatch on float64
+ * (pydtnn/cython_modules/im2row_nhwc_cython.pyx:25-49, im2col_nchw_cython.pyx:28-52) and utils.matmul is a plain
+ * a @ b (pydtnn/utils/__init__.py:148-158); libconvGemm is float32 only (conv_gemm.py:101-107).  Same index
+ * maps, summation orders and argument meaning as the float32 entry points of the same name.
+ *   pydtnn_hip_dgemm: C = op(A) op(B) (+ bias[n], ReLU) on v_mfma_f64_16x16x4_f64, operands row-major or the
+ *       transposed view of a row-major matrix; small C with a long reduction is split along k into
+ *       `workspace` (pydtnn_hip_dgemm_workspace_bytes, 0 = not needed; then C must be dense, ldc == n).
+ *   pydtnn_hip_transpose_1023_f64: dst[d1][d0][inner] = src[d0][d1][inner], the (co,N,ho,wo) <-> (N,co,ho,wo)
+ *       copy of pydtnn/utils/best_transpose_1023.py:50-58.
+ *   pydtnn_hip_bias_grad_f64: db[ch] = sum of dy over (outer, inner); needs no workspace.
+ * ---------------------------------------------------------------------------------------- */
+size_t pydtnn_hip_dgemm_workspace_bytes(long m, long n, long k);
+int pydtnn_hip_dgemm(int transa, int transb, long m, long n, long k, const double *a, long lda, const double *b,
+                     long ldb, double *c, long ldc, const double *bias, int relu, void *workspace,
+                     size_t workspace_bytes, void *stream);
+int pydtnn_hip_im2col_nchw_f64(const double *x, double *cols, int b, int c, int h, int w, int kh, int kw,
+                               int vpadding, int hpadding, int vstride, int hstride, int vdilation, int hdilation,
+                               void *stream);
+int pydtnn_hip_col2im_nchw_f64(const double *cols, double *dx, int b, int c, int h, int w, int kh, int kw,
+                               int vpadding, int hpadding, int vstride, int hstride, int vdilation, int hdilation,
+                               void *stream);
+int pydtnn_hip_im2row_nhwc_f64(const double *x, double *rows, int b, int h, int w, int c, int kh, int kw,
+                               int vpadding, int hpadding, int vstride, int hstride, int vdilation, int hdilation,
+                               void *stream);
+int pydtnn_hip_row2im_nhwc_f64(const double *rows, double *dx, int b, int h, int w, int c, int kh, int kw,
+                               int vpadding, int hpadding, int vstride, int hstride, int vdilation, int hdilation,
+                               void *stream);
+int pydtnn_hip_chan_eltwise_f64(const double *x, const double *residual, double *y, long total, long inner,
+                                int channels, const double *bias, const double *bn_running_mean,
+                                const double *bn_inv_std, const double *bn_gamma, const double *bn_beta, int relu,
+                                void *stream);
+int pydtnn_hip_relu_fwd_f64(const double *x, double *y, int8_t *mask, long total, void *stream);
+int pydtnn_hip_relu_bwd_f64(const double *dy, const int8_t *mask, double *dx, long total, void *stream);
+int pydtnn_hip_bias_grad_f64(const double *dy, double *db, long outer, int channels, long inner, void *stream);
+int pydtnn_hip_transpose_1023_f64(const double *src, double *dst, int d0, int d1, long inner, void *stream);
+
+/* ------------------------------------------------------------------------------------------
  * Host-pointer compatibility flavour (exported by libconvGemm.so only).  Signatures are those
  * PyDTNN's ctypes shim calls (pydtnn/backends/cpu/libs/conv_gemm.py:91-92, :191-205, :234-248,
  * :299-307, :321-328).  ac_pack / bc_pack are accepted and ignored; alloc_pack_buffs hands out two

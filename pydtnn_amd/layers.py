@@ -285,9 +285,9 @@ class Conv2D(Layer):
         self.wo = (self.wi + 2 * self.hpadding - self.hdilation * (self.kw - 1) - 1) // self.hstride + 1
         self.shape = encode_tensor((self.ho, self.wo, self.co), self.model.tensor_format)
         self.nparams = int(np.prod(self.weights_shape)) + (self.co if self.use_bias else 0)
-        self.weights = self.weights_initializer(self.weights_shape)
+        self.weights = self.weights_initializer(self.weights_shape).to(self.model.dtype)
         if self.use_bias:
-            self.biases = self.biases_initializer((self.co,))
+            self.biases = self.biases_initializer((self.co,)).to(self.model.dtype)
         if self.model.enable_conv_gemm:
             self.cg = ConvGemm(dtype=self.model.dtype, debug=self.debug, parent_layer=self)
         variant = "cg" if self.model.enable_conv_gemm else "i2c"  # conv_2d_cpu.py:89, :139-140
@@ -524,9 +524,9 @@ class FC(Layer):
 
     def initialize(self, prev_shape, need_dx=True):
         super().initialize(prev_shape, need_dx)
-        self.weights = self.weights_initializer((*prev_shape, *self.shape))
+        self.weights = self.weights_initializer((*prev_shape, *self.shape)).to(self.model.dtype)
         if self.use_bias:
-            self.biases = self.biases_initializer(self.shape)
+            self.biases = self.biases_initializer(self.shape).to(self.model.dtype)
         self.nparams = self.weights.numel() + (self.biases.numel() if self.use_bias else 0)
 
     def forward(self, x):
@@ -682,10 +682,10 @@ class BatchNormalization(Layer):
         if self.spatial:
             self.hi, self.wi, self.ci = decode_tensor(self.shape, self.model.tensor_format)
             shape_ = (self.ci,)
-        self.gamma = torch.full(shape_, self.gamma_init_val, dtype=torch.float32, device="cuda")
-        self.beta = torch.full(shape_, self.beta_init_val, dtype=torch.float32, device="cuda")
-        self.running_mean = self.moving_mean_initializer(shape_)
-        self.running_var = self.moving_variance_initializer(shape_)
+        self.gamma = torch.full(shape_, self.gamma_init_val, dtype=self.model.dtype, device="cuda")
+        self.beta = torch.full(shape_, self.beta_init_val, dtype=self.model.dtype, device="cuda")
+        self.running_mean = self.moving_mean_initializer(shape_).to(self.model.dtype)
+        self.running_var = self.moving_variance_initializer(shape_).to(self.model.dtype)
         self.inv_std = 1.0 / torch.sqrt(self.running_var + self.epsilon)
         self.nparams = self.gamma.numel() + self.beta.numel() + self.running_mean.numel() + self.running_var.numel()
 

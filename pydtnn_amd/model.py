@@ -57,9 +57,15 @@ class Model:
         self.kwargs.update(kwargs)
         if isinstance(dtype, str):
             dtype = {"float32": torch.float32, "float64": torch.float64}[dtype]
-        if dtype != torch.float32:
-            raise ValueError("only float32 models run on the MI355X kernels")
+        if dtype not in (torch.float32, torch.float64):
+            raise ValueError("models compute in float32 or float64")
         self.dtype = dtype
+        if dtype == torch.float64:
+            # libconvGemm is float32 only (pydtnn/backends/cpu/libs/conv_gemm.py:101-107): a float64 model takes
+            # the explicit im2col / im2row + GEMM route, as it does in the reference
+            if kwargs.get("enable_conv_gemm"):
+                raise ValueError("the implicit ConvGemm route is float32 only; a float64 model uses the explicit one")
+            self.kwargs["enable_conv_gemm"] = False
         self.tracer = NullTracer()
         self.layers = []
         self.layer_id = _layer_id_generator()
@@ -295,7 +301,7 @@ class Model:
                     if current is not None and tuple(ary.shape) != tuple(current.shape):
                         raise ValueError(f"'{base}' has shape {tuple(ary.shape)}, the layer expects "
                                          f"{tuple(current.shape)}")
-                    setattr(layer, key, torch.from_numpy(np.ascontiguousarray(ary, dtype=np.float32)).cuda())
+                    setattr(layer, key, torch.from_numpy(np.ascontiguousarray(ary)).to(self.dtype).cuda())
                 elif mode == "store":
                     d[base] = getattr(layer, key).detach().cpu().numpy()
 

@@ -70,6 +70,20 @@ SIGNATURES = {
                                                         _c.c_int, _vp, _c.c_size_t, _vp]),
     "pydtnn_hip_sgd_momentum": (_c.c_int, [_f32p, _f32p, _f32p, _c.c_long, _c.c_float, _c.c_float, _c.c_float,
                                            _c.c_int, _vp]),
+    # float64 route
+    "pydtnn_hip_dgemm_workspace_bytes": (_c.c_size_t, [_c.c_long] * 3),
+    "pydtnn_hip_dgemm": (_c.c_int, [_c.c_int, _c.c_int, _c.c_long, _c.c_long, _c.c_long, _vp, _c.c_long, _vp, _c.c_long,
+                                    _vp, _c.c_long, _vp, _c.c_int, _vp, _c.c_size_t, _vp]),
+    "pydtnn_hip_im2col_nchw_f64": (_c.c_int, [_vp, _vp] + [_c.c_int] * 12 + [_vp]),
+    "pydtnn_hip_col2im_nchw_f64": (_c.c_int, [_vp, _vp] + [_c.c_int] * 12 + [_vp]),
+    "pydtnn_hip_im2row_nhwc_f64": (_c.c_int, [_vp, _vp] + [_c.c_int] * 12 + [_vp]),
+    "pydtnn_hip_row2im_nhwc_f64": (_c.c_int, [_vp, _vp] + [_c.c_int] * 12 + [_vp]),
+    "pydtnn_hip_chan_eltwise_f64": (_c.c_int, [_vp, _vp, _vp, _c.c_long, _c.c_long, _c.c_int] + [_vp] * 5 +
+                                    [_c.c_int, _vp]),
+    "pydtnn_hip_relu_fwd_f64": (_c.c_int, [_vp, _vp, _i8p, _c.c_long, _vp]),
+    "pydtnn_hip_relu_bwd_f64": (_c.c_int, [_vp, _i8p, _vp, _c.c_long, _vp]),
+    "pydtnn_hip_bias_grad_f64": (_c.c_int, [_vp, _vp, _c.c_long, _c.c_int, _c.c_long, _vp]),
+    "pydtnn_hip_transpose_1023_f64": (_c.c_int, [_vp, _vp, _c.c_int, _c.c_int, _c.c_long, _vp]),
 }
 
 # Host-pointer flavour exported by libconvGemm.so with the reference's own names

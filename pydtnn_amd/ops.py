@@ -21,53 +21,66 @@ def _need_f32(*tensors):
     for t in tensors:
         if t is not None and t.dtype != torch.float32:
             # pydtnn/cython_modules/im2col_nchw_cython.pyx:49-50 raises TypeError for unsupported dtypes
-            raise TypeError(f"Type '{t.dtype}' is not supported by the MI355X kernels (float32 only)")
+            raise TypeError(f"Type '{t.dtype}' is not supported by this kernel (float32 only)")
+
+
+def _is_f64(*tensors):
+    """True when the operands are float64 (the explicit route's second dtype, as in the reference's Cython
+    modules); every operand must then be float64.  Any dtype other than float32 / float64 raises TypeError."""
+    kinds = {t.dtype for t in tensors if t is not None}
+    if kinds == {torch.float64}:
+        return True
+    if kinds - {torch.float32}:
+        raise TypeError(f"Type(s) {sorted(str(k) for k in kinds)} not supported (float32, or float64 throughout)")
+    return False
+
+
 
 
 # --------------------------------------------------------------------------- im2col family
 
 def im2col_nchw(x, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation):
     """pydtnn/cython_modules/im2col_nchw_cython.pyx:28-52"""
-    _need_f32(x)
+    fn = lib().pydtnn_hip_im2col_nchw_f64 if _is_f64(x) else lib().pydtnn_hip_im2col_nchw
     n, c, h, w = x.shape
     hh, ww = _out_hw(h, w, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
     cols = torch.empty((c * kh * kw, n * hh * ww), dtype=x.dtype, device=x.device)
-    check(lib().pydtnn_hip_im2col_nchw(f32(x), f32(cols), n, c, h, w, kh, kw, vpadding, hpadding, vstride, hstride,
+    check(fn(ptr(x), ptr(cols), n, c, h, w, kh, kw, vpadding, hpadding, vstride, hstride,
                                        vdilation, hdilation, stream_ptr()), "im2col_nchw")
     return cols
 
 
 def col2im_nchw(cols, n, c, h, w, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation):
     """pydtnn/cython_modules/im2col_nchw_cython.pyx:150-173"""
-    _need_f32(cols)
+    fn = lib().pydtnn_hip_col2im_nchw_f64 if _is_f64(cols) else lib().pydtnn_hip_col2im_nchw
     hh, ww = _out_hw(h, w, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
     if tuple(cols.shape) != (c * kh * kw, n * hh * ww):
         raise ValueError(f"cols has shape {tuple(cols.shape)}, expected {(c * kh * kw, n * hh * ww)}")
     dx = torch.empty((n, c, h, w), dtype=cols.dtype, device=cols.device)
-    check(lib().pydtnn_hip_col2im_nchw(f32(cols), f32(dx), n, c, h, w, kh, kw, vpadding, hpadding, vstride, hstride,
+    check(fn(ptr(cols), ptr(dx), n, c, h, w, kh, kw, vpadding, hpadding, vstride, hstride,
                                        vdilation, hdilation, stream_ptr()), "col2im_nchw")
     return dx
 
 
 def im2row_nhwc(x, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation):
     """pydtnn/cython_modules/im2row_nhwc_cython.pyx:25-49"""
-    _need_f32(x)
+    fn = lib().pydtnn_hip_im2row_nhwc_f64 if _is_f64(x) else lib().pydtnn_hip_im2row_nhwc
     n, h, w, c = x.shape
     hh, ww = _out_hw(h, w, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
     rows = torch.empty((n * hh * ww, c * kh * kw), dtype=x.dtype, device=x.device)
-    check(lib().pydtnn_hip_im2row_nhwc(f32(x), f32(rows), n, h, w, c, kh, kw, vpadding, hpadding, vstride, hstride,
+    check(fn(ptr(x), ptr(rows), n, h, w, c, kh, kw, vpadding, hpadding, vstride, hstride,
                                        vdilation, hdilation, stream_ptr()), "im2row_nhwc")
     return rows
 
 
 def row2im_nhwc(rows, n, h, w, c, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation):
     """pydtnn/cython_modules/im2row_nhwc_cython.pyx:123-146"""
-    _need_f32(rows)
+    fn = lib().pydtnn_hip_row2im_nhwc_f64 if _is_f64(rows) else lib().pydtnn_hip_row2im_nhwc
     hh, ww = _out_hw(h, w, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
     if tuple(rows.shape) != (n * hh * ww, c * kh * kw):
         raise ValueError(f"rows has shape {tuple(rows.shape)}, expected {(n * hh * ww, c * kh * kw)}")
     dx = torch.empty((n, h, w, c), dtype=rows.dtype, device=rows.device)
-    check(lib().pydtnn_hip_row2im_nhwc(f32(rows), f32(dx), n, h, w, c, kh, kw, vpadding, hpadding, vstride, hstride,
+    check(fn(ptr(rows), ptr(dx), n, h, w, c, kh, kw, vpadding, hpadding, vstride, hstride,
                                        vdilation, hdilation, stream_ptr()), "row2im_nhwc")
     return dx
 
@@ -92,7 +105,7 @@ def matmul(a, b, c=None, bias=None, relu=False):
     Operands may be the ``.T`` view of a contiguous matrix, as in the reference's
     ``x_cols.T`` / ``weights.T`` call sites (conv_2d_cpu.py:454, fc_cpu.py:67,75).
     """
-    _need_f32(a, b, c, bias)
+    f64 = _is_f64(a, b, c, bias)
     a_, ta, lda = _as_gemm_operand(a)
     b_, tb, ldb = _as_gemm_operand(b)
     m, k = a.shape
@@ -103,6 +116,11 @@ def matmul(a, b, c=None, bias=None, relu=False):
         c = torch.empty((m, n), dtype=a.dtype, device=a.device)
     elif tuple(c.shape) != (m, n) or not c.is_contiguous():
         raise ValueError("matmul: output must be a contiguous (m, n) matrix")
+    if f64:
+        ws, ws_bytes = native.workspace(lib().pydtnn_hip_dgemm_workspace_bytes(m, n, k))
+        check(lib().pydtnn_hip_dgemm(ta, tb, m, n, k, ptr(a_), lda, ptr(b_), ldb, ptr(c), n, ptr(bias), int(relu),
+                                     ws, ws_bytes, stream_ptr()), "dgemm")
+        return c
     ws, ws_bytes = native.workspace(lib().pydtnn_hip_sgemm_workspace_bytes(m, n, k))
     check(lib().pydtnn_hip_sgemm(ta, tb, m, n, k, ptr(a_), lda, ptr(b_), ldb, ptr(c), n, f32(bias), int(relu),
                                  ws, ws_bytes, stream_ptr()), "sgemm")
@@ -113,12 +131,15 @@ def matmul(a, b, c=None, bias=None, relu=False):
 
 def chan_eltwise(x, channels, inner, residual=None, bias=None, bn=None, relu=False, out=None):
     """y = relu?(bn?(x (+ residual) + bias)), channel = (index // inner) % channels."""
-    _need_f32(x, residual, bias)
     mean = inv_std = gamma = beta = None
     if bn is not None:
         mean, inv_std, gamma, beta = bn
-        _need_f32(mean, inv_std, gamma, beta)
     y = torch.empty_like(x) if out is None else out
+    if _is_f64(x, residual, bias, mean, inv_std, gamma, beta, y):
+        check(lib().pydtnn_hip_chan_eltwise_f64(ptr(x), ptr(residual), ptr(y), x.numel(), inner, channels, ptr(bias),
+                                                ptr(mean), ptr(inv_std), ptr(gamma), ptr(beta), int(relu),
+                                                stream_ptr()), "chan_eltwise_f64")
+        return y
     check(lib().pydtnn_hip_chan_eltwise(f32(x), f32(residual), f32(y), x.numel(), inner, channels, f32(bias),
                                         f32(mean), f32(inv_std), f32(gamma), f32(beta), int(relu), stream_ptr()),
           "chan_eltwise")
@@ -163,26 +184,28 @@ def _need_gate(gate, dx):
 
 def relu(x, with_mask=True):
     """pydtnn/cython_modules/relu_cython.pyx:25-39 -> (max(x, 0), int8 mask)"""
-    _need_f32(x)
+    fn = lib().pydtnn_hip_relu_fwd_f64 if _is_f64(x) else lib().pydtnn_hip_relu_fwd
     y = torch.empty_like(x)
     mask = torch.empty(x.shape, dtype=torch.int8, device=x.device) if with_mask else None
-    check(lib().pydtnn_hip_relu_fwd(f32(x), f32(y), ptr(mask), x.numel(), stream_ptr()), "relu_fwd")
+    check(fn(ptr(x), ptr(y), ptr(mask), x.numel(), stream_ptr()), "relu_fwd")
     return y, mask
 
 
 def relu_backward(dy, mask):
     """dy * mask (pydtnn/backends/cpu/activations/relu_cpu.py:38-40)"""
-    _need_f32(dy)
+    fn = lib().pydtnn_hip_relu_bwd_f64 if _is_f64(dy) else lib().pydtnn_hip_relu_bwd
     dx = torch.empty_like(dy)
-    check(lib().pydtnn_hip_relu_bwd(f32(dy), ptr(mask), f32(dx), dy.numel(), stream_ptr()), "relu_bwd")
+    check(fn(ptr(dy), ptr(mask), ptr(dx), dy.numel(), stream_ptr()), "relu_bwd")
     return dx
 
 
 def bias_grad(dy, channels, inner):
     """Sum of dy over everything but the channel axis; dy viewed as (outer, channels, inner)."""
-    _need_f32(dy)
     outer = dy.numel() // (channels * inner)
     db = torch.empty((channels,), dtype=dy.dtype, device=dy.device)
+    if _is_f64(dy):
+        check(lib().pydtnn_hip_bias_grad_f64(ptr(dy), ptr(db), outer, channels, inner, stream_ptr()), "bias_grad_f64")
+        return db
     ws, ws_bytes = native.workspace(2048 * channels)
     check(lib().pydtnn_hip_bias_grad(f32(dy), f32(db), outer, channels, inner, ws, ws_bytes, stream_ptr()),
           "bias_grad")
@@ -345,15 +368,68 @@ def _geom13(b, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilat
     return (b, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
 
 
+def transpose_1023(src):
+    """(d0, d1, h, w) -> (d1, d0, h, w) copy: pydtnn/utils/best_transpose_1023.py:50-58.  float64 only here: the
+    float32 kernels store in the tensor format directly and never need the copy."""
+    if not _is_f64(src):
+        raise TypeError("transpose_1023 is part of the float64 route only")
+    d0, d1 = src.shape[0], src.shape[1]
+    inner = src.numel() // (d0 * d1)
+    dst = torch.empty((d1, d0) + tuple(src.shape[2:]), dtype=src.dtype, device=src.device)
+    check(lib().pydtnn_hip_transpose_1023_f64(ptr(src), ptr(dst), d0, d1, inner, stream_ptr()), "transpose_1023_f64")
+    return dst
+
+
+def _i2c_forward_f64(nhwc, geom13, weights, mat, y, biases):
+    """The reference's own steps (conv_2d_cpu.py:183-209, :264-291): matmul, bias pass, and for NCHW the
+    (co,N,ho,wo) -> (N,co,ho,wo) copy."""
+    b, c, h, w, kn, kh, kw = geom13[:7]
+    if nhwc:
+        matmul(mat, weights.reshape(-1, kn), c=y.view(-1, kn), bias=biases)
+        return y
+    ho, wo = y.shape[2], y.shape[3]
+    res = matmul(weights.reshape(kn, -1), mat)
+    if biases is not None:
+        add_nchw(res, biases)
+    y.copy_(transpose_1023(res.view(kn, b, ho, wo)))
+    return y
+
+
+def _i2c_dw_f64(nhwc, geom13, dy, mat, dw):
+    """conv_2d_cpu.py:370 (x_rows.T @ dy_rows) and :454 (dy_cols @ x_cols.T)."""
+    kn = geom13[4]
+    if nhwc:
+        matmul(mat.t(), dy.reshape(-1, kn), c=dw.view(-1, kn))
+    else:
+        dy_cols = transpose_1023(dy).reshape(kn, -1)
+        matmul(dy_cols, mat.t(), c=dw.view(kn, -1))
+    return dw
+
+
+def _i2c_dx_f64(nhwc, geom13, weights, dy, dx):
+    """conv_2d_cpu.py:389-395 (dy_rows @ W.T, row2im) and :473-479 (W.T @ dy_cols, col2im)."""
+    b, c, h, w, kn, kh, kw, vp, hp, vs, hs, vd, hd = geom13
+    if nhwc:
+        res = matmul(dy.reshape(-1, kn), weights.reshape(-1, kn).t())
+        dx.copy_(row2im_nhwc(res, b, h, w, c, kh, kw, vp, hp, vs, hs, vd, hd))
+    else:
+        dy_cols = transpose_1023(dy).reshape(kn, -1)
+        res = matmul(weights.reshape(kn, -1).t(), dy_cols)
+        dx.copy_(col2im_nchw(res, b, c, h, w, kh, kw, vp, hp, vs, hs, vd, hd))
+    return dx
+
+
 def conv_i2c_forward(nhwc, geom13, weights, mat, y, biases):
-    _need_f32(weights, mat, y, biases)
+    if _is_f64(weights, mat, y, biases):
+        return _i2c_forward_f64(nhwc, geom13, weights, mat, y, biases)
     check(lib().pydtnn_hip_conv_i2c_forward(int(nhwc), *geom13, f32(weights), f32(mat), f32(y), f32(biases),
                                             stream_ptr()), "conv_i2c_forward")
     return y
 
 
 def conv_i2c_dw(nhwc, geom13, dy, mat, dw):
-    _need_f32(dy, mat, dw)
+    if _is_f64(dy, mat, dw):
+        return _i2c_dw_f64(nhwc, geom13, dy, mat, dw)
     ws, ws_bytes = native.conv_workspace(native.OP_DW, nhwc, geom13)
     check(lib().pydtnn_hip_conv_i2c_dw(int(nhwc), *geom13, f32(dy), f32(mat), f32(dw), ws, ws_bytes, stream_ptr()),
           "conv_i2c_dw")
@@ -361,7 +437,8 @@ def conv_i2c_dw(nhwc, geom13, dy, mat, dw):
 
 
 def conv_i2c_dx(nhwc, geom13, weights, dy, dx):
-    _need_f32(weights, dy, dx)
+    if _is_f64(weights, dy, dx):
+        return _i2c_dx_f64(nhwc, geom13, weights, dy, dx)
     ws, ws_bytes = native.conv_workspace(native.OP_DX_I2C, nhwc, geom13)
     check(lib().pydtnn_hip_conv_i2c_dx(int(nhwc), *geom13, f32(weights), f32(dy), f32(dx), ws, ws_bytes,
                                        stream_ptr()), "conv_i2c_dx")

@@ -83,8 +83,12 @@ def test_host_tensors_are_rejected_before_any_launch(native):
     from pydtnn_amd import ops
     with pytest.raises(ValueError):
         ops.im2col_nchw(torch.zeros((1, 1, 4, 4)), 3, 3, 0, 0, 1, 1, 1, 1)
-    with pytest.raises(TypeError):
+    with pytest.raises(ValueError):  # float64 is the explicit route's second dtype: same rule, no launch
         ops.im2col_nchw(torch.zeros((1, 1, 4, 4), dtype=torch.float64), 3, 3, 0, 0, 1, 1, 1, 1)
+    with pytest.raises(TypeError):   # pydtnn/cython_modules/im2col_nchw_cython.pyx:49-50
+        ops.im2col_nchw(torch.zeros((1, 1, 4, 4), dtype=torch.int32), 3, 3, 0, 0, 1, 1, 1, 1)
+    with pytest.raises(TypeError):   # float32 and float64 operands do not mix
+        ops.matmul(torch.zeros((2, 2)), torch.zeros((2, 2), dtype=torch.float64))
 
 
 def test_tensor_format_helpers():

@@ -30,7 +30,8 @@ def oracle_forward(oracle, layer, x, fmt):
         fwd = oracle.conv2d_forward_nchw_i2c if fmt == "NCHW" else oracle.conv2d_forward_nhwc_i2c
         return fwd(x, host(layer.weights), host(layer.biases) if layer.use_bias else None, p)[0]
     if name == "BatchNormalization":
-        inv_std = (1.0 / np.sqrt(host(layer.running_var) + np.float32(layer.epsilon))).astype(np.float32)
+        var = host(layer.running_var)
+        inv_std = (1.0 / np.sqrt(var + var.dtype.type(layer.epsilon))).astype(var.dtype)
         return oracle.fused_epilogue(x, fmt if x.ndim == 4 else "NHWC",
                                      bn=(host(layer.running_mean), inv_std, host(layer.gamma), host(layer.beta)))
     if name == "Relu":
