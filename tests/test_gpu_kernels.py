@@ -216,6 +216,35 @@ def test_streaming_kernel_shapes_nhwc(cg, oracle, d):
     assert_close(host(dw), dw_ref, what="dw")
 
 
+# unpadded NCHW layers with wide filter rows (AlexNet-style first layers): rows of 5 .. 12 taps, strides 1 .. 4,
+# vertical dilation, filter counts on and off the 96-row tile
+quad_grid = [
+    D(4, 3, 35, 35, 96, 11, 11, 0, 0, 4, 4, 1, 1), D(3, 2, 30, 41, 64, 3, 5, 0, 0, 1, 1, 1, 1),
+    D(2, 5, 33, 40, 130, 7, 6, 0, 0, 2, 3, 1, 1), D(2, 1, 40, 37, 20, 5, 7, 0, 0, 1, 2, 2, 1),
+    D(5, 4, 29, 29, 192, 2, 8, 0, 0, 3, 1, 1, 1), D(2, 3, 31, 45, 33, 4, 9, 0, 0, 2, 2, 1, 1),
+    D(3, 3, 64, 64, 96, 12, 12, 0, 0, 4, 4, 1, 1), D(2, 7, 26, 30, 257, 1, 10, 0, 0, 1, 1, 1, 1),
+]
+
+
+@pytest.mark.parametrize("d", quad_grid, ids=repr)
+def test_wide_unpadded_filter_rows_nchw(cg, oracle, d):
+    announce("wide filter rows forward", d)
+    x, w, b, _ = case(d)
+    ref = _fwd_ref(oracle, x, w, b, d)
+    y = cg.conv_gemm_nchw(dev(w), dev(x), biases_vector=dev(b), **_kw(d))
+    assert_close(host(y), ref, what="y")
+    y = cg.conv_gemm_nchw(dev(w), dev(x), biases_vector=dev(b), relu=True, **_kw(d))
+    assert_close(host(y), np.maximum(ref, 0), what="relu(y)")
+    # a non-finite value in a column no window reaches must not leak in
+    x2 = x.copy()
+    x2[:, :, :, d.w - 1] = np.inf if (d.w - d.kw) % d.hstride != 0 else x2[:, :, :, d.w - 1]
+    if np.isinf(x2).any():
+        y2 = host(cg.conv_gemm_nchw(dev(w), dev(x2), biases_vector=dev(b), **_kw(d)))
+        ref2 = _fwd_ref(oracle, np.where(np.isinf(x2), 0, x2).astype(np.float32), w, b, d)
+        assert np.isfinite(y2).all()
+        assert_close(y2, ref2, what="y with an unused non-finite column")
+
+
 @pytest.mark.parametrize("x,w,stride", [
     (x_2x4, w_1x1, 1), (x_2x4, w_1x2, 1), (x_2x4, w_2x2, 1), (x_4x4, w_2x2, 2), (x_4x8, w_2x2, (1, 2)),
     (x_8x8, w_3x3, 3), (x_8x8, w_2x2, 1), (x_2x4_c2, w_c2_1234_4567, 1)])
