@@ -14,6 +14,7 @@
 // All four are HBM-bound streams: every matrix element is written (or read) once, lanes run along
 // the contiguous axis of the matrix, and padding zeros are produced in the same pass.
 #include "common.h"
+#include "gemm_engine.h"
 
 namespace {
 
@@ -261,7 +262,8 @@ __global__ void __launch_bounds__(kThreads) im2row_nhwc_quads_kernel(const float
     __shared__ float4 staged[kThreads * KHW];
     const int c4n = g.c >> 2, rows_per_block = kThreads / c4n;
     const int r = threadIdx.x / c4n, q = threadIdx.x - r * c4n;
-    const long p0 = (long)blockIdx.x * rows_per_block;
+    // each XCD takes one contiguous run of pixels, so the taps its workgroups share come from its own L2
+    const long p0 = (long)gemm::xcd_remap((int)blockIdx.x, (int)gridDim.x) * rows_per_block;
     const long p = p0 + r;
     float4 v[KHW];
 #pragma unroll
@@ -497,11 +499,140 @@ __global__ void __launch_bounds__(kThreads) row2im_nhwc_patch_kernel(const float
     }
 }
 
+
+// 3x3 taps, unit strides and dilations, c % 32 == 0: the matrix is read once, in full cache lines.
+// A workgroup owns (image, band of dx rows, strip of at most 8*S dx columns, chunk of 32 channels) and
+// walks down the output rows that feed its band.  The 32 x 9 floats a pixel of the matrix holds for the
+// chunk are one 1152-byte run (nine 128-byte lines when the matrix is so aligned); the runs of one output
+// row go to LDS through 128-bit loads, next row's loads in flight while this row is consumed.  Thread
+// (channel, slot) owns dx columns slot, slot + 8, ...; an output row gives taps i = 2, 1, 0 to the dx rows
+// one below, at and one above it (for vpadding 1), so each column keeps three running sums that rotate
+// as the walk advances, and a dx element receives its taps in descending (i, j) order as above.  Runs
+// outside the matrix read as zeros, which leaves a sum that starts at +0 unchanged.
+template <int S>
+__global__ void __launch_bounds__(kThreads) row2im_nhwc_walk_kernel(const float* __restrict__ rows,
+                                                                   float* __restrict__ dx, ConvGeom g, int strips,
+                                                                   int tw, int bands, int band_rows)
+{
+    constexpr int CB = 32, RUN4 = CB * 9 / 4;              // 72 float4 per (pixel, chunk)
+    constexpr int NLD = ((8 * S + 2) * RUN4 + kThreads - 1) / kThreads;
+    extern __shared__ float4 walk_lds[];
+    const int chunks = g.c / CB;
+    uint32_t bid = (uint32_t)gemm::xcd_remap((int)blockIdx.x, (int)gridDim.x);
+    const uint32_t cb = bid % (uint32_t)chunks; bid /= (uint32_t)chunks;
+    const uint32_t strip = bid % (uint32_t)strips; bid /= (uint32_t)strips;
+    const uint32_t band = bid % (uint32_t)bands;
+    const uint32_t nn = bid / (uint32_t)bands;
+    const int w0 = (int)strip * tw, wn = min(tw, g.w - w0);
+    const int h0 = (int)band * band_rows, hn = min(band_rows, g.h - h0);
+    const int ox0 = w0 + g.hpadding - 2;                  // output column of LDS column 0
+    const int ncols = wn + 2;
+    const gemm::rsrc_t src = gemm::make_rsrc(rows + (size_t)nn * g.howo * g.k + cb * (CB * 9), (long)g.howo * g.k - cb * (CB * 9));
+
+    // byte offset of this thread's j-th float4 of an output row, less the row's own offset
+    uint32_t off[NLD];
+#pragma unroll
+    for (int j = 0; j < NLD; ++j) {
+        const int f4 = (int)threadIdx.x + j * kThreads;
+        const int lc = f4 / RUN4, f = f4 - lc * RUN4;
+        const int ox = ox0 + lc;
+        off[j] = (lc < ncols && (unsigned)ox < (unsigned)g.wo) ? ((uint32_t)ox * g.k * 4u + (uint32_t)f * 16u) : gemm::kOob;
+    }
+    auto fetch = [&](int oy, gemm::floatx4* v) {
+        const bool row_ok = (unsigned)oy < (unsigned)g.ho;
+        const uint32_t soff = row_ok ? (uint32_t)oy * g.wo * g.k * 4u : 0u;
+#pragma unroll
+        for (int j = 0; j < NLD; ++j) v[j] = gemm::buf_load4(src, row_ok ? off[j] : gemm::kOob, soff);
+    };
+
+    const int cc = threadIdx.x & (CB - 1), slot = threadIdx.x / CB;
+    const float* mine = reinterpret_cast<const float*>(walk_lds) + (slot * CB + cc) * 9;
+    float* out = dx + ((size_t)nn * g.h * g.w + w0 + slot) * g.c + cb * CB + cc;
+    float a0[S], a1[S], a2[S];
+#pragma unroll
+    for (int s = 0; s < S; ++s) a0[s] = a1[s] = a2[s] = 0.0f;
+
+    const int oy_first = h0 + g.vpadding - 2, oy_last = h0 + hn - 1 + g.vpadding;
+    gemm::floatx4 v[NLD];
+    fetch(oy_first, v);
+    for (int oy = oy_first; oy <= oy_last; ++oy) {
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < NLD; ++j) {
+            const int f4 = (int)threadIdx.x + j * kThreads;
+            if (f4 < (8 * S + 2) * RUN4) walk_lds[f4] = make_float4(v[j][0], v[j][1], v[j][2], v[j][3]);
+        }
+        __syncthreads();
+        fetch(oy + 1 <= oy_last ? oy + 1 : -1, v);
+        // LDS column of tap j for dx column q is q + 2 - j
+#pragma unroll
+        for (int s = 0; s < S; ++s) {
+            const float* px = mine + s * 8 * CB * 9;
+            a2[s] = ((a2[s] + px[0 * CB * 9 + 8]) + px[1 * CB * 9 + 7]) + px[2 * CB * 9 + 6];
+            a1[s] = ((a1[s] + px[0 * CB * 9 + 5]) + px[1 * CB * 9 + 4]) + px[2 * CB * 9 + 3];
+            a0[s] = ((a0[s] + px[0 * CB * 9 + 2]) + px[1 * CB * 9 + 1]) + px[2 * CB * 9 + 0];
+        }
+        const int hh = oy - g.vpadding;  // the dx row whose last taps this output row held
+        if (hh >= h0) {
+            float* orow = out + (size_t)hh * g.w * g.c;
+#pragma unroll
+            for (int s = 0; s < S; ++s)
+                if (slot + 8 * s < wn) orow[(size_t)(8 * s) * g.c] = a0[s];
+        }
+#pragma unroll
+        for (int s = 0; s < S; ++s) { a0[s] = a1[s]; a1[s] = a2[s]; a2[s] = 0.0f; }
+    }
+}
+
+template <int S>
+int launch_row2im_walk(const float* rows, float* dx, const ConvGeom& g, int strips, int tw, int bands, int band_rows,
+                       hipStream_t stream)
+{
+    const size_t lds = (size_t)(8 * S + 2) * 32 * 9 * sizeof(float);
+    static std::atomic<bool> raised{false};
+    if (lds > 64 * 1024 && !raised.load(std::memory_order_acquire)) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&row2im_nhwc_walk_kernel<S>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+            return PYDTNN_HIP_ERR_LAUNCH;
+        raised.store(true, std::memory_order_release);
+    }
+    const long blocks = (long)g.n * bands * strips * (g.c / 32);
+    hipLaunchKernelGGL(row2im_nhwc_walk_kernel<S>, dim3((unsigned)blocks), dim3(kThreads), lds, stream, rows, dx, g,
+                       strips, tw, bands, band_rows);
+    HIP_RETURN_IF_LAUNCH_FAILED();
+    return PYDTNN_HIP_OK;
+}
+
+// 0 when the walk kernel does not cover the geometry.
+bool row2im_walk_plan(const ConvGeom& g, const float* rows, int* strips, int* tw, int* bands, int* band_rows)
+{
+    if (g.kh != 3 || g.kw != 3 || g.vstride != 1 || g.hstride != 1 || g.vdilation != 1 || g.hdilation != 1) return false;
+    if (g.c % 32 != 0 || (reinterpret_cast<uintptr_t>(rows) & 15) != 0) return false;
+    if ((long)g.howo * g.k >= (1l << 29) || g.vpadding > 2 || g.hpadding > 2) return false;
+    *strips = (g.w + 63) / 64;
+    *tw = (g.w + *strips - 1) / *strips;
+    // whole images while they fill the chip; else bands of rows (each re-reads two output rows)
+    const long per_band = (long)g.n * *strips * (g.c / 32);
+    int b = 1;
+    while (per_band * b < 512 && g.h / (b * 2) >= 8) b *= 2;
+    *band_rows = (g.h + b - 1) / b;
+    *bands = (g.h + *band_rows - 1) / *band_rows;
+    return per_band * *bands < (1l << 31);
+}
+
 }  // namespace
 
 int launch_row2im_nhwc(const float* rows, float* dx, const ConvGeom& g, hipStream_t stream)
 {
     constexpr int CB = 32;
+    int strips, tw, bands, band_rows;
+    if (row2im_walk_plan(g, rows, &strips, &tw, &bands, &band_rows)) {
+        if (tw <= 8) return launch_row2im_walk<1>(rows, dx, g, strips, tw, bands, band_rows, stream);
+        if (tw <= 16) return launch_row2im_walk<2>(rows, dx, g, strips, tw, bands, band_rows, stream);
+        if (tw <= 32) return launch_row2im_walk<4>(rows, dx, g, strips, tw, bands, band_rows, stream);
+        if (tw <= 56) return launch_row2im_walk<7>(rows, dx, g, strips, tw, bands, band_rows, stream);
+        return launch_row2im_walk<8>(rows, dx, g, strips, tw, bands, band_rows, stream);
+    }
     if (g.c % CB == 0) {
         const int chunks = g.c / CB;
         const long groups = ((long)g.h * g.w + (kThreads / CB) - 1) / (kThreads / CB);

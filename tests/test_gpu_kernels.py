@@ -102,6 +102,34 @@ def test_im2row_row2im_nhwc_bit_exact(ops, oracle, d):
     assert np.array_equal(host(dx), oracle.row2im_nhwc(rmat, d.b, d.h, d.w, d.c, *d.geom()))
 
 
+# 3x3 at unit stride with channels in chunks of 32: row2im walks bands of dx rows (strips of at most 64
+# columns; 8, 16, 32, 56 or 64 columns per strip by template), im2row hands its pixel runs to the XCDs
+walk_grid = [
+    D(3, 32, 7, 7, 2, 3, 3, 1, 1, 1, 1, 1, 1),
+    D(2, 64, 14, 14, 2, 3, 3, 1, 1, 1, 1, 1, 1),
+    D(2, 32, 28, 28, 2, 3, 3, 1, 1, 1, 1, 1, 1),
+    D(2, 96, 56, 56, 2, 3, 3, 1, 1, 1, 1, 1, 1),
+    D(1, 32, 64, 64, 2, 3, 3, 1, 1, 1, 1, 1, 1),
+    D(1, 32, 33, 70, 2, 3, 3, 1, 1, 1, 1, 1, 1),
+    D(1, 64, 19, 131, 2, 3, 3, 0, 2, 1, 1, 1, 1),
+    D(2, 32, 37, 23, 2, 3, 3, 2, 0, 1, 1, 1, 1),
+    D(1, 32, 40, 9, 2, 3, 3, 0, 0, 1, 1, 1, 1),
+    D(1, 32, 3, 3, 2, 3, 3, 0, 0, 1, 1, 1, 1),
+    D(1, 32, 2, 5, 2, 3, 3, 2, 2, 1, 1, 1, 1),
+]
+
+
+@pytest.mark.parametrize("d", walk_grid, ids=repr)
+def test_nhwc_gathers_walk_form_bit_exact(ops, oracle, d):
+    announce("im2row/row2im nhwc walk", d)
+    rng = np.random.default_rng(3)
+    xr = rng.standard_normal((d.b, d.h, d.w, d.c)).astype(np.float32)
+    assert np.array_equal(host(ops.im2row_nhwc(dev(xr), *d.geom())), oracle.im2row_nhwc(xr, *d.geom()))
+    rmat = rng.standard_normal((d.b * d.ho * d.wo, d.c * d.kh * d.kw)).astype(np.float32)
+    dx = ops.row2im_nhwc(dev(rmat), d.b, d.h, d.w, d.c, *d.geom())
+    assert np.array_equal(host(dx), oracle.row2im_nhwc(rmat, d.b, d.h, d.w, d.c, *d.geom()))
+
+
 @pytest.mark.parametrize("d", wide_channel_grid, ids=repr)
 def test_nhwc_gathers_staged_form_bit_exact(ops, oracle, d):
     announce("im2row/row2im nhwc staged", d)
