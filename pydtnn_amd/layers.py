@@ -87,7 +87,7 @@ class Layer:
         self.model = None
         self.prev_shape = None
         self.is_block_layer = False
-        # set by Model.add when ReLU folding is enabled (see Relu)
+        # set by Model.add unless ReLU folding is disabled (see Relu)
         self.relu_above = None
         self.relu_below = None
 
@@ -121,6 +121,16 @@ class Layer:
     def set_model(self, parent_model):
         self.model = parent_model
         self.id = next(self.model.layer_id)
+
+    # The neighbours do a Relu layer's work only inside the model's own training step, where the Relu layer is
+    # known to be the next consumer; a forward / backward called by hand computes what the reference's does.
+    def _folds_relu_above(self):
+        return self.relu_above is not None and self.model.mode == TRAIN_MODE and self.model.stepping
+
+    def _gate_below(self, dx_shape):
+        if self.relu_below is None or not self.model.stepping:
+            return None
+        return self.relu_below.gate_for(dx_shape)
 
     def initialize(self, prev_shape, need_dx=True):
         self.prev_shape = prev_shape
@@ -168,8 +178,8 @@ class Input(Layer):
 class Relu(Layer):
     """pydtnn/backends/cpu/activations/relu_cpu.py:25-40.
 
-    With ``Model(enable_relu_folding=True)`` and in TRAIN_MODE the neighbours may do this layer's work in their
-    own kernels: a convolution below hands over ``(y, mask)`` already rectified (``take_folded``), and the
+    Inside ``Model.train_batch`` (unless ``Model(enable_relu_folding=False)``) the neighbours do this layer's work
+    in their own kernels: a convolution below hands over ``(y, mask)`` already rectified (``take_folded``), and the
     layer above announces a dy it has already multiplied by the mask (``take_gated``).  Both are recognised by
     the identity of the tensor passed to forward / backward, so any other caller gets the plain computation."""
 
@@ -440,7 +450,7 @@ class Conv2D(Layer):
             self.cg_x = x
         biases_vector = self.biases if self.use_bias else None
         self._op(ev.PYDTNN_OPS_FORWARD_CONVGEMM)
-        if self.model.mode == TRAIN_MODE and self.relu_above is not None:
+        if self._folds_relu_above():
             y = self._folded_forward(self.cg.conv_gemm_nhwc, x, (x.shape[0], self.ho, self.wo, self.co),
                                      biases_vector)
         else:
@@ -460,7 +470,7 @@ class Conv2D(Layer):
             self._end()
         if self.need_dx:
             dx = torch.empty((dy.shape[0], self.hi, self.wi, self.ci), dtype=dy.dtype, device=dy.device)
-            gate = self.relu_below.gate_for(dx.shape) if self.relu_below is not None else None
+            gate = self._gate_below(dx.shape)
             self._op(ev.PYDTNN_OPS_BACKWARD_DECONV_GEMM)
             self.cg.deconv_gemm_nhwc(self.weights, dy, dx, gate=gate, **self._cg_kwargs())
             self._end()
@@ -474,7 +484,7 @@ class Conv2D(Layer):
             self.cg_x = x
         biases_vector = self.biases if self.use_bias else None
         self._op(ev.PYDTNN_OPS_FORWARD_CONVGEMM)
-        if self.model.mode == TRAIN_MODE and self.relu_above is not None:
+        if self._folds_relu_above():
             y = self._folded_forward(self.cg.conv_gemm_nchw, x, (x.shape[0], self.co, self.ho, self.wo),
                                      biases_vector)
         else:
@@ -495,7 +505,7 @@ class Conv2D(Layer):
             self._end()
         if self.need_dx:
             dx = torch.empty((dy.shape[0], self.ci, self.hi, self.wi), dtype=dy.dtype, device=dy.device)
-            gate = self.relu_below.gate_for(dx.shape) if self.relu_below is not None else None
+            gate = self._gate_below(dx.shape)
             self._op(ev.PYDTNN_OPS_BACKWARD_DECONV_GEMM)
             self.cg.deconv_gemm_nchw(self.weights, dy, dx, gate=gate, **self._cg_kwargs())
             self._end()
@@ -593,7 +603,7 @@ class MaxPool2D(Layer):
                 bwd, dims = ops.max_pool_2d_bwd_nchw, (b, self.ci, self.hi, self.wi)
             else:
                 bwd, dims = ops.max_pool_2d_bwd_nhwc, (b, self.hi, self.wi, self.ci)
-            gate = self.relu_below.gate_for(dims) if self.relu_below is not None else None
+            gate = self._gate_below(dims)
             dx = bwd(dy, self.idx_max, *dims, *self._geom(), gate=gate)
             if gate is not None:
                 self.relu_below.take_gated(dx)

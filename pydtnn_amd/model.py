@@ -38,12 +38,13 @@ _DEFAULTS = dict(
     enable_fused_conv_relu=False,
     enable_fused_conv_bn=False,
     enable_fused_conv_bn_relu=False,
-    # Not a reference flag.  In TRAIN_MODE a Relu layer of the top-level sequence is computed by the stores of
-    # its neighbours (the convolution before it, the convolution or pooling layer after it) instead of by two
-    # passes of its own.  Losses, gradients, masks and updated weights are bit-identical either way; what
-    # changes is visible only between the layers: the convolution's forward returns the rectified tensor and
-    # the layer above the Relu returns a dx already multiplied by the mask.  Off by default for that reason.
-    enable_relu_folding=False,
+    # Not a reference flag.  Inside train_batch a Relu layer of the top-level sequence is computed by the stores
+    # of its neighbours (the convolution before it, the convolution or pooling layer after it) instead of by
+    # two passes of its own.  Losses, gradients, masks and updated weights are bit-identical either way; what
+    # changes is visible only between the layers of that loop (the convolution hands the Relu layer a tensor it
+    # has already rectified, the layer above the Relu a dx already multiplied by the mask), and a layer's
+    # forward / backward called outside train_batch never does it.  False restores the separate passes.
+    enable_relu_folding=True,
 )
 
 
@@ -78,6 +79,7 @@ class Model:
         self.tensor_format = PYDTNN_TENSOR_FORMAT_NHWC if fmt == "NHWC" else PYDTNN_TENSOR_FORMAT_NCHW
         self.batch_size = self.kwargs["batch_size"]
         self._fused = False
+        self.stepping = False  # True while train_batch runs its own forward / backward loops
         # pydtnn/model.py:216-218: without the flag every BestOf just calls its first alternative
         BestOf.use_always_the_first_alternative(not self.kwargs["enable_best_of"])
 
@@ -191,15 +193,19 @@ class Model:
         if global_batch_size is None:
             global_batch_size = x.shape[0]
         emit = self.tracer.emit_event
-        for i in range(1, len(self.layers)):
-            emit(PYDTNN_MDL_EVENT, self.layers[i].id * PYDTNN_MDL_EVENTS + PYDTNN_MDL_FORWARD)
-            x = self.layers[i].forward(x)
-            emit(PYDTNN_MDL_EVENT, 0)
-        loss, dx = loss_func(x, y_targ, global_batch_size)
-        for i in range(len(self.layers) - 1, 0, -1):
-            emit(PYDTNN_MDL_EVENT, self.layers[i].id * PYDTNN_MDL_EVENTS + PYDTNN_MDL_BACKWARD)
-            dx = self.layers[i].backward(dx)
-            emit(PYDTNN_MDL_EVENT, 0)
+        self.stepping = True
+        try:
+            for i in range(1, len(self.layers)):
+                emit(PYDTNN_MDL_EVENT, self.layers[i].id * PYDTNN_MDL_EVENTS + PYDTNN_MDL_FORWARD)
+                x = self.layers[i].forward(x)
+                emit(PYDTNN_MDL_EVENT, 0)
+            loss, dx = loss_func(x, y_targ, global_batch_size)
+            for i in range(len(self.layers) - 1, 0, -1):
+                emit(PYDTNN_MDL_EVENT, self.layers[i].id * PYDTNN_MDL_EVENTS + PYDTNN_MDL_BACKWARD)
+                dx = self.layers[i].backward(dx)
+                emit(PYDTNN_MDL_EVENT, 0)
+        finally:
+            self.stepping = False
         for i in range(len(self.layers) - 1, 0, -1):
             self.layers[i].reduce_weights_sync()
             emit(PYDTNN_MDL_EVENT, self.layers[i].id * PYDTNN_MDL_EVENTS + PYDTNN_MDL_UPDATE_DW)

@@ -394,19 +394,30 @@ def test_relu_folding_changes_no_bit_of_a_training_run(pd, fmt, monkeypatch):
     assert calls_a == {"fwd": 2, "bwd": 2}   # only the Relu between the FC layers
 
 
-def test_relu_layer_called_by_hand_ignores_a_stale_hand_over(pd):
-    """The hand-over is recognised by tensor identity: a Relu given any other tensor computes normally."""
-    model = pd.Model(tensor_format="NCHW", batch_size=2, enable_relu_folding=True)
+def test_relu_folding_stays_inside_the_training_step(pd):
+    """Outside train_batch a convolution's forward returns conv(x) + b as the reference's does, whatever follows
+    it in the model; and the hand-over is recognised by tensor identity: a Relu given any other tensor
+    computes normally and drops it."""
+    model = pd.Model(tensor_format="NCHW", batch_size=2)
+    assert model.enable_relu_folding
     model.add(pd.Input(shape=(6, 6, 2)))
     model.add(pd.Conv2D(nfilters=3, filter_shape=(3, 3), padding=1, activation="relu"))
     model.mode = pd.TRAIN_MODE
     conv, relu = model.layers[1], model.layers[2]
     assert conv.relu_above is relu
-    y = conv.forward(torch.randn(2, 2, 6, 6, device="cuda"))       # hands (y, mask) to relu
+    x = torch.randn(2, 2, 6, 6, device="cuda")
+    y_plain = conv.forward(x)                                      # by hand: not rectified, nothing handed over
+    assert bool((y_plain < 0).any()) and relu._folded is None
+    model.stepping = True                                          # as train_batch's loop sets it
+    try:
+        y = conv.forward(x)                                        # hands (y, mask) to relu
+    finally:
+        model.stepping = False
+    assert torch.equal(y, torch.clamp(y_plain, min=0)) and relu._folded is not None
     other = torch.randn(2, 3, 6, 6, device="cuda")
-    out = relu.forward(other)                                       # ... which must not use it for `other`
+    out = relu.forward(other)                                      # ... which must not use it for `other`
     assert torch.equal(out, torch.clamp(other, min=0)) and torch.equal(relu.mask, (other > 0).to(torch.int8))
-    assert relu.forward(y) is not y                                 # the hand-over was dropped, not kept
+    assert relu.forward(y) is not y                                # the hand-over was dropped, not kept
 
 
 # ------------------------------------------------------------------ BatchNormalization in training mode
