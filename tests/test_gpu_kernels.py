@@ -155,8 +155,12 @@ def test_im2col_unaligned_column_count(ops, oracle):
 
 
 def test_unsupported_dtype_raises(ops):
+    """float32 and float64 have kernels; anything else, and a mix of the two, is refused."""
     with pytest.raises(TypeError):
-        ops.im2col_nchw(torch.zeros((1, 1, 4, 4), dtype=torch.float64, device="cuda"), 3, 3, 0, 0, 1, 1, 1, 1)
+        ops.im2col_nchw(torch.zeros((1, 1, 4, 4), dtype=torch.float16, device="cuda"), 3, 3, 0, 0, 1, 1, 1, 1)
+    with pytest.raises(TypeError):
+        ops.matmul(torch.zeros((4, 4), dtype=torch.float32, device="cuda"),
+                   torch.zeros((4, 4), dtype=torch.float64, device="cuda"))
 
 
 # ------------------------------------------------------------------ GEMM
