@@ -2,7 +2,7 @@
 oracle's float64 functions on the same seeded inputs.
 
 Bar: bit-exact for the index-only kernels (their float64 sums follow the reference's order); max |a - b| / max |b|
-<= 1e-10, the task's float64 tolerance, for everything that goes through a GEMM (measured around 1e-15).
+<= 1e-10, the float64 tolerance of this path, for everything that goes through a GEMM (measured around 1e-15).
 """
 import numpy as np
 import pytest
