@@ -277,6 +277,45 @@ def test_wide_unpadded_filter_rows_nchw(cg, oracle, d):
         assert_close(y2, ref2, what="y with an unused non-finite column")
 
 
+# unpadded NCHW first layers with 96 filters and 3 x 11 x 11 taps that take the NCHW streaming kernel (filter
+# matrix resident in LDS, at least 32768 output pixels): AlexNet's, then strides 2 x 3 on a non-square image whose
+# planes end inside a unit of 32 pixels, then dilation 2 x 1
+stream_nchw_grid = [
+    D(11, 3, 227, 227, 96, 11, 11, 0, 0, 4, 4, 1, 1),
+    D(15, 3, 120, 131, 96, 11, 11, 0, 0, 2, 3, 1, 1),
+    D(9, 3, 140, 90, 96, 11, 11, 0, 0, 2, 1, 2, 1),
+]
+
+
+@pytest.mark.parametrize("d", stream_nchw_grid, ids=repr)
+def test_streaming_kernel_shapes_nchw(cg, oracle, d):
+    """Forward alone, with bias, with bias + BN + ReLU, and with the ReLU mask of the folded training step."""
+    announce("stream shapes nchw", d)
+    assert d.b * d.ho * d.wo >= 32768
+    x, w, b, _ = case(d)
+    rng = np.random.default_rng(10)
+    bn = [rng.uniform(0.5, 1.5, d.kn).astype(np.float32) for _ in range(4)]
+    ref = _fwd_ref(oracle, x, w, b, d)
+    xd, wd, bd = dev(x), dev(w), dev(b)
+    y = cg.conv_gemm_nchw(wd, xd, **_kw(d))
+    assert_close(host(y), ref - b.reshape(1, -1, 1, 1), what="y without bias")
+    y = cg.conv_gemm_nchw(wd, xd, biases_vector=bd, **_kw(d))
+    assert_close(host(y), ref, what="y")
+    y_bn = cg.conv_gemm_nchw(wd, xd, biases_vector=bd, bn_running_mean=dev(bn[0]), bn_inv_std=dev(bn[1]),
+                             bn_gamma=dev(bn[2]), bn_beta=dev(bn[3]), relu=True, **_kw(d))
+    assert_close(host(y_bn), oracle.fused_epilogue(ref, "NCHW", bn=bn, relu_flag=True), what="fused y")
+    y_relu = torch.full(y.shape, np.nan, device="cuda")
+    mask = torch.full(y.shape, 7, dtype=torch.int8, device="cuda")
+    cg.conv_gemm_nchw(wd, xd, biases=y_relu, biases_vector=bd, relu=True, relu_mask=mask, **_kw(d))
+    assert torch.equal(y_relu, torch.clamp(y, min=0)) and torch.equal(mask, (y > 0).to(torch.int8))
+    # non-finite values where no window reaches (the last columns at these strides) must not leak in
+    if (d.w - d.hdilation * (d.kw - 1) - 1) % d.hstride != 0:
+        x2 = x.copy()
+        x2[:, :, :, d.w - 1] = np.inf
+        y2 = host(cg.conv_gemm_nchw(wd, dev(x2), biases_vector=bd, **_kw(d)))
+        assert np.array_equal(y2, host(y))
+
+
 @pytest.mark.parametrize("x,w,stride", [
     (x_2x4, w_1x1, 1), (x_2x4, w_1x2, 1), (x_2x4, w_2x2, 1), (x_4x4, w_2x2, 2), (x_4x8, w_2x2, (1, 2)),
     (x_8x8, w_3x3, 3), (x_8x8, w_2x2, 1), (x_2x4_c2, w_c2_1234_4567, 1)])
