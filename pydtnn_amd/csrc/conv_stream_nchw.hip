@@ -44,7 +44,7 @@ typedef uint32_t uintx4 __attribute__((ext_vector_type(4)));
 
 // MB: filters / 32;  CHUNKS: chunks of 16 reduction indices (kh*kw*c rounded up);  WAVES: wavefronts of the
 // workgroup, 12 (168 registers) or 16 (128 registers; same code, no spills).
-template <int MB, int CHUNKS, int MASKS, int WAVES>
+template <int MB, int CHUNKS, int MASKS, int WAVES, bool PAD>
 __global__ void __launch_bounds__(64 * WAVES) conv_stream_nchw_kernel(StreamNchwArgs a)
 {
     constexpr int KN = 32 * MB, GROUPS = CHUNKS * 2, SLOTS = CHUNKS * 16;
@@ -55,7 +55,9 @@ __global__ void __launch_bounds__(64 * WAVES) conv_stream_nchw_kernel(StreamNchw
     floatx4* wl = reinterpret_cast<floatx4*>(lds);
     // tap offsets in bytes: quad [group*2 + h] holds those of the same four taps
     uintx4* toff = reinterpret_cast<uintx4*>(lds + (size_t)GROUPS * 2 * KN * 4);
-    float* params = lds + (size_t)GROUPS * 2 * KN * 4 + GROUPS * 2 * 4;  // [5][KN]
+    // with padding: the taps' row / column bits (1 << i) | (1 << (16 + j)), laid out like the offsets
+    [[maybe_unused]] uintx4* tbits = toff + GROUPS * 2;
+    float* params = lds + (size_t)GROUPS * 2 * KN * 4 + GROUPS * 2 * 4 * 2;  // [5][KN]
     int* counter = reinterpret_cast<int*>(params + 5 * KN);
 
     const int tid = threadIdx.x, lane = tid & 63, wave = uniform(tid >> 6);
@@ -89,14 +91,16 @@ __global__ void __launch_bounds__(64 * WAVES) conv_stream_nchw_kernel(StreamNchw
         }
         uint32_t* tf = reinterpret_cast<uint32_t*>(toff);
         for (int s = tid; s < SLOTS; s += kThreadsNchw) {
-            uint32_t off = kOob;
+            uint32_t off = kOob, bits = 0;
             if (s < g.k) {
                 const int cc = (int)fd_div((uint32_t)s, g.fd_khw), rem = s - cc * g.khw;
                 const int ti = (int)fd_div((uint32_t)rem, g.fd_kw), tj = rem - ti * g.kw;
                 off = (uint32_t)(((long)cc * g.h + ti * g.vdilation) * g.w + tj * g.hdilation) * 4u;
+                bits = (1u << ti) | (1u << (16 + tj));
             }
             const int m = s >> 1, h = s & 1;
             tf[((m >> 2) * 2 + h) * 4 + (m & 3)] = off;
+            if constexpr (PAD) tf[GROUPS * 2 * 4 + ((m >> 2) * 2 + h) * 4 + (m & 3)] = bits;
         }
         for (int i = tid; i < KN; i += kThreadsNchw) {
             params[i] = a.chan.bias ? a.chan.bias[i] : 0.0f;
@@ -116,21 +120,49 @@ __global__ void __launch_bounds__(64 * WAVES) conv_stream_nchw_kernel(StreamNchw
     [[maybe_unused]] rsrc_t mask_rsrc;
     if constexpr (MASKS == kReluMask) mask_rsrc = make_rsrc_bytes(a.masks.relu_mask, y_floats);
 
-    // byte offset of this lane's pixel of a unit at tap (0, 0, 0), or kDead when the unit ends before it
-    auto pixel_base = [&](int unit) __attribute__((always_inline)) -> uint32_t {
+    // Per-lane data of a unit.  Without padding: `base` is the byte offset of the lane's pixel at tap (0, 0, 0), or
+    // kDead when the plane ends before it.  With padding: the same offset (which may be "negative", i.e. wrap), and
+    // `bad` holds bit i for every filter row i and bit 16 + j for every filter column j that falls outside the
+    // image for this pixel (all ones beyond the end of the plane): a tap is read when bad & its bits == 0.
+    struct Lane {
+        uint32_t base;
+        uint32_t bad;
+    };
+    auto pixel_lane = [&](int unit) __attribute__((always_inline)) -> Lane {
         const int gu = u0 + unit;
         const int img = gu / a.units_per_image;
         const int p = (gu - img * a.units_per_image) * 32 + lp;
         const uint32_t oy = fd_div((uint32_t)p, g.fd_wo), ox = (uint32_t)p - oy * (uint32_t)g.wo;
-        const uint32_t off = (uint32_t)(((long)img * g.c * g.h + oy * g.vstride) * g.w + ox * g.hstride) * 4u;
-        return p < g.howo ? off : kDead;
+        const int ih0 = (int)oy * g.vstride - g.vpadding, iw0 = (int)ox * g.hstride - g.hpadding;
+        Lane l;
+        l.base = (uint32_t)(((long)img * g.c * g.h + ih0) * g.w + iw0) * 4u;
+        l.bad = 0;
+        if constexpr (PAD) {
+            for (int t = 0; t < g.kh; ++t)
+                if ((unsigned)(ih0 + t * g.vdilation) >= (unsigned)g.h) l.bad |= 1u << t;
+            for (int t = 0; t < g.kw; ++t)
+                if ((unsigned)(iw0 + t * g.hdilation) >= (unsigned)g.w) l.bad |= 1u << (16 + t);
+            if (p >= g.howo) l.bad = 0xffffffffu;
+        } else {
+            if (p >= g.howo) l.base = kDead;
+        }
+        return l;
     };
-    auto load_chunk = [&](uint32_t base, int chunk, float (&r)[8]) __attribute__((always_inline)) {
+    const Lane dead_lane = {kDead, 0xffffffffu};
+    auto load_chunk = [&](const Lane& l, int chunk, float (&r)[8]) __attribute__((always_inline)) {
 #pragma unroll
         for (int gg = 0; gg < 2; ++gg) {
             const uintx4 t = toff[(chunk * 2 + gg) * 2 + lh];
+            [[maybe_unused]] uintx4 tb;
+            if constexpr (PAD) tb = tbits[(chunk * 2 + gg) * 2 + lh];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) r[gg * 4 + i] = buf_load(x_rsrc, base + t[i], 0);
+            for (int i = 0; i < 4; ++i) {
+                uint32_t voff = l.base + t[i];
+                // a reduction slot beyond the last tap has no bits and the offset kOob, which stays beyond the
+                // descriptor for every base (|base| < 2^30)
+                if constexpr (PAD) voff = (l.bad & tb[i]) != 0 ? kOob : voff;
+                r[gg * 4 + i] = buf_load(x_rsrc, voff, 0);
+            }
         }
     };
     auto claim = [&]() __attribute__((always_inline)) -> int {
@@ -180,8 +212,8 @@ __global__ void __launch_bounds__(64 * WAVES) conv_stream_nchw_kernel(StreamNchw
     floatx16 acc[MB];
     int cur = wave < units ? wave : -1;
     if (cur < 0) return;
-    uint32_t base = pixel_base(cur);
-    load_chunk(base, 0, bbuf[0]);
+    Lane ln = pixel_lane(cur);
+    load_chunk(ln, 0, bbuf[0]);
     const floatx4* wq0 = wl + (size_t)lh * KN + lp;
 
     // One unit, straight-line: chunk ch is consumed from bbuf[(P0 + ch) & 1] while the next chunk (of this unit, or
@@ -189,14 +221,14 @@ __global__ void __launch_bounds__(64 * WAVES) conv_stream_nchw_kernel(StreamNchw
     auto unit_body = [&](auto parity_tag) __attribute__((always_inline)) {
         constexpr int P0 = decltype(parity_tag)::value;
         const int next = claim();
-        const uint32_t base_next = next >= 0 ? pixel_base(next) : kDead;
+        const Lane ln_next = next >= 0 ? pixel_lane(next) : dead_lane;
 #pragma unroll
         for (int ch = 0; ch < CHUNKS; ++ch) {
             const int B = (P0 + ch) & 1;
             if (ch + 1 < CHUNKS)
-                load_chunk(base, ch + 1, bbuf[B ^ 1]);
+                load_chunk(ln, ch + 1, bbuf[B ^ 1]);
             else
-                load_chunk(base_next, 0, bbuf[B ^ 1]);
+                load_chunk(ln_next, 0, bbuf[B ^ 1]);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int gg = 0; gg < 2; ++gg) {
@@ -225,7 +257,7 @@ __global__ void __launch_bounds__(64 * WAVES) conv_stream_nchw_kernel(StreamNchw
         case 6: store_unit(std::integral_constant<int, 6>{}, acc, cur); break;
         default: store_unit(std::integral_constant<int, 7>{}, acc, cur); break;
         }
-        base = base_next;
+        ln = ln_next;
         cur = next;
     };
 
@@ -244,16 +276,16 @@ __global__ void __launch_bounds__(64 * WAVES) conv_stream_nchw_kernel(StreamNchw
 template <int MB, int CHUNKS>
 constexpr size_t stream_nchw_lds_bytes()
 {
-    return ((size_t)CHUNKS * 2 * 2 * 32 * MB * 4 + CHUNKS * 2 * 2 * 4 + 5 * 32 * MB) * 4 + 16;
+    return ((size_t)CHUNKS * 2 * 2 * 32 * MB * 4 + CHUNKS * 2 * 2 * 4 * 2 + 5 * 32 * MB) * 4 + 16;
 }
 
-template <int MB, int CHUNKS, int MASKS, int WAVES>
+template <int MB, int CHUNKS, int MASKS, int WAVES, bool PAD>
 int launch_stream_nchw_waves(const StreamNchwArgs& a, int grid, hipStream_t stream)
 {
     static bool attr_set = false;
     constexpr size_t lds_bytes = stream_nchw_lds_bytes<MB, CHUNKS>();
     static_assert(lds_bytes <= 160 * 1024, "filter matrix must fit LDS");
-    auto kernel = conv_stream_nchw_kernel<MB, CHUNKS, MASKS, WAVES>;
+    auto kernel = conv_stream_nchw_kernel<MB, CHUNKS, MASKS, WAVES, PAD>;
     if (!attr_set) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 160 * 1024) != hipSuccess)
@@ -265,7 +297,7 @@ int launch_stream_nchw_waves(const StreamNchwArgs& a, int grid, hipStream_t stre
     return PYDTNN_HIP_OK;
 }
 
-template <int MB, int CHUNKS, int MASKS>
+template <int MB, int CHUNKS, int MASKS, bool PAD>
 int launch_stream_nchw(const StreamNchwArgs& a, hipStream_t stream)
 {
     static int cus = 0;
@@ -280,29 +312,33 @@ int launch_stream_nchw(const StreamNchwArgs& a, hipStream_t stream)
     // idle slots in the last round (24 units: two full rounds of 12, but 32 slots of 16).
     const int per_wg = (a.units + grid - 1) / grid;
     const int slots16 = (per_wg + 15) / 16 * 16, slots12 = (per_wg + 11) / 12 * 12;
-    if (slots12 < slots16) return launch_stream_nchw_waves<MB, CHUNKS, MASKS, 12>(a, grid, stream);
-    return launch_stream_nchw_waves<MB, CHUNKS, MASKS, 16>(a, grid, stream);
+    if (slots12 < slots16) return launch_stream_nchw_waves<MB, CHUNKS, MASKS, 12, PAD>(a, grid, stream);
+    return launch_stream_nchw_waves<MB, CHUNKS, MASKS, 16, PAD>(a, grid, stream);
 }
 
-// The (filters / 32, chunks of 16 reduction indices) pairs that are built: AlexNet's first layer
-// (96 filters, 3 x 11 x 11 = 363 taps).
-bool stream_nchw_shape_built(int kn, int k)
+// The (filters, chunks of 16 reduction indices, padded?) triples that are built: AlexNet's first layer (96 filters,
+// 3 x 11 x 11 = 363 taps, no padding), VGG's (64 filters, 3 x 3 x 3 = 27 taps, padded) and ResNet's (64 filters,
+// 3 x 7 x 7 = 147 taps, padded).
+bool stream_nchw_shape_built(int kn, int k, bool padded)
 {
     const int chunks = (k + 15) / 16;
-    return kn == 96 && chunks == 23;
+    if (!padded) return kn == 96 && chunks == 23;
+    return kn == 64 && (chunks == 2 || chunks == 10);
 }
 
 }  // namespace
 
 bool conv_stream_nchw_eligible(const ConvGeom& g, const ElemMasks& masks)
 {
-    if (!stream_nchw_shape_built(g.kn, g.k)) return false;
-    if (g.vpadding != 0 || g.hpadding != 0) return false;  // taps never leave the image
+    const bool padded = g.vpadding != 0 || g.hpadding != 0;
+    if (!stream_nchw_shape_built(g.kn, g.k, padded)) return false;
+    if (padded && (g.kh > 16 || g.kw > 16)) return false;  // row and column bits share one word
     const int mk = mask_kind(masks);
     if (mk != kNoMasks && mk != kReluMask) return false;
     if (g.p < 32 * 1024) return false;                      // enough units for every compute unit
-    // offsets of valid loads stay below kDead, and the descriptors below 1 GiB
-    return (long)g.n * g.c * g.h * g.w < (1l << 28) && g.p * g.kn < (1l << 28);
+    // every byte offset the kernel forms stays below 2^30 in magnitude, and so do the descriptors
+    const long reach = (long)g.n * g.c * g.h * g.w + ((long)g.vpadding + 1) * g.w + g.hpadding;
+    return reach < (1l << 28) && g.p * g.kn < (1l << 28);
 }
 
 int conv_stream_nchw(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan,
@@ -314,11 +350,14 @@ int conv_stream_nchw(const ConvGeom& g, const float* w, const float* x, float* y
     a.units = g.n * a.units_per_image;
     const int chunks = (g.k + 15) / 16;
     const bool mask = mask_kind(masks) == kReluMask;
-#define STREAM_NCHW_CASE(KN, CH)                                                              \
-    if (g.kn == KN && chunks == CH)                                                           \
-        return mask ? launch_stream_nchw<KN / 32, CH, kReluMask>(a, stream)                   \
-                    : launch_stream_nchw<KN / 32, CH, kNoMasks>(a, stream)
-    STREAM_NCHW_CASE(96, 23);
+    const bool padded = g.vpadding != 0 || g.hpadding != 0;
+#define STREAM_NCHW_CASE(KN, CH, PAD)                                                         \
+    if (g.kn == KN && chunks == CH && padded == PAD)                                          \
+        return mask ? launch_stream_nchw<KN / 32, CH, kReluMask, PAD>(a, stream)              \
+                    : launch_stream_nchw<KN / 32, CH, kNoMasks, PAD>(a, stream)
+    STREAM_NCHW_CASE(96, 23, false);
+    STREAM_NCHW_CASE(64, 2, true);
+    STREAM_NCHW_CASE(64, 10, true);
 #undef STREAM_NCHW_CASE
     return PYDTNN_HIP_ERR_UNSUPPORTED;
 }

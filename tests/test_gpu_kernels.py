@@ -277,13 +277,20 @@ def test_wide_unpadded_filter_rows_nchw(cg, oracle, d):
         assert_close(y2, ref2, what="y with an unused non-finite column")
 
 
-# unpadded NCHW first layers with 96 filters and 3 x 11 x 11 taps that take the NCHW streaming kernel (filter
-# matrix resident in LDS, at least 32768 output pixels): AlexNet's, then strides 2 x 3 on a non-square image whose
-# planes end inside a unit of 32 pixels, then dilation 2 x 1
+# NCHW first layers that take the NCHW streaming kernel (filter matrix resident in LDS, at least 32768 output
+# pixels).  Unpadded, 96 filters, 3 x 11 x 11 taps: AlexNet's, then strides 2 x 3 on a non-square image whose planes
+# end inside a unit of 32 pixels, then dilation 2 x 1.  Padded, 64 filters, 17 .. 32 taps (VGG's 3 x 3 x 3, with
+# ragged planes, mixed padding and stride, dilation, one channel of 5 x 5) and 145 .. 160 taps (ResNet's 3 x 7 x 7).
 stream_nchw_grid = [
     D(11, 3, 227, 227, 96, 11, 11, 0, 0, 4, 4, 1, 1),
     D(15, 3, 120, 131, 96, 11, 11, 0, 0, 2, 3, 1, 1),
     D(9, 3, 140, 90, 96, 11, 11, 0, 0, 2, 1, 2, 1),
+    D(2, 3, 224, 224, 64, 3, 3, 1, 1, 1, 1, 1, 1),
+    D(20, 3, 50, 47, 64, 3, 3, 1, 1, 1, 1, 1, 1),
+    D(20, 3, 57, 61, 64, 3, 3, 2, 0, 1, 2, 1, 1),
+    D(3, 3, 130, 130, 64, 3, 3, 2, 2, 1, 1, 2, 2),
+    D(4, 1, 120, 120, 64, 5, 5, 2, 2, 1, 1, 1, 1),
+    D(3, 3, 224, 224, 64, 7, 7, 3, 3, 2, 2, 1, 1),
 ]
 
 
@@ -308,8 +315,8 @@ def test_streaming_kernel_shapes_nchw(cg, oracle, d):
     mask = torch.full(y.shape, 7, dtype=torch.int8, device="cuda")
     cg.conv_gemm_nchw(wd, xd, biases=y_relu, biases_vector=bd, relu=True, relu_mask=mask, **_kw(d))
     assert torch.equal(y_relu, torch.clamp(y, min=0)) and torch.equal(mask, (y > 0).to(torch.int8))
-    # non-finite values where no window reaches (the last columns at these strides) must not leak in
-    if (d.w - d.hdilation * (d.kw - 1) - 1) % d.hstride != 0:
+    # non-finite values where no window reaches (the last column at some of these strides) must not leak in
+    if (d.wo - 1) * d.hstride - d.hpadding + d.hdilation * (d.kw - 1) < d.w - 1:
         x2 = x.copy()
         x2[:, :, :, d.w - 1] = np.inf
         y2 = host(cg.conv_gemm_nchw(wd, dev(x2), biases_vector=bd, **_kw(d)))
