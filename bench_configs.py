@@ -261,7 +261,7 @@ def run_cfg3(torch, pd, timed_steps, steps, warmup):
     ms, _ = timed_steps(torch, step, steps, warmup)
     flop = 2.0 * 96 * 363 * 64 * 55 * 55
     tf = flop / (ms * 1e-3) / 1e12
-    roofline = {"bound": "mfma", "kernel": "implicit GEMM on 96-row tiles, Im2colNchwMN, EpiNchw (bias + ReLU)",
+    roofline = {"bound": "mfma", "kernel": "conv_stream_nchw_kernel<3, 23> (filter matrix in LDS, bias + ReLU in the store)",
                 "achieved": round(tf, 3), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(tf / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": None}
     workload = ("cfg3: AlexNet conv1 forward + fused bias + ReLU, fp32 NCHW, N=64, 3x227x227 -> 96, 11x11, "
