@@ -557,6 +557,40 @@ __global__ void __launch_bounds__(kThreads) max_pool_bwd_windows_nchw_kernel(con
     }
 }
 
+// The same for 2 x 2 windows with an even number of windows per row: one thread owns two neighbouring windows
+// and writes their four columns of both rows as one 128-bit store each (indices and gradients arrive as 64-bit
+// loads, gate bytes as one 32-bit load per row).
+__global__ void __launch_bounds__(kThreads) max_pool_bwd_window_pairs_nchw_kernel(const float2* __restrict__ dy,
+                                                                                 const int2* __restrict__ idx_max,
+                                                                                 float4* __restrict__ dx, ConvGeom g,
+                                                                                 const uint32_t* __restrict__ gate)
+{
+    const uint32_t pairs = (uint32_t)g.howo >> 1, half_wo = (uint32_t)g.wo >> 1;
+    const uint32_t pr = blockIdx.x * kThreads + threadIdx.x;
+    if (pr >= pairs) return;
+    const uint32_t oy = pr / half_wo, px = pr - oy * half_wo;
+    const uint32_t planes = (uint32_t)(g.n * g.c);
+    const size_t plane_quads = (size_t)g.h * g.w / 4, row_quads = (size_t)g.w / 4;
+    for (uint32_t plane = blockIdx.y; plane < planes; plane += gridDim.y) {
+        const int2 rec = idx_max[(size_t)plane * pairs + pr];
+        const float2 gr = dy[(size_t)plane * pairs + pr];
+        const float g0 = 0.0f + gr.x, g1 = 0.0f + gr.y;
+        const size_t first = (size_t)plane * plane_quads + (size_t)(2 * oy) * row_quads + px;
+#pragma unroll
+        for (int ii = 0; ii < 2; ++ii) {
+            // the reference's decode for 2 x 2 windows: row = idx / 2, column = idx % 2
+            float4 v = make_float4(rec.x == 2 * ii ? g0 : 0.0f, rec.x == 2 * ii + 1 ? g0 : 0.0f,
+                                   rec.y == 2 * ii ? g1 : 0.0f, rec.y == 2 * ii + 1 ? g1 : 0.0f);
+            if (gate) {
+                const uint32_t gt = gate[first + ii * row_quads];
+                v.x *= (float)(int8_t)(gt & 0xff); v.y *= (float)(int8_t)((gt >> 8) & 0xff);
+                v.z *= (float)(int8_t)((gt >> 16) & 0xff); v.w *= (float)(int8_t)(gt >> 24);
+            }
+            dx[first + ii * row_quads] = v;
+        }
+    }
+}
+
 // Output rows (or columns) whose window covers input coordinate `t = coord + padding`, for windows of `k` taps at
 // stride `stride` without dilation: [lo, hi], empty when lo > hi.
 __device__ __forceinline__ void pool_window_range(int t, int k, int stride, const FastDiv fd_stride, int extent,
@@ -1471,7 +1505,14 @@ int launch_max_pool_bwd_nchw(const float* dy, const int32_t* idx_max, float* dx,
                        g.hpadding == 0 && g.vdilation == 1 && g.hdilation == 1;
     if (tiled && g.h == g.ho * g.kh && g.w == g.wo * g.kw) {
         dim3 wgrid(blocks_for(g.howo), (unsigned)(planes < 65535 ? planes : 65535));
-        if (g.kw == 2 && (reinterpret_cast<uintptr_t>(dx) & 7) == 0)
+        const uintptr_t all = reinterpret_cast<uintptr_t>(dx) | reinterpret_cast<uintptr_t>(dy) |
+                              reinterpret_cast<uintptr_t>(idx_max) | reinterpret_cast<uintptr_t>(gate);
+        if (g.kw == 2 && g.wo % 2 == 0 && (all & 15) == 0 && g.howo / 2 < (1 << 30)) {
+            dim3 pgrid(blocks_for(g.howo / 2), wgrid.y);
+            hipLaunchKernelGGL(max_pool_bwd_window_pairs_nchw_kernel, pgrid, dim3(kThreads), 0, stream,
+                               reinterpret_cast<const float2*>(dy), reinterpret_cast<const int2*>(idx_max),
+                               reinterpret_cast<float4*>(dx), g, reinterpret_cast<const uint32_t*>(gate));
+        } else if (g.kw == 2 && (reinterpret_cast<uintptr_t>(dx) & 7) == 0)
             hipLaunchKernelGGL(max_pool_bwd_windows_nchw_kernel<2>, wgrid, dim3(kThreads), 0, stream, dy, idx_max, dx,
                                g, gate);
         else

@@ -567,7 +567,8 @@ def test_bias_grad_of_a_row_matrix(ops, rows, channels):
 def test_maxpool_matches_oracle(ops, oracle):
     rng = np.random.default_rng(10)
     for (shape, k, s, p) in [((2, 3, 8, 10), 2, 2, 0), ((2, 4, 9, 9), 3, 2, 1), ((1, 2, 7, 7), 3, 1, 1),
-                             ((2, 3, 9, 11), 2, 2, 0), ((1, 2, 9, 12), 3, 3, 0), ((3, 5, 14, 14), 2, 2, 0)]:
+                             ((2, 3, 9, 11), 2, 2, 0), ((1, 2, 9, 12), 3, 3, 0), ((3, 5, 14, 14), 2, 2, 0),
+                             ((2, 3, 8, 12), 2, 2, 0), ((3, 5, 16, 32), 2, 2, 0)]:  # the last two: pairs of windows
         announce("maxpool", shape, k, s, p)
         x = rng.standard_normal(shape).astype(np.float32)
         x[0, 0, :2, :2] = 1.5  # ties: the first tap must win
@@ -931,7 +932,8 @@ def test_maxpool_backward_with_gate_equals_backward_then_relu_backward(ops):
     rng = np.random.default_rng(12)
     for (shape, kh, kw, s, p) in [((2, 3, 8, 10), 2, 2, 2, 0), ((2, 4, 9, 9), 3, 3, 2, 1), ((2, 3, 9, 11), 2, 2, 2, 0),
                                   ((1, 2, 9, 12), 3, 3, 3, 0), ((3, 5, 14, 14), 2, 2, 2, 0), ((2, 3, 8, 9), 2, 3, 2, 0), ((2, 4, 8, 10), 2, 2, 2, 0),
-                                  ((2, 8, 9, 12), 3, 3, 3, 0), ((1, 64, 6, 6), 2, 2, 2, 0)]:
+                                  ((2, 8, 9, 12), 3, 3, 3, 0), ((1, 64, 6, 6), 2, 2, 2, 0), ((2, 3, 8, 12), 2, 2, 2, 0),
+                                  ((3, 5, 16, 32), 2, 2, 2, 0)]:
         announce("gated maxpool bwd", shape, kh, kw, s, p)
         x = rng.standard_normal(shape).astype(np.float32)
         gate = dev((rng.random(shape) < 0.6).astype(np.int8))
