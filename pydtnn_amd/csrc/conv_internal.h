@@ -3,6 +3,7 @@
 #pragma once
 #include "../../include/pydtnn_hip.h"
 #include "gemm_engine.h"
+#include <atomic>
 
 int launch_im2col_nchw(const float*, float*, const ConvGeom&, hipStream_t);
 int launch_col2im_nchw(const float*, float*, const ConvGeom&, hipStream_t);

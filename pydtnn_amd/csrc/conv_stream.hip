@@ -312,20 +312,13 @@ __global__ void __launch_bounds__(64 * stream_waves(CHUNKS, MASKS)) conv_stream_
 template <int N, int NB, int CHUNKS, int MASKS>
 int launch_stream(const StreamArgs& a, hipStream_t stream)
 {
-    static int cus = 0;
-    static bool attr_set = false;
+    static std::atomic<unsigned> raised{0};
     const size_t lds_bytes = ((size_t)a.g.k * N + 5 * N) * 4 + 16;
     auto kernel = conv_stream_nhwc_kernel<N, NB, CHUNKS, MASKS>;
-    if (!attr_set) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                160 * 1024) != hipSuccess)
-            return PYDTNN_HIP_ERR_LAUNCH;
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess ||
-            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-            return PYDTNN_HIP_ERR_LAUNCH;
-        attr_set = true;
-    }
+    int cus = 0;
+    int rc = raise_lds_limit(reinterpret_cast<const void*>(kernel), raised, 160 * 1024);
+    if (rc == PYDTNN_HIP_OK) rc = device_compute_units(&cus);
+    if (rc != PYDTNN_HIP_OK) return rc;
     const int grid = a.row_blocks < cus ? a.row_blocks : cus;
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(64 * stream_waves(CHUNKS, MASKS)), lds_bytes, stream, a);
     HIP_RETURN_IF_LAUNCH_FAILED();

@@ -282,16 +282,12 @@ constexpr size_t stream_nchw_lds_bytes()
 template <int MB, int CHUNKS, int MASKS, int WAVES, bool PAD>
 int launch_stream_nchw_waves(const StreamNchwArgs& a, int grid, hipStream_t stream)
 {
-    static bool attr_set = false;
+    static std::atomic<unsigned> raised{0};
     constexpr size_t lds_bytes = stream_nchw_lds_bytes<MB, CHUNKS>();
     static_assert(lds_bytes <= 160 * 1024, "filter matrix must fit LDS");
     auto kernel = conv_stream_nchw_kernel<MB, CHUNKS, MASKS, WAVES, PAD>;
-    if (!attr_set) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                160 * 1024) != hipSuccess)
-            return PYDTNN_HIP_ERR_LAUNCH;
-        attr_set = true;
-    }
+    const int rc = raise_lds_limit(reinterpret_cast<const void*>(kernel), raised, 160 * 1024);
+    if (rc != PYDTNN_HIP_OK) return rc;
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(64 * WAVES), lds_bytes, stream, a);
     HIP_RETURN_IF_LAUNCH_FAILED();
     return PYDTNN_HIP_OK;
@@ -300,13 +296,9 @@ int launch_stream_nchw_waves(const StreamNchwArgs& a, int grid, hipStream_t stre
 template <int MB, int CHUNKS, int MASKS, bool PAD>
 int launch_stream_nchw(const StreamNchwArgs& a, hipStream_t stream)
 {
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess ||
-            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-            return PYDTNN_HIP_ERR_LAUNCH;
-    }
+    int cus = 0;
+    const int rc = device_compute_units(&cus);
+    if (rc != PYDTNN_HIP_OK) return rc;
     const int grid = a.units < cus ? a.units : cus;
     // A workgroup's units are taken by its wavefronts in rounds: sixteen wavefronts unless twelve leave fewer
     // idle slots in the last round (24 units: two full rounds of 12, but 32 slots of 16).

@@ -589,12 +589,10 @@ int launch_row2im_walk(const float* rows, float* dx, const ConvGeom& g, int stri
                        hipStream_t stream)
 {
     const size_t lds = (size_t)(8 * S + 2) * 32 * 9 * sizeof(float);
-    static std::atomic<bool> raised{false};
-    if (lds > 64 * 1024 && !raised.load(std::memory_order_acquire)) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&row2im_nhwc_walk_kernel<S>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-            return PYDTNN_HIP_ERR_LAUNCH;
-        raised.store(true, std::memory_order_release);
+    static std::atomic<unsigned> raised{0};
+    if (lds > 64 * 1024) {
+        const int rc = gemm::raise_lds_limit(reinterpret_cast<const void*>(&row2im_nhwc_walk_kernel<S>), raised, (int)lds);
+        if (rc != PYDTNN_HIP_OK) return rc;
     }
     const long blocks = (long)g.n * bands * strips * (g.c / 32);
     hipLaunchKernelGGL(row2im_nhwc_walk_kernel<S>, dim3((unsigned)blocks), dim3(kThreads), lds, stream, rows, dx, g,

@@ -81,6 +81,37 @@ static inline SplitInfo make_split(int seg_len, int images, int ips, int cpg, in
 
 static inline SplitInfo no_split(int k) { return make_split(k, 1, 1, 1, k); }
 
+// ---------------------------------------------------------------- host helpers
+// A kernel's dynamic LDS limit belongs to the device's copy of the kernel: raised once per device (bit `device` of
+// `done`), from any thread.
+inline int raise_lds_limit(const void* kernel, std::atomic<unsigned>& done, int bytes)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return PYDTNN_HIP_ERR_LAUNCH;
+    const unsigned bit = 1u << (dev & 31);
+    if (done.load(std::memory_order_acquire) & bit) return PYDTNN_HIP_OK;
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess)
+        return PYDTNN_HIP_ERR_LAUNCH;
+    done.fetch_or(bit, std::memory_order_release);
+    return PYDTNN_HIP_OK;
+}
+
+// Compute units of the current device (cached for the first 32 devices).
+inline int device_compute_units(int* cus)
+{
+    static std::atomic<int> cached[32];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return PYDTNN_HIP_ERR_LAUNCH;
+    int v = dev < 32 ? cached[dev].load(std::memory_order_relaxed) : 0;
+    if (v <= 0) {
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
+            return PYDTNN_HIP_ERR_LAUNCH;
+        if (dev < 32) cached[dev].store(v, std::memory_order_relaxed);
+    }
+    *cus = v;
+    return PYDTNN_HIP_OK;
+}
+
 // ---------------------------------------------------------------- buffer access
 // `p` must be wave-uniform.  `avail_elems` = floats between p and the end of the tensor.
 __device__ __forceinline__ rsrc_t make_rsrc(const float* p, long avail_elems)
