@@ -158,7 +158,8 @@ struct DgemmPlan {
 DgemmPlan plan_dgemm(long m, long n, long k)
 {
     const long tiles = ((m + kBM - 1) / kBM) * ((n + kBN - 1) / kBN);
-    long want = tiles >= 256 ? 1 : (512 + tiles - 1) / tiles;
+    // as many chunks as fill the 512 resident workgroups (two per CU) once: a few more would run alone in a second round
+    long want = tiles >= 256 ? 1 : 512 / tiles;
     long chunk = ((k + want - 1) / want + 15) / 16 * 16;
     if (chunk < 256) chunk = 256;
     if (chunk > k) chunk = (k + 15) / 16 * 16;
