@@ -169,7 +169,8 @@ inline FastDiv group_div(int seg, int ips)
 inline SplitPlan plan_plain_split(long tiles, long k, long out_elems)
 {
     SplitPlan p;
-    long want = tiles >= 256 ? 1 : (kTargetBlocks + tiles - 1) / tiles;
+    // as many chunks as fill one resident round of workgroups: a few more would run alone in a second round
+    long want = tiles >= 256 ? 1 : kTargetBlocks / tiles;
     const long max_by_ws = (long)(kMaxPartialBytes / ((size_t)out_elems * 4));
     if (want > max_by_ws) want = max_by_ws < 1 ? 1 : max_by_ws;
     long chunk = round_up((k + want - 1) / want, BK);
