@@ -291,6 +291,8 @@ stream_nchw_grid = [
     D(3, 3, 130, 130, 64, 3, 3, 2, 2, 1, 1, 2, 2),
     D(4, 1, 120, 120, 64, 5, 5, 2, 2, 1, 1, 1, 1),
     D(3, 3, 224, 224, 64, 7, 7, 3, 3, 2, 2, 1, 1),
+    D(3, 2, 120, 120, 64, 3, 3, 1, 1, 1, 1, 1, 1),
+    D(2, 27, 130, 130, 64, 1, 1, 1, 1, 1, 1, 1, 1),   # 27 taps that are channels: padded 1 x 1
 ]
 
 
