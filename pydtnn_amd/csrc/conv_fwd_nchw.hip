@@ -69,7 +69,7 @@ int conv_fwd_nchw(const ConvGeom& g, const float* w, const float* x, float* y, c
                   size_t ws_bytes, hipStream_t stream, const ElemMasks& masks)
 {
     if (!taps_supported(g)) return PYDTNN_HIP_ERR_UNSUPPORTED;
-    if (conv_stream_nchw_eligible(g, masks)) return conv_stream_nchw(g, w, x, y, chan, stream, masks);
+    if (conv_stream_first_eligible(0, g, masks)) return conv_stream_first(0, g, w, x, y, chan, stream, masks);
     return taps_wide(g) ? conv_fwd_nchw_t<true>(g, w, x, y, chan, ws, ws_bytes, stream, masks)
                         : conv_fwd_nchw_t<false>(g, w, x, y, chan, ws, ws_bytes, stream, masks);
 }

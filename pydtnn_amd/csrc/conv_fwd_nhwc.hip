@@ -43,6 +43,7 @@ int conv_fwd_nhwc_t(const ConvGeom& g, const float* w, const float* x, float* y,
 int conv_fwd_nhwc(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan, float* ws,
                   size_t ws_bytes, hipStream_t stream, const ElemMasks& masks)
 {
+    if (conv_stream_first_eligible(1, g, masks)) return conv_stream_first(1, g, w, x, y, chan, stream, masks);
     if (conv_stream_nhwc_eligible(g, w, x)) return conv_stream_nhwc(g, w, x, y, chan, stream, masks);
     if (pointwise_nhwc(g)) return conv_fwd_nhwc_pointwise(g, w, x, y, chan, ws, ws_bytes, stream, masks);
     if (!taps_supported(g)) return PYDTNN_HIP_ERR_UNSUPPORTED;

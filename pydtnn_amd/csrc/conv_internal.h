@@ -321,10 +321,10 @@ int conv_fwd_nhwc_pointwise(const ConvGeom& g, const float* w, const float* x, f
 bool conv_stream_nhwc_eligible(const ConvGeom& g, const float* w, const float* x);
 int conv_stream_nhwc(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan,
                      hipStream_t stream, const ElemMasks& masks);
-// conv_stream_nchw.hip: the same idea for NCHW first layers (few channels, large filters, any stride)
-bool conv_stream_nchw_eligible(const ConvGeom& g, const ElemMasks& masks);
-int conv_stream_nchw(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan,
-                     hipStream_t stream, const ElemMasks& masks);
+// conv_stream_nchw.hip: the same idea for first layers (few channels, large filters, any stride), both formats
+bool conv_stream_first_eligible(int nhwc, const ConvGeom& g, const ElemMasks& masks);
+int conv_stream_first(int nhwc, const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan,
+                      hipStream_t stream, const ElemMasks& masks);
 // conv_bwd.hip
 SplitPlan plan_dw(const ConvGeom& g, int nhwc);
 int conv_dw_nchw(const ConvGeom& g, const float* dy, const float* x, const float* cols, float* dw, float* ws,

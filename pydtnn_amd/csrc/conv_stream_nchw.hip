@@ -1,5 +1,6 @@
-// NCHW forward convolutions whose whole filter matrix fits LDS and whose reduction is short (the first layer
-// of a network: few input channels, any filter size and stride), as a streaming kernel.
+// Forward convolutions whose whole filter matrix fits LDS and whose reduction is short (the first layer of a
+// network: few input channels, any filter size and stride), as a streaming kernel; written for NCHW, with NHWC as a
+// variant of the offset tables and the store.
 //
 // On the tile engine such a layer is tiles of 2 to 23 reduction steps: filling the pipeline and storing the tile
 // take as long as the steps between them, and every workgroup does so at the same time.  Here, as in the NHWC
@@ -44,7 +45,8 @@ typedef uint32_t uintx4 __attribute__((ext_vector_type(4)));
 
 // MB: filters / 32;  CHUNKS: chunks of 16 reduction indices (kh*kw*c rounded up);  WAVES: wavefronts of the
 // workgroup, 12 (168 registers) or 16 (128 registers; same code, no spills).
-template <int MB, int CHUNKS, int MASKS, int WAVES, bool PAD>
+// NHWC: x is (n, h, w, c), the filter (c, kh, kw, kn) and y (n, ho, wo, kn); the taps keep their (c, i, j) order.
+template <int MB, int CHUNKS, int MASKS, int WAVES, bool PAD, bool NHWC>
 __global__ void __launch_bounds__(64 * WAVES) conv_stream_nchw_kernel(StreamNchwArgs a)
 {
     constexpr int KN = 32 * MB, GROUPS = CHUNKS * 2, SLOTS = CHUNKS * 16;
@@ -78,9 +80,10 @@ __global__ void __launch_bounds__(64 * WAVES) conv_stream_nchw_kernel(StreamNchw
 #pragma unroll
             for (int u = 0; u < kBatch; ++u) {
                 const int e = e0 + u * kThreadsNchw + tid;
-                const int f = e / SLOTS, s = e - f * SLOTS;
+                // consecutive threads walk along the tensor's contiguous axis: taps in NCHW, filters in NHWC
+                const int f = NHWC ? e % KN : e / SLOTS, s = NHWC ? e / KN : e - f * SLOTS;
                 const bool real = e < KN * SLOTS && s < g.k;
-                v[u] = a.w[real ? (size_t)f * g.k + s : 0];
+                v[u] = a.w[real ? (NHWC ? (size_t)s * KN + f : (size_t)f * g.k + s) : 0];
                 if (!real) v[u] = 0.0f;
                 const int m = s >> 1, h = s & 1;
                 dst[u] = e < KN * SLOTS ? (((m >> 2) * 2 + h) * KN + f) * 4 + (m & 3) : -1;
@@ -95,7 +98,8 @@ __global__ void __launch_bounds__(64 * WAVES) conv_stream_nchw_kernel(StreamNchw
             if (s < g.k) {
                 const int cc = (int)fd_div((uint32_t)s, g.fd_khw), rem = s - cc * g.khw;
                 const int ti = (int)fd_div((uint32_t)rem, g.fd_kw), tj = rem - ti * g.kw;
-                off = (uint32_t)(((long)cc * g.h + ti * g.vdilation) * g.w + tj * g.hdilation) * 4u;
+                off = NHWC ? (uint32_t)(((long)ti * g.vdilation * g.w + tj * g.hdilation) * g.c + cc) * 4u
+                           : (uint32_t)(((long)cc * g.h + ti * g.vdilation) * g.w + tj * g.hdilation) * 4u;
                 bits = (1u << ti) | (1u << (16 + tj));
             }
             const int m = s >> 1, h = s & 1;
@@ -135,7 +139,8 @@ __global__ void __launch_bounds__(64 * WAVES) conv_stream_nchw_kernel(StreamNchw
         const uint32_t oy = fd_div((uint32_t)p, g.fd_wo), ox = (uint32_t)p - oy * (uint32_t)g.wo;
         const int ih0 = (int)oy * g.vstride - g.vpadding, iw0 = (int)ox * g.hstride - g.hpadding;
         Lane l;
-        l.base = (uint32_t)(((long)img * g.c * g.h + ih0) * g.w + iw0) * 4u;
+        l.base = NHWC ? (uint32_t)((((long)img * g.h + ih0) * g.w + iw0) * g.c) * 4u
+                      : (uint32_t)(((long)img * g.c * g.h + ih0) * g.w + iw0) * 4u;
         l.bad = 0;
         if constexpr (PAD) {
             for (int t = 0; t < g.kh; ++t)
@@ -185,8 +190,46 @@ __global__ void __launch_bounds__(64 * WAVES) conv_stream_nchw_kernel(StreamNchw
         const int img = gu / a.units_per_image;
         const int p0 = (gu - img * a.units_per_image) * 32;
         // lane (p, h) holds filters 32*mb + 8*(v/4) + 4*h + v%4 of pixel p0 + p
-        const uint32_t e = p0 + lp < g.howo ? (uint32_t)(4 * lh * g.howo + lp) : kDead;
         const float* pl = params + 4 * lh;
+        if constexpr (NHWC) {
+            // a lane's registers 4q .. 4q+3 are four consecutive filters of its pixel: stored as two pairs, and the
+            // mask bytes of the four as one word
+            const uint32_t e4 = p0 + lp < g.howo ? (uint32_t)(lp * KN + 4 * lh) : kDead;
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int f = 32 * mb + 8 * q;
+                    const uint32_t soff = (uint32_t)(((long)img * g.howo + p0) * KN + f);
+                    uintx4 out;
+                    uint32_t bytes = 0;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        float val = ac[mb][4 * q + i];
+                        if constexpr ((F & kEpiBias) != 0) val += pl[f + i];
+                        if constexpr ((F & kEpiBn) != 0) {
+                            const float t = (val - pl[KN + f + i]) * pl[2 * KN + f + i];
+                            val = t * pl[3 * KN + f + i] + pl[4 * KN + f + i];
+                        }
+                        if constexpr ((F & kEpiRelu) != 0) val = val > 0.0f ? val : 0.0f;
+                        out[i] = __builtin_bit_cast(uint32_t, val);
+                        bytes |= (val > 0.0f ? 1u : 0u) << (8 * i);
+                    }
+                    // two 64-bit stores: a 128-bit buffer store with a register offset, followed at once by an
+                    // instruction that overwrites its data registers, stored the new values for some lanes on this
+                    // part (the compiler inserts the wait state only for a constant offset)
+                    typedef uint32_t uintx2 __attribute__((ext_vector_type(2)));
+                    const uintx2 lo = {out[0], out[1]}, hi = {out[2], out[3]};
+                    const int voff = (int)(e4 == kDead ? kOob : e4 * 4u);
+                    __builtin_amdgcn_raw_buffer_store_b64(lo, y_rsrc, voff, (int)(soff * 4u), 0);
+                    __builtin_amdgcn_raw_buffer_store_b64(hi, y_rsrc, voff, (int)(soff * 4u + 8u), 0);
+                    if constexpr (MASKS == kReluMask)
+                        __builtin_amdgcn_raw_buffer_store_b32(bytes, mask_rsrc, (int)(e4 == kDead ? kOob : e4),
+                                                              (int)soff, 0);
+                }
+            return;
+        }
+        const uint32_t e = p0 + lp < g.howo ? (uint32_t)(4 * lh * g.howo + lp) : kDead;
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
@@ -279,13 +322,13 @@ constexpr size_t stream_nchw_lds_bytes()
     return ((size_t)CHUNKS * 2 * 2 * 32 * MB * 4 + CHUNKS * 2 * 2 * 4 * 2 + 5 * 32 * MB) * 4 + 16;
 }
 
-template <int MB, int CHUNKS, int MASKS, int WAVES, bool PAD>
+template <int MB, int CHUNKS, int MASKS, int WAVES, bool PAD, bool NHWC>
 int launch_stream_nchw_waves(const StreamNchwArgs& a, int grid, hipStream_t stream)
 {
     static std::atomic<unsigned> raised{0};
     constexpr size_t lds_bytes = stream_nchw_lds_bytes<MB, CHUNKS>();
     static_assert(lds_bytes <= 160 * 1024, "filter matrix must fit LDS");
-    auto kernel = conv_stream_nchw_kernel<MB, CHUNKS, MASKS, WAVES, PAD>;
+    auto kernel = conv_stream_nchw_kernel<MB, CHUNKS, MASKS, WAVES, PAD, NHWC>;
     const int rc = raise_lds_limit(reinterpret_cast<const void*>(kernel), raised, 160 * 1024);
     if (rc != PYDTNN_HIP_OK) return rc;
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(64 * WAVES), lds_bytes, stream, a);
@@ -293,7 +336,7 @@ int launch_stream_nchw_waves(const StreamNchwArgs& a, int grid, hipStream_t stre
     return PYDTNN_HIP_OK;
 }
 
-template <int MB, int CHUNKS, int MASKS, bool PAD>
+template <int MB, int CHUNKS, int MASKS, bool PAD, bool NHWC>
 int launch_stream_nchw(const StreamNchwArgs& a, hipStream_t stream)
 {
     int cus = 0;
@@ -304,37 +347,39 @@ int launch_stream_nchw(const StreamNchwArgs& a, hipStream_t stream)
     // idle slots in the last round (24 units: two full rounds of 12, but 32 slots of 16).
     const int per_wg = (a.units + grid - 1) / grid;
     const int slots16 = (per_wg + 15) / 16 * 16, slots12 = (per_wg + 11) / 12 * 12;
-    if (slots12 < slots16) return launch_stream_nchw_waves<MB, CHUNKS, MASKS, 12, PAD>(a, grid, stream);
-    return launch_stream_nchw_waves<MB, CHUNKS, MASKS, 16, PAD>(a, grid, stream);
+    if (slots12 < slots16) return launch_stream_nchw_waves<MB, CHUNKS, MASKS, 12, PAD, NHWC>(a, grid, stream);
+    return launch_stream_nchw_waves<MB, CHUNKS, MASKS, 16, PAD, NHWC>(a, grid, stream);
 }
 
-// The (filters, chunks of 16 reduction indices, padded?) triples that are built: AlexNet's first layer (96 filters,
-// 3 x 11 x 11 = 363 taps, no padding), VGG's (64 filters, 3 x 3 x 3 = 27 taps, padded) and ResNet's (64 filters,
-// 3 x 7 x 7 = 147 taps, padded).
-bool stream_nchw_shape_built(int kn, int k, bool padded)
+// The (format, filters, chunks of 16 reduction indices, padded?) combinations that are built.  NCHW: AlexNet's first
+// layer (96 filters, 3 x 11 x 11 = 363 taps, no padding), VGG's (64 filters, 3 x 3 x 3 = 27 taps, padded) and
+// ResNet's (64 filters, 3 x 7 x 7 = 147 taps, padded).  NHWC: VGG's, and 32 filters over at most 16 taps (a 3 x 3
+// layer on one channel).
+bool stream_first_shape_built(int nhwc, int kn, int k, bool padded)
 {
     const int chunks = (k + 15) / 16;
+    if (nhwc) return padded && ((kn == 64 && chunks == 2) || (kn == 32 && chunks == 1));
     if (!padded) return kn == 96 && chunks == 23;
     return kn == 64 && (chunks == 2 || chunks == 10);
 }
 
 }  // namespace
 
-bool conv_stream_nchw_eligible(const ConvGeom& g, const ElemMasks& masks)
+bool conv_stream_first_eligible(int nhwc, const ConvGeom& g, const ElemMasks& masks)
 {
     const bool padded = g.vpadding != 0 || g.hpadding != 0;
-    if (!stream_nchw_shape_built(g.kn, g.k, padded)) return false;
+    if (!stream_first_shape_built(nhwc, g.kn, g.k, padded)) return false;
     if (padded && (g.kh > 16 || g.kw > 16)) return false;  // row and column bits share one word
     const int mk = mask_kind(masks);
     if (mk != kNoMasks && mk != kReluMask) return false;
     if (g.p < 32 * 1024) return false;                      // enough units for every compute unit
     // every byte offset the kernel forms stays below 2^30 in magnitude, and so do the descriptors
-    const long reach = (long)g.n * g.c * g.h * g.w + ((long)g.vpadding + 1) * g.w + g.hpadding;
+    const long reach = (long)g.n * g.c * g.h * g.w + (((long)g.vpadding + 1) * g.w + g.hpadding) * (nhwc ? g.c : 1);
     return reach < (1l << 28) && g.p * g.kn < (1l << 28);
 }
 
-int conv_stream_nchw(const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan,
-                     hipStream_t stream, const ElemMasks& masks)
+int conv_stream_first(int nhwc, const ConvGeom& g, const float* w, const float* x, float* y, const ChanEpilogue& chan,
+                      hipStream_t stream, const ElemMasks& masks)
 {
     StreamNchwArgs a;
     a.x = x; a.w = w; a.y = y; a.g = g; a.chan = chan; a.masks = masks;
@@ -343,14 +388,16 @@ int conv_stream_nchw(const ConvGeom& g, const float* w, const float* x, float* y
     const int chunks = (g.k + 15) / 16;
     const bool mask = mask_kind(masks) == kReluMask;
     const bool padded = g.vpadding != 0 || g.hpadding != 0;
-#define STREAM_NCHW_CASE(KN, CH, PAD)                                                         \
-    if (g.kn == KN && chunks == CH && padded == PAD)                                          \
-        return mask ? launch_stream_nchw<KN / 32, CH, kReluMask, PAD>(a, stream)              \
-                    : launch_stream_nchw<KN / 32, CH, kNoMasks, PAD>(a, stream)
-    STREAM_NCHW_CASE(96, 23, false);
-    STREAM_NCHW_CASE(64, 2, true);
-    STREAM_NCHW_CASE(64, 10, true);
-#undef STREAM_NCHW_CASE
+#define STREAM_FIRST_CASE(FMT, KN, CH, PAD)                                                        \
+    if ((nhwc != 0) == FMT && g.kn == KN && chunks == CH && padded == PAD)                         \
+        return mask ? launch_stream_nchw<KN / 32, CH, kReluMask, PAD, FMT>(a, stream)              \
+                    : launch_stream_nchw<KN / 32, CH, kNoMasks, PAD, FMT>(a, stream)
+    STREAM_FIRST_CASE(false, 96, 23, false);
+    STREAM_FIRST_CASE(false, 64, 2, true);
+    STREAM_FIRST_CASE(false, 64, 10, true);
+    STREAM_FIRST_CASE(true, 64, 2, true);
+    STREAM_FIRST_CASE(true, 32, 1, true);
+#undef STREAM_FIRST_CASE
     return PYDTNN_HIP_ERR_UNSUPPORTED;
 }
 

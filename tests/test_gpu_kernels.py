@@ -325,6 +325,42 @@ def test_streaming_kernel_shapes_nchw(cg, oracle, d):
         assert np.array_equal(y2, host(y))
 
 
+# NHWC first layers on the same kernel: VGG's 3 x 3 x 3 -> 64 (ragged planes, mixed padding and stride, dilation)
+# and 32 filters over at most 16 taps (MNIST's 3 x 3 on one channel; 2 x 2 x 4 taps; a padded 1 x 1 on 9 channels)
+stream_first_nhwc_grid = [
+    D(2, 3, 224, 224, 64, 3, 3, 1, 1, 1, 1, 1, 1),
+    D(20, 3, 50, 47, 64, 3, 3, 1, 1, 1, 1, 1, 1),
+    D(20, 3, 57, 61, 64, 3, 3, 2, 0, 1, 2, 1, 1),
+    D(3, 3, 130, 130, 64, 3, 3, 2, 2, 1, 1, 2, 2),
+    D(64, 1, 28, 28, 32, 3, 3, 1, 1, 1, 1, 1, 1),
+    D(7, 4, 70, 81, 32, 2, 2, 1, 1, 1, 1, 1, 1),
+    D(3, 9, 110, 110, 32, 1, 1, 1, 1, 1, 1, 1, 1),
+]
+
+
+@pytest.mark.parametrize("d", stream_first_nhwc_grid, ids=repr)
+def test_streaming_kernel_first_layers_nhwc(cg, oracle, d):
+    announce("stream first layers nhwc", d)
+    assert d.b * d.ho * d.wo >= 32768
+    x, w, b, _ = case(d)
+    rng = np.random.default_rng(11)
+    bn = [rng.uniform(0.5, 1.5, d.kn).astype(np.float32) for _ in range(4)]
+    xr, wr = nhwc(x), w_nhwc(w)
+    ref, _ = oracle.conv2d_forward_nhwc_i2c(xr, wr, b, oracle.ConvParams(*d.geom()))
+    xd, wd, bd = dev(xr), dev(wr), dev(b)
+    y = cg.conv_gemm_nhwc(wd, xd, **_kw(d))
+    assert_close(host(y), ref - b.reshape(1, 1, 1, -1), what="y without bias")
+    y = cg.conv_gemm_nhwc(wd, xd, biases_vector=bd, **_kw(d))
+    assert_close(host(y), ref, what="y")
+    y_bn = cg.conv_gemm_nhwc(wd, xd, biases_vector=bd, bn_running_mean=dev(bn[0]), bn_inv_std=dev(bn[1]),
+                             bn_gamma=dev(bn[2]), bn_beta=dev(bn[3]), relu=True, **_kw(d))
+    assert_close(host(y_bn), oracle.fused_epilogue(ref, "NHWC", bn=bn, relu_flag=True), what="fused y")
+    y_relu = torch.full(y.shape, np.nan, device="cuda")
+    mask = torch.full(y.shape, 7, dtype=torch.int8, device="cuda")
+    cg.conv_gemm_nhwc(wd, xd, biases=y_relu, biases_vector=bd, relu=True, relu_mask=mask, **_kw(d))
+    assert torch.equal(y_relu, torch.clamp(y, min=0)) and torch.equal(mask, (y > 0).to(torch.int8))
+
+
 @pytest.mark.parametrize("x,w,stride", [
     (x_2x4, w_1x1, 1), (x_2x4, w_1x2, 1), (x_2x4, w_2x2, 1), (x_4x4, w_2x2, 2), (x_4x8, w_2x2, (1, 2)),
     (x_8x8, w_3x3, 3), (x_8x8, w_2x2, 1), (x_2x4_c2, w_c2_1234_4567, 1)])
