@@ -242,7 +242,7 @@ def run_cfg1(torch, pd, timed_steps, steps, warmup):
     flop = 2.0 * 32 * 9 * 64 * 28 * 28
     nbytes = x.nbytes + w.nbytes + 64 * 28 * 28 * 32 * 4
     gbs = nbytes / (ms * 1e-3) / 1e9
-    roofline = {"bound": "hbm", "kernel": "gemm_kernel<64x64, Im2colNchwMN<NHWC>, PlainMN, EpiPlain>",
+    roofline = {"bound": "hbm", "kernel": "conv_stream_nchw_kernel<1, 1, 0, 12, true, true>",
                 "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
                 "traffic": None}
     workload = "cfg1: Conv2D forward, fp32 NHWC, N=64, 28x28x1 -> 32, 3x3, stride 1, pad 1 (launch-latency bound)"

@@ -167,5 +167,16 @@ def workspace(nbytes):
     return ctypes.c_void_p(buf.data_ptr()), buf.numel()
 
 
+_WORKSPACE_BYTES = {}
+
+
 def conv_workspace(op, nhwc, geom13):
-    return workspace(lib().pydtnn_hip_conv_workspace_bytes(op, int(nhwc), *geom13))
+    """Scratch buffer for one convolution call; the size query is remembered per (device, operation, geometry),
+    since it depends on nothing else and a layer asks with the same geometry at every step."""
+    key = (torch.cuda.current_device(), op, int(nhwc), tuple(geom13))
+    nbytes = _WORKSPACE_BYTES.get(key)
+    if nbytes is None:
+        nbytes = lib().pydtnn_hip_conv_workspace_bytes(op, int(nhwc), *geom13)
+        if len(_WORKSPACE_BYTES) < 4096:
+            _WORKSPACE_BYTES[key] = nbytes
+    return workspace(nbytes)
