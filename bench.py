@@ -363,10 +363,23 @@ def run_cfg5(torch, pd, args, steps=None, warmup=None):
     if not args.no_folding_extra:
         plain_ms, _ = timed_steps(torch, plain_step, steps or args.steps,
                                    warmup if warmup is not None else args.warmup)
+    # ... and with the whole backward pass on one stream (Model(enable_backward_overlap=False); same bits again)
+    one_stream_ms = None
+    if not args.no_folding_extra:
+        del plain_model
+        np.random.seed(0)
+        one_stream_model = build_vgg16(pd, n, enable_backward_overlap=False)
+        one_stream_losses, one_stream_opt = [], pd.SGD(learning_rate=0.01, momentum=0.9)
+
+        def one_stream_step(timers):
+            one_stream_losses.append(one_stream_model.train_batch(x, y_targ, loss_fn, one_stream_opt))
+
+        one_stream_ms, _ = timed_steps(torch, one_stream_step, steps or args.steps,
+                                        warmup if warmup is not None else args.warmup)
+        del one_stream_model
     # the same step in the reference's other tensor format (its default on the CPU), also beside the headline
     nhwc_ms = None
     if not args.no_folding_extra:
-        del plain_model
         np.random.seed(0)
         nhwc_model = build_vgg16(pd, n, tensor_format="NHWC")
         x_nhwc = x.permute(0, 2, 3, 1).contiguous()
@@ -386,6 +399,10 @@ def run_cfg5(torch, pd, args, steps=None, warmup=None):
         extra.update({"vgg16_separate_relu_img_per_s": round(n / (plain_ms * 1e-3), 1),
                       "vgg16_separate_relu_ms_per_step": round(plain_ms, 2),
                       "vgg16_separate_relu_same_losses": [float(a) for a in losses] == [float(b) for b in plain_losses]})
+    if one_stream_ms is not None:
+        extra.update({"vgg16_one_stream_img_per_s": round(n / (one_stream_ms * 1e-3), 1),
+                      "vgg16_one_stream_ms_per_step": round(one_stream_ms, 2),
+                      "vgg16_one_stream_same_losses": [float(a) for a in losses] == [float(b) for b in one_stream_losses]})
     if nhwc_ms is not None:
         extra.update({"vgg16_nhwc_train_img_per_s": round(n / (nhwc_ms * 1e-3), 1),
                       "vgg16_nhwc_ms_per_step": round(nhwc_ms, 2)})

@@ -389,13 +389,14 @@ class Conv2D(Layer):
     def _backward_nhwc_i2c(self, dy):
         b = dy.shape[0]
         self.dw = torch.empty_like(self.weights)
-        self._op(ev.PYDTNN_OPS_COMP_DW_MATMUL)
-        ops.conv_i2c_dw(True, self._geom13(b), dy, self.x_rows, self.dw)
-        self._end()
-        if self.use_bias:
-            self._op(ev.PYDTNN_OPS_BACKWARD_SUM_BIASES)
-            self.db = ops.bias_grad(dy, self.co, 1)
+        with self.model.beside_backward(dy, self.x_rows):
+            self._op(ev.PYDTNN_OPS_COMP_DW_MATMUL)
+            ops.conv_i2c_dw(True, self._geom13(b), dy, self.x_rows, self.dw)
             self._end()
+            if self.use_bias:
+                self._op(ev.PYDTNN_OPS_BACKWARD_SUM_BIASES)
+                self.db = ops.bias_grad(dy, self.co, 1)
+                self._end()
         if self.need_dx:
             dx = torch.empty((b, self.hi, self.wi, self.ci), dtype=dy.dtype, device=dy.device)
             self._op(ev.PYDTNN_OPS_COMP_DX_MATMUL)  # the GEMM and row2im of the explicit route
@@ -421,13 +422,14 @@ class Conv2D(Layer):
     def _backward_nchw_i2c(self, dy):
         b = dy.shape[0]
         self.dw = torch.empty_like(self.weights)
-        self._op(ev.PYDTNN_OPS_COMP_DW_MATMUL)
-        ops.conv_i2c_dw(False, self._geom13(b), dy, self.x_cols, self.dw)
-        self._end()
-        if self.use_bias:
-            self._op(ev.PYDTNN_OPS_BACKWARD_SUM_BIASES)
-            self.db = ops.bias_grad(dy, self.co, self.ho * self.wo)
+        with self.model.beside_backward(dy, self.x_cols):
+            self._op(ev.PYDTNN_OPS_COMP_DW_MATMUL)
+            ops.conv_i2c_dw(False, self._geom13(b), dy, self.x_cols, self.dw)
             self._end()
+            if self.use_bias:
+                self._op(ev.PYDTNN_OPS_BACKWARD_SUM_BIASES)
+                self.db = ops.bias_grad(dy, self.co, self.ho * self.wo)
+                self._end()
         if self.need_dx:
             dx = torch.empty((b, self.ci, self.hi, self.wi), dtype=dy.dtype, device=dy.device)
             self._op(ev.PYDTNN_OPS_COMP_DX_MATMUL)  # the GEMM and col2im of the explicit route
@@ -458,16 +460,20 @@ class Conv2D(Layer):
         self._end()
         return y
 
-    def _backward_nhwc_cg(self, dy):
+    def _filter_and_bias_gradients(self, dy, conv_gemm, rows):
         res = torch.empty(self.weights.shape, dtype=dy.dtype, device=dy.device)
-        self._op(ev.PYDTNN_OPS_BACKWARD_CONVGEMM)
-        self.cg.conv_gemm_nhwc(dy, self.cg_x, biases=res, trans=True, **self._cg_kwargs())
-        self._end()
-        self.dw = res
-        if self.use_bias:
-            self._op(ev.PYDTNN_OPS_BACKWARD_SUM_BIASES)
-            self.db = ops.bias_grad(dy, self.co, 1)
+        with self.model.beside_backward(dy, self.cg_x):
+            self._op(ev.PYDTNN_OPS_BACKWARD_CONVGEMM)
+            conv_gemm(dy, self.cg_x, biases=res, trans=True, **self._cg_kwargs())
             self._end()
+            self.dw = res
+            if self.use_bias:
+                self._op(ev.PYDTNN_OPS_BACKWARD_SUM_BIASES)
+                self.db = ops.bias_grad(dy, self.co, rows)
+                self._end()
+
+    def _backward_nhwc_cg(self, dy):
+        self._filter_and_bias_gradients(dy, self.cg.conv_gemm_nhwc, 1)
         if self.need_dx:
             dx = torch.empty((dy.shape[0], self.hi, self.wi, self.ci), dtype=dy.dtype, device=dy.device)
             gate = self._gate_below(dx.shape)
@@ -494,15 +500,7 @@ class Conv2D(Layer):
         return y
 
     def _backward_nchw_cg(self, dy):
-        res = torch.empty(self.weights.shape, dtype=dy.dtype, device=dy.device)
-        self._op(ev.PYDTNN_OPS_BACKWARD_CONVGEMM)
-        self.cg.conv_gemm_nchw(dy, self.cg_x, biases=res, trans=True, **self._cg_kwargs())
-        self._end()
-        self.dw = res
-        if self.use_bias:
-            self._op(ev.PYDTNN_OPS_BACKWARD_SUM_BIASES)
-            self.db = ops.bias_grad(dy, self.co, self.ho * self.wo)
-            self._end()
+        self._filter_and_bias_gradients(dy, self.cg.conv_gemm_nchw, self.ho * self.wo)
         if self.need_dx:
             dx = torch.empty((dy.shape[0], self.ci, self.hi, self.wi), dtype=dy.dtype, device=dy.device)
             gate = self._gate_below(dx.shape)
@@ -549,9 +547,10 @@ class FC(Layer):
         return self.model.matmul(x, self.weights, bias=self.biases)
 
     def backward(self, dy):
-        self.dw = self.model.matmul(self.x.t(), dy)
-        if self.use_bias:
-            self.db = ops.bias_grad(dy, dy.shape[1], 1)
+        with self.model.beside_backward(dy, self.x):
+            self.dw = self.model.matmul(self.x.t(), dy)
+            if self.use_bias:
+                self.db = ops.bias_grad(dy, dy.shape[1], 1)
         if self.need_dx:
             return self.model.matmul(dy, self.weights.t())
 

@@ -8,6 +8,8 @@ Kept from the reference: keyword flags readable as attributes (``tensor_format``
 (pydtnn/model.py:450-492, :623-644).  Datasets, MPI, checkpoints, schedulers and the CLI are not
 part of this build.
 """
+import contextlib
+
 import numpy as np
 import torch
 
@@ -45,6 +47,12 @@ _DEFAULTS = dict(
     # has already rectified, the layer above the Relu a dx already multiplied by the mask), and a layer's
     # forward / backward called outside train_batch never does it.  False restores the separate passes.
     enable_relu_folding=True,
+    # Not a reference flag.  Inside train_batch the filter / weight and bias gradients of a Conv2D or FC layer are
+    # enqueued on a second stream (default priority) while the layer's input gradient, and the layers below, go on
+    # with the caller's stream; the weight updates wait for both.  Same kernels and bit-identical results: only
+    # their order on the device changes, so that one kernel's last, partly idle round of workgroups is filled by
+    # the other's.  False keeps everything on the caller's stream.
+    enable_backward_overlap=True,
 )
 
 
@@ -80,6 +88,8 @@ class Model:
         self.batch_size = self.kwargs["batch_size"]
         self._fused = False
         self.stepping = False  # True while train_batch runs its own forward / backward loops
+        self._side_streams = {}  # device index -> second stream of enable_backward_overlap
+        self._side_refs = []     # (stream, tensors it still reads): kept alive until the caller's stream has waited
         # pydtnn/model.py:216-218: without the flag every BestOf just calls its first alternative
         BestOf.use_always_the_first_alternative(not self.kwargs["enable_best_of"])
 
@@ -206,12 +216,36 @@ class Model:
                 emit(PYDTNN_MDL_EVENT, 0)
         finally:
             self.stepping = False
+            self._join_side_stream()
         for i in range(len(self.layers) - 1, 0, -1):
             self.layers[i].reduce_weights_sync()
             emit(PYDTNN_MDL_EVENT, self.layers[i].id * PYDTNN_MDL_EVENTS + PYDTNN_MDL_UPDATE_DW)
             self.layers[i].update_weights(optimizer)
             emit(PYDTNN_MDL_EVENT, 0)
         return loss
+
+    @contextlib.contextmanager
+    def beside_backward(self, *tensors):
+        """Inside train_batch with ``enable_backward_overlap``: the body's work goes to the model's second stream,
+        after everything enqueued so far on the caller's; ``tensors`` (what the body reads) stay referenced until
+        the caller's stream has waited for that stream, so the allocator cannot hand their memory out in between.
+        Otherwise the body runs in place."""
+        if not (self.stepping and self.kwargs["enable_backward_overlap"] and tensors and tensors[0].is_cuda):
+            yield
+            return
+        device = tensors[0].device
+        side = self._side_streams.get(device.index)
+        if side is None:
+            side = self._side_streams[device.index] = torch.cuda.Stream(device=device)     # default priority
+        side.wait_stream(torch.cuda.current_stream(device))
+        self._side_refs.append((side, tensors))
+        with torch.cuda.stream(side):
+            yield
+
+    def _join_side_stream(self):
+        for side in {s for s, _ in self._side_refs}:
+            torch.cuda.current_stream(side.device).wait_stream(side)
+        self._side_refs.clear()
 
     def evaluate_batch(self, x):
         """Forward pass of pydtnn/model.py:623-644."""

@@ -394,6 +394,69 @@ def test_relu_folding_changes_no_bit_of_a_training_run(pd, fmt, monkeypatch):
     assert calls_a == {"fwd": 2, "bwd": 2}   # only the Relu between the FC layers
 
 
+@pytest.mark.parametrize("conv_gemm", [True, False])
+@pytest.mark.parametrize("fmt", ["NCHW", "NHWC"])
+def test_backward_overlap_changes_no_bit_of_a_training_run(pd, fmt, conv_gemm):
+    """Three training steps of a small network with a residual block, with the filter / bias gradients on the
+    model's second stream (the default) and with everything on the caller's stream: losses, every gradient and
+    every updated weight are identical; the second stream is used by the one run only, and nothing of a step is
+    left on it when train_batch returns."""
+    announce("backward overlap", fmt, conv_gemm)
+    n, classes = 8, 10
+    rng = np.random.default_rng(23)
+    x = dev(rng.random((n, 3, 16, 16) if fmt == "NCHW" else (n, 16, 16, 3)).astype(np.float32))
+    y_targ = dev(np.eye(classes, dtype=np.float32)[rng.integers(0, classes, n)])
+
+    def run(overlap):
+        np.random.seed(7)
+        model = pd.Model(tensor_format=fmt, batch_size=n, enable_backward_overlap=overlap, enable_conv_gemm=conv_gemm)
+        model.add(pd.Input(shape=(16, 16, 3)))
+        model.add(pd.Conv2D(nfilters=8, filter_shape=(3, 3), padding=1, activation="relu", weights_initializer="he_normal"))
+        model.add(pd.AdditionBlock([pd.Conv2D(nfilters=8, filter_shape=(3, 3), padding=1, weights_initializer="he_normal"),
+                                    pd.BatchNormalization(), pd.Relu(),
+                                    pd.Conv2D(nfilters=8, filter_shape=(1, 1), weights_initializer="he_normal")], []))
+        model.add(pd.Relu())
+        model.add(pd.Conv2D(nfilters=12, filter_shape=(3, 3), padding=1, stride=2, activation="relu",
+                            weights_initializer="he_normal"))
+        model.add(pd.MaxPool2D(pool_shape=(2, 2), stride=2))
+        model.add(pd.Flatten())
+        model.add(pd.FC(shape=(32,), activation="relu", weights_initializer="he_normal"))
+        model.add(pd.FC(shape=(classes,), activation="softmax", weights_initializer="he_normal"))
+        loss_fn, opt = pd.CategoricalCrossEntropy(), pd.SGD(learning_rate=0.05, momentum=0.9)
+        losses = []
+        for _ in range(3):
+            losses.append(float(model.train_batch(x, y_targ, loss_fn, opt)))
+            assert not model._side_refs
+        state = {}
+        for l in model.get_all_layers():
+            for var, grad in l.grad_vars.items():
+                state[f"{l.id}.{var}"] = getattr(l, var).clone()
+                state[f"{l.id}.{grad}"] = getattr(l, grad).clone()
+        return losses, state, bool(model._side_streams)
+
+    losses_a, state_a, used_a = run(True)
+    losses_b, state_b, used_b = run(False)
+    assert used_a and not used_b
+    assert losses_a == losses_b and len(state_a) >= 12
+    assert state_a.keys() == state_b.keys()
+    for k in state_a:
+        assert torch.equal(state_a[k], state_b[k]), k
+
+
+def test_backward_overlap_stays_inside_the_training_step(pd):
+    """A layer's backward called by hand enqueues everything on the caller's stream."""
+    model = pd.Model(tensor_format="NCHW", batch_size=2)
+    assert model.enable_backward_overlap
+    model.add(pd.Input(shape=(6, 6, 2)))
+    model.add(pd.Conv2D(nfilters=3, filter_shape=(3, 3), padding=1))
+    model.add(pd.Conv2D(nfilters=3, filter_shape=(3, 3), padding=1))
+    model.mode = pd.TRAIN_MODE
+    conv = model.layers[2]
+    conv.forward(torch.randn(2, 3, 6, 6, device="cuda"))
+    conv.backward(torch.randn(2, 3, 6, 6, device="cuda"))
+    assert not model._side_streams and not model._side_refs
+
+
 def test_relu_folding_stays_inside_the_training_step(pd):
     """Outside train_batch a convolution's forward returns conv(x) + b as the reference's does, whatever follows
     it in the model; and the hand-over is recognised by tensor identity: a Relu given any other tensor
