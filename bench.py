@@ -44,6 +44,9 @@ def parse_args():
     ap.add_argument("--no-vgg16", action="store_true", help="skip the VGG16 training-step extra of the default run")
     ap.add_argument("--no-other-configs", action="store_true",
                     help="skip cfg1, cfg3 and cfg4 (GPU and CPU legs) in the default run's extra")
+    ap.add_argument("--one-stream", action="store_true",
+                    help="cfg5: build the headline model with enable_backward_overlap=False (kernel traces then show "
+                         "each kernel alone on the chip)")
     ap.add_argument("--no-folding-extra", action="store_true",
                     help="skip the extra VGG16 runs (enable_relu_folding=False; NHWC) that are reported beside the headline one")
     ap.add_argument("--conv-layers", action="store_true",
@@ -337,7 +340,7 @@ def run_cfg5(torch, pd, args, steps=None, warmup=None):
     import numpy as np
     np.random.seed(0)
     n = 64
-    model = build_vgg16(pd, n)
+    model = build_vgg16(pd, n, enable_backward_overlap=not args.one_stream)
     # the same network with every Relu layer making its own two passes (Model(enable_relu_folding=False); same
     # losses, gradients and weights bit for bit): reported beside the headline number
     np.random.seed(0)
