@@ -89,6 +89,7 @@ class Model:
         self._fused = False
         self.stepping = False  # True while train_batch runs its own forward / backward loops
         self._side_streams = {}  # device index -> second stream of enable_backward_overlap
+        self._overlap_min_elements = 1 << 16
         self._side_refs = []     # (stream, tensors it still reads): kept alive until the caller's stream has waited
         # pydtnn/model.py:216-218: without the flag every BestOf just calls its first alternative
         BestOf.use_always_the_first_alternative(not self.kwargs["enable_best_of"])
@@ -229,8 +230,10 @@ class Model:
         """Inside train_batch with ``enable_backward_overlap``: the body's work goes to the model's second stream,
         after everything enqueued so far on the caller's; ``tensors`` (what the body reads) stay referenced until
         the caller's stream has waited for that stream, so the allocator cannot hand their memory out in between.
-        Otherwise the body runs in place."""
-        if not (self.stepping and self.kwargs["enable_backward_overlap"] and tensors and tensors[0].is_cuda):
+        Otherwise, and for small problems (under 2^16 elements read: nothing to overlap but launches), the body
+        runs in place."""
+        if not (self.stepping and self.kwargs["enable_backward_overlap"] and tensors and tensors[0].is_cuda
+                and sum(t.numel() for t in tensors) >= self._overlap_min_elements):
             yield
             return
         device = tensors[0].device

@@ -410,6 +410,7 @@ def test_backward_overlap_changes_no_bit_of_a_training_run(pd, fmt, conv_gemm):
     def run(overlap):
         np.random.seed(7)
         model = pd.Model(tensor_format=fmt, batch_size=n, enable_backward_overlap=overlap, enable_conv_gemm=conv_gemm)
+        model._overlap_min_elements = 0      # problems this small would otherwise stay on one stream
         model.add(pd.Input(shape=(16, 16, 3)))
         model.add(pd.Conv2D(nfilters=8, filter_shape=(3, 3), padding=1, activation="relu", weights_initializer="he_normal"))
         model.add(pd.AdditionBlock([pd.Conv2D(nfilters=8, filter_shape=(3, 3), padding=1, weights_initializer="he_normal"),
@@ -452,6 +453,7 @@ def test_backward_overlap_stays_inside_the_training_step(pd):
     model.add(pd.Conv2D(nfilters=3, filter_shape=(3, 3), padding=1))
     model.mode = pd.TRAIN_MODE
     conv = model.layers[2]
+    model._overlap_min_elements = 0
     conv.forward(torch.randn(2, 3, 6, 6, device="cuda"))
     conv.backward(torch.randn(2, 3, 6, 6, device="cuda"))
     assert not model._side_streams and not model._side_refs
