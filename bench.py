@@ -44,6 +44,9 @@ def parse_args():
     ap.add_argument("--no-vgg16", action="store_true", help="skip the VGG16 training-step extra of the default run")
     ap.add_argument("--no-other-configs", action="store_true",
                     help="skip cfg1, cfg3 and cfg4 (GPU and CPU legs) in the default run's extra")
+    ap.add_argument("--settle", type=float, default=SETTLE_SECONDS,
+                    help="least duration in seconds of the untimed part before each timed region (counter passes of "
+                         "a profiler, whose figures do not depend on the clocks, use 0)")
     ap.add_argument("--one-stream", action="store_true",
                     help="cfg5: build the headline model with enable_backward_overlap=False (kernel traces then show "
                          "each kernel alone on the chip)")
@@ -99,10 +102,22 @@ class Timer:
         return times[len(times) // 2]
 
 
+SETTLE_SECONDS = 0.1
+
+
 def timed_steps(torch, step, steps, warmup):
+    """`warmup` untimed steps, then exactly `steps` timed ones between two synchronizations.  The untimed part
+    lasts at least SETTLE_SECONDS: after an idle spell the GPU runs below its sustained clocks for some 20 ms
+    (the ResNet block measures 0.33 ms for its first 50 steps and 0.295 ms from then on), which the warm-up
+    steps of a sub-millisecond workload would not cover."""
+    t_start = time.perf_counter()
     for _ in range(warmup):
         step(None)
     torch.cuda.synchronize()
+    while time.perf_counter() - t_start < SETTLE_SECONDS:
+        for _ in range(10):
+            step(None)
+        torch.cuda.synchronize()
     timers = {}
     t0 = time.perf_counter()
     for _ in range(steps):
@@ -443,7 +458,9 @@ def vgg16_conv_layers(torch, n=64, reps=5):
 
 
 def main():
+    global SETTLE_SECONDS
     args = parse_args()
+    SETTLE_SECONDS = args.settle
     if args.gpus != 1:
         print(f"bench.py: this build runs on one GPU; --gpus {args.gpus} is not supported "
               f"(no collectives or sharding are part of it).", file=sys.stderr)
@@ -504,7 +521,8 @@ def main():
         "metric": METRIC, "value": round(value, 1), "unit": unit, "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": workload}, "roofline": roofline, "cpu_baseline": cpu, "extra": extra}))
+        "config": {"workload": workload, "untimed_seconds_before_each_timed_region": SETTLE_SECONDS},
+        "roofline": roofline, "cpu_baseline": cpu, "extra": extra}))
 
 
 if __name__ == "__main__":
