@@ -160,6 +160,9 @@ class Layer:
         return children
 
     def update_weights(self, optimizer):
+        ready = self.__dict__.pop("grads_ready", None)   # set when the gradients were computed on another stream
+        if ready is not None:
+            torch.cuda.current_stream().wait_event(ready)
         optimizer.update(self)
 
 
@@ -389,7 +392,7 @@ class Conv2D(Layer):
     def _backward_nhwc_i2c(self, dy):
         b = dy.shape[0]
         self.dw = torch.empty_like(self.weights)
-        with self.model.beside_backward(dy, self.x_rows):
+        with self.model.beside_backward(self, dy, self.x_rows):
             self._op(ev.PYDTNN_OPS_COMP_DW_MATMUL)
             ops.conv_i2c_dw(True, self._geom13(b), dy, self.x_rows, self.dw)
             self._end()
@@ -422,7 +425,7 @@ class Conv2D(Layer):
     def _backward_nchw_i2c(self, dy):
         b = dy.shape[0]
         self.dw = torch.empty_like(self.weights)
-        with self.model.beside_backward(dy, self.x_cols):
+        with self.model.beside_backward(self, dy, self.x_cols):
             self._op(ev.PYDTNN_OPS_COMP_DW_MATMUL)
             ops.conv_i2c_dw(False, self._geom13(b), dy, self.x_cols, self.dw)
             self._end()
@@ -462,7 +465,7 @@ class Conv2D(Layer):
 
     def _filter_and_bias_gradients(self, dy, conv_gemm, rows):
         res = torch.empty(self.weights.shape, dtype=dy.dtype, device=dy.device)
-        with self.model.beside_backward(dy, self.cg_x):
+        with self.model.beside_backward(self, dy, self.cg_x):
             self._op(ev.PYDTNN_OPS_BACKWARD_CONVGEMM)
             conv_gemm(dy, self.cg_x, biases=res, trans=True, **self._cg_kwargs())
             self._end()
@@ -547,7 +550,7 @@ class FC(Layer):
         return self.model.matmul(x, self.weights, bias=self.biases)
 
     def backward(self, dy):
-        with self.model.beside_backward(dy, self.x):
+        with self.model.beside_backward(self, dy, self.x):
             self.dw = self.model.matmul(self.x.t(), dy)
             if self.use_bias:
                 self.db = ops.bias_grad(dy, dy.shape[1], 1)

@@ -215,20 +215,28 @@ class Model:
                 emit(PYDTNN_MDL_EVENT, self.layers[i].id * PYDTNN_MDL_EVENTS + PYDTNN_MDL_BACKWARD)
                 dx = self.layers[i].backward(dx)
                 emit(PYDTNN_MDL_EVENT, 0)
+        except BaseException:
+            self._join_side_stream()
+            raise
         finally:
             self.stepping = False
+        # each layer's update waits for that layer's gradients only (Layer.update_weights), so the updates of the
+        # upper layers run while the second stream still works on the filter gradients of the lowest ones
+        try:
+            for i in range(len(self.layers) - 1, 0, -1):
+                self.layers[i].reduce_weights_sync()
+                emit(PYDTNN_MDL_EVENT, self.layers[i].id * PYDTNN_MDL_EVENTS + PYDTNN_MDL_UPDATE_DW)
+                self.layers[i].update_weights(optimizer)
+                emit(PYDTNN_MDL_EVENT, 0)
+        finally:
             self._join_side_stream()
-        for i in range(len(self.layers) - 1, 0, -1):
-            self.layers[i].reduce_weights_sync()
-            emit(PYDTNN_MDL_EVENT, self.layers[i].id * PYDTNN_MDL_EVENTS + PYDTNN_MDL_UPDATE_DW)
-            self.layers[i].update_weights(optimizer)
-            emit(PYDTNN_MDL_EVENT, 0)
         return loss
 
     @contextlib.contextmanager
-    def beside_backward(self, *tensors):
-        """Inside train_batch with ``enable_backward_overlap``: the body's work goes to the model's second stream,
-        after everything enqueued so far on the caller's; ``tensors`` (what the body reads) stay referenced until
+    def beside_backward(self, layer, *tensors):
+        """Inside train_batch with ``enable_backward_overlap``: the body's work (the gradients of ``layer``'s
+        variables) goes to the model's second stream, after everything enqueued so far on the caller's, and
+        ``layer.grads_ready`` is the event that marks its end; ``tensors`` (what the body reads) stay referenced until
         the caller's stream has waited for that stream, so the allocator cannot hand their memory out in between.
         Otherwise, and for small problems (under 2^16 elements read: nothing to overlap but launches), the body
         runs in place."""
@@ -244,6 +252,8 @@ class Model:
         self._side_refs.append((side, tensors))
         with torch.cuda.stream(side):
             yield
+            layer.grads_ready = torch.cuda.Event()
+            layer.grads_ready.record(side)
 
     def _join_side_stream(self):
         for side in {s for s, _ in self._side_refs}:
