@@ -308,6 +308,38 @@ def run_other(torch, pd, args, Timer, timed_steps):
     return fn(torch, pd, timed_steps, args.steps, args.warmup)
 
 
+def resnet50_inference_extra(torch, pd, timed_steps, n=64, steps=10, warmup=2):
+    """ResNet-50 at 224x224 (pydtnn/models/resnet50_imagenet.py), NHWC, batch n, inference through
+    evaluate_dataset_batch: the fusion pass of pydtnn/model.py:294-349 with every enable_fused_* flag on, against
+    the same network layer by layer.  FLOPs are those of its convolutions and FC layer (2 per multiply-add)."""
+    import numpy as np
+    out = {}
+    x = torch.from_numpy(np.random.default_rng(0).random((n, 224, 224, 3), dtype=np.float32)).cuda()
+    for key, flags in (("fused", dict(enable_fused_bn_relu=True, enable_fused_conv_relu=True, enable_fused_conv_bn=True,
+                                      enable_fused_conv_bn_relu=True)), ("layerwise", {})):
+        np.random.seed(0)
+        model = pd.Model(tensor_format="NHWC", batch_size=n, **flags)
+        pd.models.create_resnet50_imagenet(model)
+        flop = 0.0   # counted before the fusion pass replaces the layers
+        for layer in model.get_all_layers():
+            if layer.canonical_name == "Conv2D":
+                flop += 2.0 * layer.co * layer.ci * layer.kh * layer.kw * layer.ho * layer.wo
+            elif layer.canonical_name == "FC":
+                flop += 2.0 * layer.weights.shape[0] * layer.weights.shape[1]
+        model.evaluate_dataset_batch(x)
+
+        def step(timers, model=model):
+            model.evaluate_batch(x)
+
+        ms, _ = timed_steps(torch, step, steps, warmup)
+        out[f"resnet50_nhwc_{key}_inference_ms"] = round(ms, 3)
+        out[f"resnet50_nhwc_{key}_inference_img_per_s"] = round(n / (ms * 1e-3), 1)
+        out["resnet50_gflop_per_image"] = round(flop / 1e9, 2)
+        out[f"resnet50_nhwc_{key}_inference_tflops"] = round(n * flop / (ms * 1e-3) / 1e12, 1)
+        del model
+    return out
+
+
 def other_configs_extra(torch, pd, timed_steps, cpu=True, steps=50, warmup=5):
     """cfg1, cfg3 and cfg4 for the default run's `extra`: GPU time and rate of each beside its CPU route."""
     out = {}
@@ -322,6 +354,7 @@ def other_configs_extra(torch, pd, timed_steps, cpu=True, steps=50, warmup=5):
         if name == "cfg4":
             out["cfg4_unfused_ms"] = extra["unfused_ms"]
             out["cfg4_gbs_of_min_traffic"] = extra["block_gbs_vs_8TBs"]
+    out.update(resnet50_inference_extra(torch, pd, timed_steps))
     if cpu:
         for name, _, budget in configs:
             out[f"{name}_cpu_baseline"] = cpu_baseline_other(name, budget)
