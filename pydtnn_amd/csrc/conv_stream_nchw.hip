@@ -353,12 +353,12 @@ int launch_stream_nchw(const StreamNchwArgs& a, hipStream_t stream)
 
 // The (format, filters, chunks of 16 reduction indices, padded?) combinations that are built.  NCHW: AlexNet's first
 // layer (96 filters, 3 x 11 x 11 = 363 taps, no padding), VGG's (64 filters, 3 x 3 x 3 = 27 taps, padded) and
-// ResNet's (64 filters, 3 x 7 x 7 = 147 taps, padded).  NHWC: VGG's, and 32 filters over at most 16 taps (a 3 x 3
-// layer on one channel).
+// ResNet's (64 filters, 3 x 7 x 7 = 147 taps, padded).  NHWC: VGG's and ResNet's, and 32 filters over at most 16
+// taps (a 3 x 3 layer on one channel).
 bool stream_first_shape_built(int nhwc, int kn, int k, bool padded)
 {
     const int chunks = (k + 15) / 16;
-    if (nhwc) return padded && ((kn == 64 && chunks == 2) || (kn == 32 && chunks == 1));
+    if (nhwc) return padded && ((kn == 64 && (chunks == 2 || chunks == 10)) || (kn == 32 && chunks == 1));
     if (!padded) return kn == 96 && chunks == 23;
     return kn == 64 && (chunks == 2 || chunks == 10);
 }
@@ -396,6 +396,7 @@ int conv_stream_first(int nhwc, const ConvGeom& g, const float* w, const float* 
     STREAM_FIRST_CASE(false, 64, 2, true);
     STREAM_FIRST_CASE(false, 64, 10, true);
     STREAM_FIRST_CASE(true, 64, 2, true);
+    STREAM_FIRST_CASE(true, 64, 10, true);
     STREAM_FIRST_CASE(true, 32, 1, true);
 #undef STREAM_FIRST_CASE
     return PYDTNN_HIP_ERR_UNSUPPORTED;

@@ -325,13 +325,16 @@ def test_streaming_kernel_shapes_nchw(cg, oracle, d):
         assert np.array_equal(y2, host(y))
 
 
-# NHWC first layers on the same kernel: VGG's 3 x 3 x 3 -> 64 (ragged planes, mixed padding and stride, dilation)
+# NHWC first layers on the same kernel: VGG's 3 x 3 x 3 -> 64 (ragged planes, mixed padding and stride, dilation),
+# ResNet's 7 x 7 x 3 -> 64 at stride 2
 # and 32 filters over at most 16 taps (MNIST's 3 x 3 on one channel; 2 x 2 x 4 taps; a padded 1 x 1 on 9 channels)
 stream_first_nhwc_grid = [
     D(2, 3, 224, 224, 64, 3, 3, 1, 1, 1, 1, 1, 1),
     D(20, 3, 50, 47, 64, 3, 3, 1, 1, 1, 1, 1, 1),
     D(20, 3, 57, 61, 64, 3, 3, 2, 0, 1, 2, 1, 1),
     D(3, 3, 130, 130, 64, 3, 3, 2, 2, 1, 1, 2, 2),
+    D(4, 3, 224, 224, 64, 7, 7, 3, 3, 2, 2, 1, 1),
+    D(9, 3, 131, 117, 64, 7, 7, 3, 2, 2, 2, 1, 1),
     D(64, 1, 28, 28, 32, 3, 3, 1, 1, 1, 1, 1, 1),
     D(7, 4, 70, 81, 32, 2, 2, 1, 1, 1, 1, 1, 1),
     D(3, 9, 110, 110, 32, 1, 1, 1, 1, 1, 1, 1, 1),
