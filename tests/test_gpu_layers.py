@@ -394,30 +394,31 @@ def test_relu_folding_changes_no_bit_of_a_training_run(pd, fmt, monkeypatch):
     assert calls_a == {"fwd": 2, "bwd": 2}   # only the Relu between the FC layers
 
 
+@pytest.mark.parametrize("n,hw,c1", [(8, 16, 8), (32, 48, 32)])
 @pytest.mark.parametrize("conv_gemm", [True, False])
 @pytest.mark.parametrize("fmt", ["NCHW", "NHWC"])
-def test_backward_overlap_changes_no_bit_of_a_training_run(pd, fmt, conv_gemm):
-    """Three training steps of a small network with a residual block, with the filter / bias gradients on the
+def test_backward_overlap_changes_no_bit_of_a_training_run(pd, fmt, conv_gemm, n, hw, c1):
+    """Eight training steps of a small network with a residual block, with the filter / bias gradients on the
     model's second stream (the default) and with everything on the caller's stream: losses, every gradient and
     every updated weight are identical; the second stream is used by the one run only, and nothing of a step is
     left on it when train_batch returns."""
-    announce("backward overlap", fmt, conv_gemm)
-    n, classes = 8, 10
+    announce("backward overlap", fmt, conv_gemm, n, hw, c1)
+    classes = 10
     rng = np.random.default_rng(23)
-    x = dev(rng.random((n, 3, 16, 16) if fmt == "NCHW" else (n, 16, 16, 3)).astype(np.float32))
+    x = dev(rng.random((n, 3, hw, hw) if fmt == "NCHW" else (n, hw, hw, 3)).astype(np.float32))
     y_targ = dev(np.eye(classes, dtype=np.float32)[rng.integers(0, classes, n)])
 
     def run(overlap):
         np.random.seed(7)
         model = pd.Model(tensor_format=fmt, batch_size=n, enable_backward_overlap=overlap, enable_conv_gemm=conv_gemm)
         model._overlap_min_elements = 0      # problems this small would otherwise stay on one stream
-        model.add(pd.Input(shape=(16, 16, 3)))
-        model.add(pd.Conv2D(nfilters=8, filter_shape=(3, 3), padding=1, activation="relu", weights_initializer="he_normal"))
-        model.add(pd.AdditionBlock([pd.Conv2D(nfilters=8, filter_shape=(3, 3), padding=1, weights_initializer="he_normal"),
+        model.add(pd.Input(shape=(hw, hw, 3)))
+        model.add(pd.Conv2D(nfilters=c1, filter_shape=(3, 3), padding=1, activation="relu", weights_initializer="he_normal"))
+        model.add(pd.AdditionBlock([pd.Conv2D(nfilters=c1, filter_shape=(3, 3), padding=1, weights_initializer="he_normal"),
                                     pd.BatchNormalization(), pd.Relu(),
-                                    pd.Conv2D(nfilters=8, filter_shape=(1, 1), weights_initializer="he_normal")], []))
+                                    pd.Conv2D(nfilters=c1, filter_shape=(1, 1), weights_initializer="he_normal")], []))
         model.add(pd.Relu())
-        model.add(pd.Conv2D(nfilters=12, filter_shape=(3, 3), padding=1, stride=2, activation="relu",
+        model.add(pd.Conv2D(nfilters=c1 + 4, filter_shape=(3, 3), padding=1, stride=2, activation="relu",
                             weights_initializer="he_normal"))
         model.add(pd.MaxPool2D(pool_shape=(2, 2), stride=2))
         model.add(pd.Flatten())
@@ -425,9 +426,10 @@ def test_backward_overlap_changes_no_bit_of_a_training_run(pd, fmt, conv_gemm):
         model.add(pd.FC(shape=(classes,), activation="softmax", weights_initializer="he_normal"))
         loss_fn, opt = pd.CategoricalCrossEntropy(), pd.SGD(learning_rate=0.05, momentum=0.9)
         losses = []
-        for _ in range(3):
-            losses.append(float(model.train_batch(x, y_targ, loss_fn, opt)))
+        for _ in range(8):     # long enough for the caching allocator to hand freed blocks out again
+            losses.append(model.train_batch(x, y_targ, loss_fn, opt))    # no synchronization between the steps
             assert not model._side_refs
+        losses = [float(v) for v in losses]
         state = {}
         for l in model.get_all_layers():
             for var, grad in l.grad_vars.items():
