@@ -19,9 +19,13 @@
 //   * the wavefronts of a compute unit are at different points of their units, so stores, loads and MFMAs
 //     of different wavefronts overlap;
 //   * units are dealt to the wavefronts of a workgroup from a counter in LDS (each workgroup owns a contiguous
-//     range of pixel blocks); which wavefront computes a unit does not change a bit of it.
+//     range of pixel blocks); which wavefront computes a unit does not change a bit of it;
+//   * a launch walks the pixel blocks from the first to the last or the other way round, whichever starts with
+//     the part of its largest input that an earlier launch on the stream touched last: a 1x1 layer on 205 MB is
+//     bound by memory, and the end of what the previous kernel wrote (or read) is still in the memory-side cache.
 // The store applies bias -> BN -> ReLU and one of: gate, ReLU mask, residual (+ ReLU), like the tile engine's.
 #include "conv_internal.h"
+#include <mutex>
 #include <type_traits>
 
 namespace convint {
@@ -47,6 +51,7 @@ struct StreamArgs {
     int chunks;          // reduction chunks of 64: kh*kw * (c / 64)
     int cchunks;         // c / 64
     int row_blocks;      // p / 32
+    int reverse;         // workgroups and their units take the pixel blocks from the last to the first
 };
 
 typedef float floatx4s __attribute__((ext_vector_type(4)));
@@ -68,8 +73,9 @@ __global__ void __launch_bounds__(64 * stream_waves(CHUNKS, MASKS)) conv_stream_
     const int ln = lane & 31, lh = lane >> 5;
 
     // this workgroup's range of pixel blocks
-    const int rb0 = (int)((long)blockIdx.x * a.row_blocks / gridDim.x);
-    const int rb1 = (int)((long)(blockIdx.x + 1) * a.row_blocks / gridDim.x);
+    const int wg = a.reverse ? (int)(gridDim.x - 1 - blockIdx.x) : (int)blockIdx.x;
+    const int rb0 = (int)((long)wg * a.row_blocks / gridDim.x);
+    const int rb1 = (int)((long)(wg + 1) * a.row_blocks / gridDim.x);
     const int units = (rb1 - rb0) * CG;
 
     // ---- set-up: filter matrix and per-channel parameters into LDS
@@ -122,7 +128,7 @@ __global__ void __launch_bounds__(64 * stream_waves(CHUNKS, MASKS)) conv_stream_
         uint32_t base;   // byte offset of (img, ih0, iw0, channel 4h) from the shifted start
         uint32_t inv;    // tap mask: bit t set when tap t lies in the padding (bit 31 always set)
     };
-    auto unit_block = [&](int unit) { return rb0 + unit / CG; };
+    auto unit_block = [&](int unit) { return a.reverse ? rb1 - 1 - unit / CG : rb0 + unit / CG; };
     auto unit_group = [&](int unit) { return unit - (unit / CG) * CG; };
     auto setup_load = [&](int unit, LoadSide& ls) {
         const long m = (long)unit_block(unit) * 32 + ln;
@@ -348,6 +354,59 @@ bool stream_shape_built(int kn, int chunks)
     }
 }
 
+// The direction of a launch.  Per stream, the tensors the last few launches walked and the direction they walked
+// them in; a new launch goes the other way than the launch that last touched its residual (if it has one: that is
+// its largest input) or else its input, so that it begins where that one ended, and forwards when neither is
+// known.  Results do not depend on the direction; the table only has to be consistent, hence the mutex.
+struct Walk {
+    const void* tensor;
+    int reverse;
+};
+struct StreamWalks {
+    hipStream_t stream;
+    bool used;
+    int next;
+    Walk walks[6];
+};
+std::mutex walks_mutex;
+StreamWalks stream_walks[8];
+int next_stream_slot = 0;
+
+int choose_direction(hipStream_t stream, const void* x, const void* residual, const void* y)
+{
+    std::lock_guard<std::mutex> lock(walks_mutex);
+    StreamWalks* sw = nullptr;
+    for (StreamWalks& c : stream_walks)
+        if (c.used && c.stream == stream) sw = &c;
+    if (!sw) {
+        sw = &stream_walks[next_stream_slot];
+        next_stream_slot = (next_stream_slot + 1) % 8;
+        *sw = StreamWalks{};
+        sw->stream = stream;
+        sw->used = true;
+    }
+    auto last_walk = [&](const void* t) {
+        if (t)
+            for (const Walk& wk : sw->walks)
+                if (wk.tensor == t) return wk.reverse;
+        return -1;
+    };
+    int seen = last_walk(residual);
+    if (seen < 0) seen = last_walk(x);
+    const int reverse = seen < 0 ? 0 : !seen;
+    auto note = [&](const void* t) {
+        if (!t) return;
+        for (Walk& wk : sw->walks)
+            if (wk.tensor == t) { wk.reverse = reverse; return; }
+        sw->walks[sw->next] = Walk{t, reverse};
+        sw->next = (sw->next + 1) % 6;
+    };
+    note(x);
+    note(residual);
+    note(y);
+    return reverse;
+}
+
 }  // namespace
 
 // Shapes the streaming kernel takes: the filter matrix fits LDS, channels come in chunks of 64 floats that
@@ -370,6 +429,7 @@ int conv_stream_nhwc(const ConvGeom& g, const float* w, const float* x, float* y
     a.cchunks = g.c / 64;
     a.chunks = g.khw * a.cchunks;
     a.row_blocks = (int)(g.p / 32);
+    a.reverse = choose_direction(stream, x, masks.residual, y);
 #define STREAM_CASE(KN, CH) \
     if (g.kn == KN && a.chunks == CH) return launch_stream_masks<KN, CH>(a, stream)
     STREAM_CASE(64, 1); STREAM_CASE(64, 2); STREAM_CASE(64, 4); STREAM_CASE(64, 9);

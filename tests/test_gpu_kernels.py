@@ -234,8 +234,13 @@ def test_streaming_kernel_shapes_nhwc(cg, oracle, d):
     xr, wr, dyr = nhwc(x), w_nhwc(w), nhwc(dy)
     p = oracle.ConvParams(*d.geom())
     y_ref, rows = oracle.conv2d_forward_nhwc_i2c(xr, wr, b, p)
-    y = cg.conv_gemm_nhwc(dev(wr), dev(xr), biases_vector=dev(b), **_kw(d))
+    xd = dev(xr)
+    y = cg.conv_gemm_nhwc(dev(wr), xd, biases_vector=dev(b), **_kw(d))
     assert_close(host(y), y_ref, what="y")
+    # the same input again: the kernel now walks the pixel blocks from the other end (it starts where the launch
+    # that last touched its input ended), and once more the first way round; not a bit may change
+    for _ in range(2):
+        assert torch.equal(cg.conv_gemm_nhwc(dev(wr), xd, biases_vector=dev(b), **_kw(d)), y)
     y = cg.conv_gemm_nhwc(dev(wr), dev(xr), biases_vector=dev(b), bn_running_mean=dev(bn[0]), bn_inv_std=dev(bn[1]),
                           bn_gamma=dev(bn[2]), bn_beta=dev(bn[3]), relu=True, **_kw(d))
     assert_close(host(y), oracle.fused_epilogue(y_ref, "NHWC", bn=bn, relu_flag=True), what="fused y")
