@@ -258,8 +258,9 @@ int pydtnn_hip_max_pool_2d_bwd_gated(int nhwc, const float *dy, const int32_t *i
  *                                           AdditionBlockCPU.forward applies it
  *                                           (pydtnn/backends/cpu/layers/addition_block_cpu.py:41-45)
  *     y = y > 0 ? y : 0                     when relu_after_add: the Relu layer that follows the block
- * with `residual` shaped like y.  Results equal the separate calls bit for bit.  residual may alias neither x
- * nor y.  Same optional workspace as the forward. */
+ * with `residual` shaped like y.  Results equal the separate calls bit for bit.  residual must not alias y;
+ * it may be x itself (both are only read: a block whose folded path is one convolution and whose other path is
+ * the identity passes the block input twice).  Same optional workspace as the forward. */
 int pydtnn_hip_sconvGemm_residual(int nhwc, unsigned b, unsigned c, unsigned h, unsigned w, unsigned kn, unsigned kh,
                                   unsigned kw, unsigned vpadding, unsigned hpadding, unsigned vstride,
                                   unsigned hstride, unsigned vdilation, unsigned hdilation, const float *weights,

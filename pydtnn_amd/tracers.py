@@ -139,6 +139,8 @@ class SimpleTracer(Tracer):
             for evt_type, events in self.events.items():
                 for value, (calls, times) in events.items():
                     times = sorted(times)
+                    if not times:   # an event that was opened and never closed has no duration to report
+                        continue
                     f.write(f"{self.type_names[evt_type]};{value};{self.name_of(evt_type, value)};{calls};"
                             f"{sum(times)};{times[len(times) // 2]}\n")
 

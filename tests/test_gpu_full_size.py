@@ -28,9 +28,12 @@ def pd():
     return pydtnn_amd
 
 
-def sampled_conv3x3_check(x, w, b, dy, y, dw, db, dx, samples=2000, dw_samples=10, seed=0):
+def sampled_conv3x3_check(x, w, b, dy, y, dw, db, dx, samples=2000, dw_samples=10, seed=0, relu_y=False,
+                          gate_dx=None):
     """x (n,c,h,w), w (co,c,3,3), dy / y (n,co,h,w), dx like x or None: NCHW host arrays of a 3x3, pad 1, stride 1
-    convolution.  Returns the largest errors relative to each result's largest magnitude."""
+    convolution.  Returns the largest errors relative to each result's largest magnitude.  ``relu_y``: y holds
+    relu(conv + b); ``gate_dx``: a boolean array like x, dx holds the input gradient where it is True and 0
+    elsewhere (the forms a training step produces when a Relu layer's work is done by its neighbours)."""
     n, c, h, wd = x.shape
     co = w.shape[0]
     rng = np.random.default_rng(seed)
@@ -55,11 +58,15 @@ def sampled_conv3x3_check(x, w, b, dy, y, dw, db, dx, samples=2000, dw_samples=1
     errs = {}
     # y[n,o,oy,ox] = b[o] + sum_{c,i,j} w[o,c,i,j] x[n,c,oy+i-1,ox+j-1]
     ref_y = np.einsum("sck,sck->s", taps(x, c, False), w[oc].reshape(s, c, 9).astype(np.float64)) + b[oc]
+    if relu_y:
+        ref_y = np.maximum(ref_y, 0.0)
     errs["y"] = float(np.max(np.abs(y[ni, oc, oy, ox] - ref_y)) / np.abs(y).max())
     if dx is not None:
         # dx[n,c,y,x] = sum_{o,i,j} w[o,c,i,j] dy[n,o,y+1-i,x+1-j]
         ref_dx = np.einsum("sok,sok->s", taps(dy, co, True),
                            w[:, ic].transpose(1, 0, 2, 3).reshape(s, co, 9).astype(np.float64))
+        if gate_dx is not None:
+            ref_dx = ref_dx * gate_dx[ni, ic, oy, ox]
         errs["dx"] = float(np.max(np.abs(dx[ni, ic, oy, ox] - ref_dx)) / np.abs(dx).max())
     # dw[o,c,i,j] = sum_{n,oy,ox} dy[n,o,oy,ox] x[n,c,oy+i-1,ox+j-1]
     worst = 0.0
@@ -143,3 +150,105 @@ def test_vgg16_fc_layers_at_batch_64(pd, shape):
     assert np.max(np.abs(got_dw[rows] - ref_dw)) / np.abs(ref_dw).max() <= FP32_REL_TOL
     # the rows outside the band: column sums are linear in dw, sum_i dw[i, :] = (sum_i x[:, i])^T dy
     assert_close(got_dw.sum(axis=0, dtype=np.float64), x64.sum(axis=1) @ dy64, what="fc dw column sums")
+
+
+# --------------------------------------------------------------------------- the training step as the benchmark runs it
+def _vgg16_for_step(pd, fmt, **flags):
+    np.random.seed(0)
+    model = pd.Model(tensor_format=fmt, batch_size=64, **flags)
+    return pd.models.create_vgg16_imagenet(model, dropout=False, initializer="he_normal")
+
+
+def _trainable_state(model):
+    """Every tensor a training step changes: (name, tensor) for weights, biases and their velocities."""
+    out = []
+    for layer in model.get_all_layers():
+        for var in layer.grad_vars:
+            out.append((f"{layer!r}.{var}", getattr(layer, var)))
+            out.append((f"{layer!r}.velocity_{var}", getattr(layer, "velocity_" + var)))
+    return out
+
+
+def _record_convolutions(model, ids):
+    """Wraps forward / backward of the named convolutions so that the tensors of the last step stay at hand:
+    x (the layer's input), y (what its forward returned), dy (what its backward received), dx (what it returned)."""
+    seen = {}
+    for layer in model.layers:
+        if layer.canonical_name != "Conv2D" or layer.id not in ids:
+            continue
+        rec = seen[layer.id] = {"layer": layer}
+
+        def wrap(fwd, bwd, rec):
+            def forward(x):
+                rec["x"] = x
+                rec["y"] = fwd(x)
+                return rec["y"]
+
+            def backward(dy):
+                rec["dy"] = dy
+                rec["dx"] = bwd(dy)
+                return rec["dx"]
+            return forward, backward
+
+        layer.forward, layer.backward = wrap(layer.forward, layer.backward, rec)
+    return seen
+
+
+@pytest.mark.parametrize("fmt", ["NCHW", "NHWC"])
+def test_vgg16_training_step_variants_at_batch_64(pd, fmt):
+    """Two train_batch steps of VGG16 at batch 64, as bench.py runs them: the default model (a Relu layer's work
+    done by the stores of its neighbours, filter gradients on a second stream), the model with every Relu layer
+    making its own passes, and the model with the whole backward pass on one stream must leave bit-identical
+    weights, biases and velocities in every layer.  For the default model in NCHW the folded tensors of three
+    convolutions, taken from inside the second step, are recomputed on the host in float64 at sampled positions:
+    y = relu(conv(x) + b), dw and db from the dy the layer received, and dx multiplied by the mask of the Relu
+    below.  The pattern of pydtnn/tests/check_conv_gemm_models.py:100-167 (same model, two code paths, layer by
+    layer) at the benchmark's size."""
+    announce("vgg16 training step, three variants", fmt)
+    n = 64
+    rng = np.random.default_rng(0)
+    x = torch.from_numpy(rng.random((n, 3, 224, 224), dtype=np.float32)).cuda()
+    if fmt == "NHWC":
+        x = x.permute(0, 2, 3, 1).contiguous()
+    y_targ = torch.zeros((n, 1000), device="cuda")
+    y_targ[torch.arange(n), torch.from_numpy(rng.integers(0, 1000, n)).cuda()] = 1.0
+    loss_fn = pd.CategoricalCrossEntropy()
+    variants = {"default": {}, "separate relu": dict(enable_relu_folding=False),
+                "one stream": dict(enable_backward_overlap=False)}
+    states, losses, recorded = {}, {}, None
+    for name, flags in variants.items():
+        announce("  variant", name)
+        model = _vgg16_for_step(pd, fmt, **flags)
+        opt = pd.SGD(learning_rate=0.01, momentum=0.9)
+        if name == "default" and fmt == "NCHW":
+            # conv1_2 (64 -> 64 at 224), conv3_2 (256 -> 256 at 56), conv5_1 (512 -> 512 at 14)
+            convs = [l for l in model.layers if l.canonical_name == "Conv2D"]
+            recorded = _record_convolutions(model, {convs[1].id, convs[5].id, convs[10].id})
+        losses[name] = [float(model.train_batch(x, y_targ, loss_fn, opt))]
+        # the parameters the second step computes with (biases are no longer zero there)
+        before = {i: (host(r["layer"].weights), host(r["layer"].biases)) for i, r in (recorded or {}).items()} \
+            if name == "default" else {}
+        losses[name].append(float(model.train_batch(x, y_targ, loss_fn, opt)))
+        torch.cuda.synchronize()
+        states[name] = [(k, t.clone()) for k, t in _trainable_state(model)]
+        for i, (w_before, b_before) in before.items():
+            rec = recorded[i]
+            layer = rec["layer"]
+            announce("  sampled float64 check of", repr(layer), tuple(rec["x"].shape))
+            assert layer.relu_above is not None and rec["y"].min().item() >= 0.0   # the store did the Relu above
+            xh = host(rec["x"])
+            gate = xh > 0 if layer.relu_below is not None else None   # ... and the dx store the Relu below
+            errs = sampled_conv3x3_check(xh, w_before, b_before, host(rec["dy"]), host(rec["y"]), host(layer.dw),
+                                         host(layer.db), host(rec["dx"]), relu_y=True, gate_dx=gate)
+            print("   max errors relative to scale:", {k: f"{e:.2e}" for k, e in errs.items()}, flush=True)
+            for k, e in errs.items():
+                assert e <= FP32_REL_TOL, f"{layer!r}: {k} error {e:.3e}"
+            rec.clear()
+        del model
+    assert losses["default"] == losses["separate relu"] == losses["one stream"], losses
+    assert np.isfinite(losses["default"]).all() and losses["default"][1] != losses["default"][0]
+    for name in ("separate relu", "one stream"):
+        for (k, a), (k2, b) in zip(states["default"], states[name]):
+            assert k == k2
+            assert torch.equal(a, b), f"{fmt}: {k} differs between the default model and '{name}'"
+    assert len(states["default"]) == 2 * 2 * 16   # 13 convolutions + 3 FC layers, weights and biases, + velocities

@@ -51,7 +51,8 @@ def test_simple_tracer_times_nested_regions_and_writes_the_table(tmp_path, monke
     tr.emit_event(t.PYDTNN_MDL_EVENT, fwd)
     with pytest.raises(ValueError):
         tr.emit_event(t.PYDTNN_OPS_EVENT, 0)                      # closes the wrong type
-    tr.write_output()
+    assert tr.events[t.PYDTNN_OPS_EVENT][12345] == [0, []]       # a lookup leaves an entry without durations behind
+    tr.write_output()                                             # ... which the table skips
     lines = out.read_text().splitlines()
     assert lines[0] == "Event type;Event value;Event name;Calls;Total time;Median of times"
     assert f"Operations;{op};001_Conv2D_forward_convgemm;4;10.0;2.0" in lines
