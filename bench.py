@@ -39,7 +39,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"])
+    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "resnet50"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-vgg16", action="store_true", help="skip the VGG16 training-step extra of the default run")
     ap.add_argument("--no-other-configs", action="store_true",
@@ -499,6 +499,19 @@ def main():
         roofline = {"bound": "mfma", "kernel": "whole step", "achieved": round(value / 1e3, 3),
                     "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(value / 1e3 / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": None}
+    elif args.workload == "resnet50":
+        # not one of the five configurations: the whole network around cfg4's block, for kernel traces
+        from bench_configs import resnet50_inference_extra
+        extra = resnet50_inference_extra(torch, pd, timed_steps, steps=args.steps, warmup=args.warmup,
+                                         layerwise=not args.no_folding_extra)
+        ms = extra["resnet50_nhwc_fused_inference_ms"]
+        value, unit = extra["resnet50_nhwc_fused_inference_tflops"] * 1e3, "GFLOP/s"
+        workload = ("ResNet-50 inference, fp32 NHWC, batch 64, 3x224x224, every enable_fused_* flag on "
+                    "(pydtnn/models/resnet50_imagenet.py)")
+        roofline = {"bound": "mfma", "kernel": "whole network", "achieved": round(value / 1e3, 3),
+                    "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(value / 1e3 / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": None}
+        args.no_cpu_baseline = True
     else:
         from bench_configs import run_other
         ms, value, unit, workload, roofline, extra = run_other(torch, pd, args, Timer, timed_steps)

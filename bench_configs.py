@@ -308,7 +308,7 @@ def run_other(torch, pd, args, Timer, timed_steps):
     return fn(torch, pd, timed_steps, args.steps, args.warmup)
 
 
-def resnet50_inference_extra(torch, pd, timed_steps, n=64, steps=10, warmup=2):
+def resnet50_inference_extra(torch, pd, timed_steps, n=64, steps=10, warmup=2, layerwise=True):
     """ResNet-50 at 224x224 (pydtnn/models/resnet50_imagenet.py), NHWC, batch n, inference through
     evaluate_dataset_batch: the fusion pass of pydtnn/model.py:294-349 with every enable_fused_* flag on, against
     the same network layer by layer.  FLOPs are those of its convolutions and FC layer (2 per multiply-add)."""
@@ -316,7 +316,7 @@ def resnet50_inference_extra(torch, pd, timed_steps, n=64, steps=10, warmup=2):
     out = {}
     x = torch.from_numpy(np.random.default_rng(0).random((n, 224, 224, 3), dtype=np.float32)).cuda()
     for key, flags in (("fused", dict(enable_fused_bn_relu=True, enable_fused_conv_relu=True, enable_fused_conv_bn=True,
-                                      enable_fused_conv_bn_relu=True)), ("layerwise", {})):
+                                      enable_fused_conv_bn_relu=True)), ("layerwise", {}))[:2 if layerwise else 1]:
         np.random.seed(0)
         model = pd.Model(tensor_format="NHWC", batch_size=n, **flags)
         pd.models.create_resnet50_imagenet(model)
