@@ -345,6 +345,42 @@ int pydtnn_hip_relu_bwd_f64(const double *dy, const int8_t *mask, double *dx, lo
 int pydtnn_hip_bias_grad_f64(const double *dy, double *db, long outer, int channels, long inner, void *stream);
 int pydtnn_hip_transpose_1023_f64(const double *src, double *dst, int d0, int d1, long inner, void *stream);
 
+/* The layers around the convolutions in float64, so that a float64 model runs a whole training step as it does in
+ * the reference: its pooling and BN-training modules dispatch on float64
+ * (pydtnn/cython_modules/max_pool_2d_nchw_cython.pyx:42-49 and :157-164, max_pool_2d_nhwc_cython.pyx,
+ * average_pool_2d_nchw_cython.pyx / _nhwc_cython.pyx, bn_training_cython.pyx), and softmax
+ * (pydtnn/backends/cpu/activations/softmax_cpu.py:32-39), categorical cross-entropy
+ * (pydtnn/backends/cpu/losses/categorical_cross_entropy_cpu.py:28-35) and SGD
+ * (pydtnn/backends/cpu/optimizers/sgd_cpu.py:28-41) are NumPy expressions in the model's dtype.  Same rules as the
+ * float32 entry points above (first maximum wins; stored index ii*kw + jj decoded as idx / kh, idx % kw; sums in
+ * the reference's order); nhwc = 0 / 1 selects the tensor format, b, c, h, w name the input's extents in either.
+ * The cross-entropy needs rows * 8 bytes of workspace, the others none. */
+int pydtnn_hip_max_pool_2d_fwd_f64(int nhwc, const double *x, double *y, int32_t *idx_max, int b, int c, int h, int w,
+                                   int kh, int kw, int vpadding, int hpadding, int vstride, int hstride, int vdilation,
+                                   int hdilation, void *stream);
+int pydtnn_hip_max_pool_2d_bwd_f64(int nhwc, const double *dy, const int32_t *idx_max, double *dx, int b, int c, int h,
+                                   int w, int kh, int kw, int vpadding, int hpadding, int vstride, int hstride,
+                                   int vdilation, int hdilation, void *stream);
+int pydtnn_hip_average_pool_2d_fwd_f64(int nhwc, const double *x, double *y, int b, int c, int h, int w, int kh, int kw,
+                                       int vpadding, int hpadding, int vstride, int hstride, int vdilation,
+                                       int hdilation, void *stream);
+int pydtnn_hip_average_pool_2d_bwd_f64(int nhwc, const double *dy, double *dx, int b, int c, int h, int w, int kh,
+                                       int kw, int vpadding, int hpadding, int vstride, int hstride, int vdilation,
+                                       int hdilation, void *stream);
+int pydtnn_hip_softmax_fwd_f64(const double *x, double *y, int rows, int cols, void *stream);
+int pydtnn_hip_softmax_bwd_f64(const double *dy, const double *y, double *dx, int rows, int cols, void *stream);
+int pydtnn_hip_categorical_cross_entropy_f64(const double *y_pred, const double *y_targ, double *dx, double *loss,
+                                             int rows, int cols, double eps, int global_batch, void *workspace,
+                                             size_t workspace_bytes, void *stream);
+int pydtnn_hip_sgd_momentum_f64(double *w, const double *dw, double *velocity, long total, double lr, double momentum,
+                                double decay, int nesterov, void *stream);
+int pydtnn_hip_bn_training_fwd_f64(const double *x, double *y, double *xn, double *std_out, const double *gamma,
+                                   const double *beta, double *running_mean, double *running_var, double momentum,
+                                   double eps, long outer, int channels, long inner, void *stream);
+int pydtnn_hip_bn_training_bwd_f64(const double *dy, const double *xn, const double *std_in, const double *gamma,
+                                   double *dgamma, double *dbeta, double *dx, long outer, int channels, long inner,
+                                   void *stream);
+
 /* ------------------------------------------------------------------------------------------
  * Host-pointer compatibility flavour (exported by libconvGemm.so only).  Signatures are those
  * PyDTNN's ctypes shim calls (pydtnn/backends/cpu/libs/conv_gemm.py:91-92, :191-205, :234-248,

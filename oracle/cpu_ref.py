@@ -211,14 +211,21 @@ def eltw_sum(acc, x):
     return acc
 
 
+def _pool_array(a):
+    """Pooling runs in the array's own float32 / float64 (pydtnn/cython_modules/max_pool_2d_nchw_cython.pyx:42-49
+    dispatches on the dtype); anything else is taken as float32."""
+    a = np.asarray(a)
+    return np.ascontiguousarray(a, dtype=a.dtype if a.dtype == np.float64 else np.float32)
+
+
 def max_pool_2d_fwd_nchw(x, kh, kw, vpadding, hpadding, vstride, hstride, vdilation=1, hdilation=1):
     """pydtnn/cython_modules/max_pool_2d_nchw_cython.pyx:25-52"""
-    x = np.ascontiguousarray(x, dtype=np.float32)
+    x = _pool_array(x)
     n, c, h, w = x.shape
     hh, ww = out_hw(h, w, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
-    y = np.zeros((n, c, hh, ww), dtype=np.float32)
+    y = np.zeros((n, c, hh, ww), dtype=x.dtype)
     idx = np.zeros((n, c, hh, ww), dtype=np.int32)
-    lib().oracle_max_pool_2d_fwd_nchw_f32(_p(x), _p(y), _p(idx), n, c, h, w, kh, kw, vpadding, hpadding,
+    getattr(lib(), "oracle_max_pool_2d_fwd_nchw_" + _sfx(x.dtype))(_p(x), _p(y), _p(idx), n, c, h, w, kh, kw, vpadding, hpadding,
                                           vstride, hstride, vdilation, hdilation)
     return y, idx
 
@@ -226,10 +233,10 @@ def max_pool_2d_fwd_nchw(x, kh, kw, vpadding, hpadding, vstride, hstride, vdilat
 def max_pool_2d_bwd_nchw(dy, idx_max, n, c, h, w, kh, kw, vpadding, hpadding, vstride, hstride,
                          vdilation=1, hdilation=1):
     """pydtnn/cython_modules/max_pool_2d_nchw_cython.pyx:140-166"""
-    dy = np.ascontiguousarray(dy, dtype=np.float32)
+    dy = _pool_array(dy)
     idx_max = np.ascontiguousarray(idx_max, dtype=np.int32)
-    dx = np.zeros((n, c, h, w), dtype=np.float32)
-    lib().oracle_max_pool_2d_bwd_nchw_f32(_p(dy), _p(idx_max), _p(dx), n, c, h, w, kh, kw, vpadding, hpadding,
+    dx = np.zeros((n, c, h, w), dtype=dy.dtype)
+    getattr(lib(), "oracle_max_pool_2d_bwd_nchw_" + _sfx(dy.dtype))(_p(dy), _p(idx_max), _p(dx), n, c, h, w, kh, kw, vpadding, hpadding,
                                           vstride, hstride, vdilation, hdilation)
     return dx
 
@@ -237,15 +244,15 @@ def max_pool_2d_bwd_nchw(dy, idx_max, n, c, h, w, kh, kw, vpadding, hpadding, vs
 def average_pool_2d_fwd(x, tensor_format, kh, kw, vpadding, hpadding, vstride, hstride, vdilation=1, hdilation=1):
     """pydtnn/cython_modules/average_pool_2d_nchw_cython.pyx:25-52 / average_pool_2d_nhwc_cython.pyx:25-52.
     ``kh`` / ``kw`` of 0 mean the whole extent (pydtnn/layers/abstract_pool_2d_layer.py:44-47)."""
-    x = np.ascontiguousarray(x, dtype=np.float32)
+    x = _pool_array(x)
     if tensor_format == "NCHW":
         n, c, h, w = x.shape
     else:
         n, h, w, c = x.shape
     kh, kw = kh or h, kw or w
     hh, ww = out_hw(h, w, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
-    y = np.zeros((n, c, hh, ww) if tensor_format == "NCHW" else (n, hh, ww, c), dtype=np.float32)
-    fn = getattr(lib(), f"oracle_average_pool_2d_{tensor_format.lower()}_fwd_f32")
+    y = np.zeros((n, c, hh, ww) if tensor_format == "NCHW" else (n, hh, ww, c), dtype=x.dtype)
+    fn = getattr(lib(), f"oracle_average_pool_2d_{tensor_format.lower()}_fwd_{_sfx(x.dtype)}")
     fn(_p(x), _p(y), n, c, h, w, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
     return y
 
@@ -253,22 +260,22 @@ def average_pool_2d_fwd(x, tensor_format, kh, kw, vpadding, hpadding, vstride, h
 def average_pool_2d_bwd(dy, tensor_format, n, c, h, w, kh, kw, vpadding, hpadding, vstride, hstride,
                         vdilation=1, hdilation=1):
     """pydtnn/cython_modules/average_pool_2d_nchw_cython.pyx:135-160 / average_pool_2d_nhwc_cython.pyx:135-160"""
-    dy = np.ascontiguousarray(dy, dtype=np.float32)
+    dy = _pool_array(dy)
     kh, kw = kh or h, kw or w
-    dx = np.zeros((n, c, h, w) if tensor_format == "NCHW" else (n, h, w, c), dtype=np.float32)
-    fn = getattr(lib(), f"oracle_average_pool_2d_{tensor_format.lower()}_bwd_f32")
+    dx = np.zeros((n, c, h, w) if tensor_format == "NCHW" else (n, h, w, c), dtype=dy.dtype)
+    fn = getattr(lib(), f"oracle_average_pool_2d_{tensor_format.lower()}_bwd_{_sfx(dy.dtype)}")
     fn(_p(dy), _p(dx), n, c, h, w, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
     return dx
 
 
 def max_pool_2d_fwd_nhwc(x, kh, kw, vpadding, hpadding, vstride, hstride, vdilation=1, hdilation=1):
     """pydtnn/cython_modules/max_pool_2d_nhwc_cython.pyx:25-52"""
-    x = np.ascontiguousarray(x, dtype=np.float32)
+    x = _pool_array(x)
     n, h, w, c = x.shape
     hh, ww = out_hw(h, w, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
-    y = np.zeros((n, hh, ww, c), dtype=np.float32)
+    y = np.zeros((n, hh, ww, c), dtype=x.dtype)
     idx = np.zeros((n, hh, ww, c), dtype=np.int32)
-    lib().oracle_max_pool_2d_fwd_nhwc_f32(_p(x), _p(y), _p(idx), n, h, w, c, kh, kw, vpadding, hpadding,
+    getattr(lib(), "oracle_max_pool_2d_fwd_nhwc_" + _sfx(x.dtype))(_p(x), _p(y), _p(idx), n, h, w, c, kh, kw, vpadding, hpadding,
                                           vstride, hstride, vdilation, hdilation)
     return y, idx
 
@@ -276,10 +283,10 @@ def max_pool_2d_fwd_nhwc(x, kh, kw, vpadding, hpadding, vstride, hstride, vdilat
 def max_pool_2d_bwd_nhwc(dy, idx_max, n, h, w, c, kh, kw, vpadding, hpadding, vstride, hstride,
                          vdilation=1, hdilation=1):
     """pydtnn/cython_modules/max_pool_2d_nhwc_cython.pyx:140-166"""
-    dy = np.ascontiguousarray(dy, dtype=np.float32)
+    dy = _pool_array(dy)
     idx_max = np.ascontiguousarray(idx_max, dtype=np.int32)
-    dx = np.zeros((n, h, w, c), dtype=np.float32)
-    lib().oracle_max_pool_2d_bwd_nhwc_f32(_p(dy), _p(idx_max), _p(dx), n, h, w, c, kh, kw, vpadding, hpadding,
+    dx = np.zeros((n, h, w, c), dtype=dy.dtype)
+    getattr(lib(), "oracle_max_pool_2d_bwd_nhwc_" + _sfx(dy.dtype))(_p(dy), _p(idx_max), _p(dx), n, h, w, c, kh, kw, vpadding, hpadding,
                                           vstride, hstride, vdilation, hdilation)
     return dx
 

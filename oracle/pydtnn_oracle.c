@@ -279,56 +279,59 @@ DEF_ELTW(oracle_eltw_sum_f64, double)
  * decoded as ii = idx / kh, jj = idx % kw (as written in the reference; equal
  * to the encoding only for kh == kw).
  * ------------------------------------------------------------------------- */
-void oracle_max_pool_2d_fwd_nchw_f32(const float *x, float *y, int32_t *idx_max,
-                                     int n, int c, int h, int w, int kh, int kw,
-                                     int vpadding, int hpadding, int vstride, int hstride,
-                                     int vdilation, int hdilation)
-{
-    const int hh = out_dim(h, vpadding, vdilation, kh, vstride);
-    const int ww = out_dim(w, hpadding, hdilation, kw, hstride);
-    #pragma omp parallel for
-    for (int nn = 0; nn < n; nn++)
-        for (int cc = 0; cc < c; cc++)
-            for (int xx = 0; xx < hh; xx++)
-                for (int yy = 0; yy < ww; yy++) {
-                    float maxval = -FLT_MAX;
-                    int idx_maxval = 0;
-                    for (int ii = 0; ii < kh; ii++) {
-                        const int x_x = vstride * xx + vdilation * ii - vpadding;
-                        if (0 <= x_x && x_x < h)
-                            for (int jj = 0; jj < kw; jj++) {
-                                const int x_y = hstride * yy + hdilation * jj - hpadding;
-                                if (0 <= x_y && x_y < w) {
-                                    const float val = x[IDX4(nn, cc, x_x, x_y, c, h, w)];
-                                    if (val > maxval) { maxval = val; idx_maxval = ii * kw + jj; }
-                                }
-                            }
-                    }
-                    y[IDX4(nn, cc, xx, yy, c, hh, ww)] = maxval;
-                    idx_max[IDX4(nn, cc, xx, yy, c, hh, ww)] = idx_maxval;
-                }
+#define DEF_MAX_POOL_NCHW(T, SFX, LOWEST)                                                            \
+void oracle_max_pool_2d_fwd_nchw_##SFX(const T *x, T *y, int32_t *idx_max,                           \
+                                     int n, int c, int h, int w, int kh, int kw,                     \
+                                     int vpadding, int hpadding, int vstride, int hstride,           \
+                                     int vdilation, int hdilation)                                   \
+{                                                                                                    \
+    const int hh = out_dim(h, vpadding, vdilation, kh, vstride);                                     \
+    const int ww = out_dim(w, hpadding, hdilation, kw, hstride);                                     \
+    _Pragma("omp parallel for")                                                                      \
+    for (int nn = 0; nn < n; nn++)                                                                   \
+        for (int cc = 0; cc < c; cc++)                                                               \
+            for (int xx = 0; xx < hh; xx++)                                                          \
+                for (int yy = 0; yy < ww; yy++) {                                                    \
+                    T maxval = LOWEST;                                                               \
+                    int idx_maxval = 0;                                                              \
+                    for (int ii = 0; ii < kh; ii++) {                                                \
+                        const int x_x = vstride * xx + vdilation * ii - vpadding;                    \
+                        if (0 <= x_x && x_x < h)                                                     \
+                            for (int jj = 0; jj < kw; jj++) {                                        \
+                                const int x_y = hstride * yy + hdilation * jj - hpadding;            \
+                                if (0 <= x_y && x_y < w) {                                           \
+                                    const T val = x[IDX4(nn, cc, x_x, x_y, c, h, w)];                \
+                                    if (val > maxval) { maxval = val; idx_maxval = ii * kw + jj; }   \
+                                }                                                                    \
+                            }                                                                        \
+                    }                                                                                \
+                    y[IDX4(nn, cc, xx, yy, c, hh, ww)] = maxval;                                     \
+                    idx_max[IDX4(nn, cc, xx, yy, c, hh, ww)] = idx_maxval;                           \
+                }                                                                                    \
+}                                                                                                    \
+                                                                                                     \
+void oracle_max_pool_2d_bwd_nchw_##SFX(const T *dy, const int32_t *idx_max, T *dx,                   \
+                                     int n, int c, int h, int w, int kh, int kw,                     \
+                                     int vpadding, int hpadding, int vstride, int hstride,           \
+                                     int vdilation, int hdilation)                                   \
+{                                                                                                    \
+    const int hh = out_dim(h, vpadding, vdilation, kh, vstride);                                     \
+    const int ww = out_dim(w, hpadding, hdilation, kw, hstride);                                     \
+    _Pragma("omp parallel for")                                                                      \
+    for (int nn = 0; nn < n; nn++)                                                                   \
+        for (int cc = 0; cc < c; cc++)                                                               \
+            for (int xx = 0; xx < hh; xx++)                                                          \
+                for (int yy = 0; yy < ww; yy++) {                                                    \
+                    const int idx_maxval = idx_max[IDX4(nn, cc, xx, yy, c, hh, ww)];                 \
+                    const int ii = idx_maxval / kh, jj = idx_maxval % kw;                            \
+                    const int x_x = vstride * xx + vdilation * ii - vpadding;                        \
+                    const int x_y = hstride * yy + hdilation * jj - hpadding;                        \
+                    if (0 <= x_x && x_x < h && 0 <= x_y && x_y < w)                                  \
+                        dx[IDX4(nn, cc, x_x, x_y, c, h, w)] += dy[IDX4(nn, cc, xx, yy, c, hh, ww)];  \
+                }                                                                                    \
 }
-
-void oracle_max_pool_2d_bwd_nchw_f32(const float *dy, const int32_t *idx_max, float *dx,
-                                     int n, int c, int h, int w, int kh, int kw,
-                                     int vpadding, int hpadding, int vstride, int hstride,
-                                     int vdilation, int hdilation)
-{
-    const int hh = out_dim(h, vpadding, vdilation, kh, vstride);
-    const int ww = out_dim(w, hpadding, hdilation, kw, hstride);
-    #pragma omp parallel for
-    for (int nn = 0; nn < n; nn++)
-        for (int cc = 0; cc < c; cc++)
-            for (int xx = 0; xx < hh; xx++)
-                for (int yy = 0; yy < ww; yy++) {
-                    const int idx_maxval = idx_max[IDX4(nn, cc, xx, yy, c, hh, ww)];
-                    const int ii = idx_maxval / kh, jj = idx_maxval % kw;
-                    const int x_x = vstride * xx + vdilation * ii - vpadding;
-                    const int x_y = hstride * yy + hdilation * jj - hpadding;
-                    if (0 <= x_x && x_x < h && 0 <= x_y && x_y < w)
-                        dx[IDX4(nn, cc, x_x, x_y, c, h, w)] += dy[IDX4(nn, cc, xx, yy, c, hh, ww)];
-                }
-}
+DEF_MAX_POOL_NCHW(float, f32, -FLT_MAX)
+DEF_MAX_POOL_NCHW(double, f64, -DBL_MAX)
 
 /* ---------------------------------------------------------------------------
  * MaxPool2D NHWC forward / backward.
@@ -338,56 +341,60 @@ void oracle_max_pool_2d_bwd_nchw_f32(const float *dy, const int32_t *idx_max, fl
  * ------------------------------------------------------------------------- */
 #define IDX_NHWC(n_, y_, x_, c_, H, W, C) ((((long)(n_) * (H) + (y_)) * (W) + (x_)) * (C) + (c_))
 
-void oracle_max_pool_2d_fwd_nhwc_f32(const float *x, float *y, int32_t *idx_max,
-                                     int n, int h, int w, int c, int kh, int kw,
-                                     int vpadding, int hpadding, int vstride, int hstride,
-                                     int vdilation, int hdilation)
-{
-    const int hh = out_dim(h, vpadding, vdilation, kh, vstride);
-    const int ww = out_dim(w, hpadding, hdilation, kw, hstride);
-    #pragma omp parallel for
-    for (int nn = 0; nn < n; nn++)
-        for (int xx = 0; xx < hh; xx++)
-            for (int yy = 0; yy < ww; yy++)
-                for (int cc = 0; cc < c; cc++) {
-                    float maxval = -FLT_MAX;
-                    int idx_maxval = 0;
-                    for (int ii = 0; ii < kh; ii++) {
-                        const int x_x = vstride * xx + vdilation * ii - vpadding;
-                        if (0 <= x_x && x_x < h)
-                            for (int jj = 0; jj < kw; jj++) {
-                                const int x_y = hstride * yy + hdilation * jj - hpadding;
-                                if (0 <= x_y && x_y < w) {
-                                    const float val = x[IDX_NHWC(nn, x_x, x_y, cc, h, w, c)];
-                                    if (val > maxval) { maxval = val; idx_maxval = ii * kw + jj; }
-                                }
-                            }
-                    }
-                    y[IDX_NHWC(nn, xx, yy, cc, hh, ww, c)] = maxval;
-                    idx_max[IDX_NHWC(nn, xx, yy, cc, hh, ww, c)] = idx_maxval;
-                }
+#define DEF_MAX_POOL_NHWC(T, SFX, LOWEST)                                                                    \
+                                                                                                             \
+void oracle_max_pool_2d_fwd_nhwc_##SFX(const T *x, T *y, int32_t *idx_max,                                   \
+                                     int n, int h, int w, int c, int kh, int kw,                             \
+                                     int vpadding, int hpadding, int vstride, int hstride,                   \
+                                     int vdilation, int hdilation)                                           \
+{                                                                                                            \
+    const int hh = out_dim(h, vpadding, vdilation, kh, vstride);                                             \
+    const int ww = out_dim(w, hpadding, hdilation, kw, hstride);                                             \
+    _Pragma("omp parallel for")                                                                              \
+    for (int nn = 0; nn < n; nn++)                                                                           \
+        for (int xx = 0; xx < hh; xx++)                                                                      \
+            for (int yy = 0; yy < ww; yy++)                                                                  \
+                for (int cc = 0; cc < c; cc++) {                                                             \
+                    T maxval = LOWEST;                                                                       \
+                    int idx_maxval = 0;                                                                      \
+                    for (int ii = 0; ii < kh; ii++) {                                                        \
+                        const int x_x = vstride * xx + vdilation * ii - vpadding;                            \
+                        if (0 <= x_x && x_x < h)                                                             \
+                            for (int jj = 0; jj < kw; jj++) {                                                \
+                                const int x_y = hstride * yy + hdilation * jj - hpadding;                    \
+                                if (0 <= x_y && x_y < w) {                                                   \
+                                    const T val = x[IDX_NHWC(nn, x_x, x_y, cc, h, w, c)];                    \
+                                    if (val > maxval) { maxval = val; idx_maxval = ii * kw + jj; }           \
+                                }                                                                            \
+                            }                                                                                \
+                    }                                                                                        \
+                    y[IDX_NHWC(nn, xx, yy, cc, hh, ww, c)] = maxval;                                         \
+                    idx_max[IDX_NHWC(nn, xx, yy, cc, hh, ww, c)] = idx_maxval;                               \
+                }                                                                                            \
+}                                                                                                            \
+                                                                                                             \
+void oracle_max_pool_2d_bwd_nhwc_##SFX(const T *dy, const int32_t *idx_max, T *dx,                           \
+                                     int n, int h, int w, int c, int kh, int kw,                             \
+                                     int vpadding, int hpadding, int vstride, int hstride,                   \
+                                     int vdilation, int hdilation)                                           \
+{                                                                                                            \
+    const int hh = out_dim(h, vpadding, vdilation, kh, vstride);                                             \
+    const int ww = out_dim(w, hpadding, hdilation, kw, hstride);                                             \
+    _Pragma("omp parallel for")                                                                              \
+    for (int nn = 0; nn < n; nn++)                                                                           \
+        for (int xx = 0; xx < hh; xx++)                                                                      \
+            for (int yy = 0; yy < ww; yy++)                                                                  \
+                for (int cc = 0; cc < c; cc++) {                                                             \
+                    const int idx_maxval = idx_max[IDX_NHWC(nn, xx, yy, cc, hh, ww, c)];                     \
+                    const int ii = idx_maxval / kh, jj = idx_maxval % kw;                                    \
+                    const int x_x = vstride * xx + vdilation * ii - vpadding;                                \
+                    const int x_y = hstride * yy + hdilation * jj - hpadding;                                \
+                    if (0 <= x_x && x_x < h && 0 <= x_y && x_y < w)                                          \
+                        dx[IDX_NHWC(nn, x_x, x_y, cc, h, w, c)] += dy[IDX_NHWC(nn, xx, yy, cc, hh, ww, c)];  \
+                }                                                                                            \
 }
-
-void oracle_max_pool_2d_bwd_nhwc_f32(const float *dy, const int32_t *idx_max, float *dx,
-                                     int n, int h, int w, int c, int kh, int kw,
-                                     int vpadding, int hpadding, int vstride, int hstride,
-                                     int vdilation, int hdilation)
-{
-    const int hh = out_dim(h, vpadding, vdilation, kh, vstride);
-    const int ww = out_dim(w, hpadding, hdilation, kw, hstride);
-    #pragma omp parallel for
-    for (int nn = 0; nn < n; nn++)
-        for (int xx = 0; xx < hh; xx++)
-            for (int yy = 0; yy < ww; yy++)
-                for (int cc = 0; cc < c; cc++) {
-                    const int idx_maxval = idx_max[IDX_NHWC(nn, xx, yy, cc, hh, ww, c)];
-                    const int ii = idx_maxval / kh, jj = idx_maxval % kw;
-                    const int x_x = vstride * xx + vdilation * ii - vpadding;
-                    const int x_y = hstride * yy + hdilation * jj - hpadding;
-                    if (0 <= x_x && x_x < h && 0 <= x_y && x_y < w)
-                        dx[IDX_NHWC(nn, x_x, x_y, cc, h, w, c)] += dy[IDX_NHWC(nn, xx, yy, cc, hh, ww, c)];
-                }
-}
+DEF_MAX_POOL_NHWC(float, f32, -FLT_MAX)
+DEF_MAX_POOL_NHWC(double, f64, -DBL_MAX)
 
 /* ---------------------------------------------------------------------------
  * AveragePool2D forward / backward, both tensor formats.
@@ -397,8 +404,8 @@ void oracle_max_pool_2d_bwd_nhwc_f32(const float *dy, const int32_t *idx_max, fl
  * number (padding is not counted); backward adds dy / items to every such
  * tap, windows visited in ascending (xx, yy) order.
  * ------------------------------------------------------------------------- */
-#define DEF_AVG_POOL(NAME, NHWC)                                                                         \
-void NAME##_fwd_f32(const float *x, float *y, int n, int c, int h, int w, int kh, int kw,               \
+#define DEF_AVG_POOL(NAME, NHWC, T, SFX)                                                                        \
+void NAME##_fwd_##SFX(const T *x, T *y, int n, int c, int h, int w, int kh, int kw,               \
                     int vpadding, int hpadding, int vstride, int hstride, int vdilation, int hdilation) \
 {                                                                                                        \
     const int hh = out_dim(h, vpadding, vdilation, kh, vstride);                                         \
@@ -408,7 +415,7 @@ void NAME##_fwd_f32(const float *x, float *y, int n, int c, int h, int w, int kh
         for (int cc = 0; cc < c; cc++)                                                                   \
             for (int xx = 0; xx < hh; xx++)                                                              \
                 for (int yy = 0; yy < ww; yy++) {                                                        \
-                    float accum = 0;                                                                     \
+                    T accum = 0;                                                                         \
                     int items = 0;                                                                       \
                     for (int ii = 0; ii < kh; ii++) {                                                    \
                         const int x_x = vstride * xx + vdilation * ii - vpadding;                        \
@@ -426,7 +433,7 @@ void NAME##_fwd_f32(const float *x, float *y, int n, int c, int h, int w, int kh
                         accum / items;                                                                   \
                 }                                                                                        \
 }                                                                                                        \
-void NAME##_bwd_f32(const float *dy, float *dx, int n, int c, int h, int w, int kh, int kw,             \
+void NAME##_bwd_##SFX(const T *dy, T *dx, int n, int c, int h, int w, int kh, int kw,             \
                     int vpadding, int hpadding, int vstride, int hstride, int vdilation, int hdilation) \
 {                                                                                                        \
     const int hh = out_dim(h, vpadding, vdilation, kh, vstride);                                         \
@@ -445,7 +452,7 @@ void NAME##_bwd_f32(const float *dy, float *dx, int n, int c, int h, int w, int 
                                 if (0 <= x_y && x_y < w) items = items + 1;                              \
                             }                                                                            \
                     }                                                                                    \
-                    const float avgval =                                                                 \
+                    const T avgval =                                                                     \
                         dy[NHWC ? IDX4(nn, xx, yy, cc, hh, ww, c) : IDX4(nn, cc, xx, yy, c, hh, ww)] / items; \
                     for (int ii = 0; ii < kh; ii++) {                                                    \
                         const int x_x = vstride * xx + vdilation * ii - vpadding;                        \
@@ -459,5 +466,7 @@ void NAME##_bwd_f32(const float *dy, float *dx, int n, int c, int h, int w, int 
                     }                                                                                    \
                 }                                                                                        \
 }
-DEF_AVG_POOL(oracle_average_pool_2d_nchw, 0)
-DEF_AVG_POOL(oracle_average_pool_2d_nhwc, 1)
+DEF_AVG_POOL(oracle_average_pool_2d_nchw, 0, float, f32)
+DEF_AVG_POOL(oracle_average_pool_2d_nhwc, 1, float, f32)
+DEF_AVG_POOL(oracle_average_pool_2d_nchw, 0, double, f64)
+DEF_AVG_POOL(oracle_average_pool_2d_nhwc, 1, double, f64)

@@ -84,6 +84,19 @@ SIGNATURES = {
     "pydtnn_hip_relu_bwd_f64": (_c.c_int, [_vp, _i8p, _vp, _c.c_long, _vp]),
     "pydtnn_hip_bias_grad_f64": (_c.c_int, [_vp, _vp, _c.c_long, _c.c_int, _c.c_long, _vp]),
     "pydtnn_hip_transpose_1023_f64": (_c.c_int, [_vp, _vp, _c.c_int, _c.c_int, _c.c_long, _vp]),
+    "pydtnn_hip_max_pool_2d_fwd_f64": (_c.c_int, [_c.c_int, _vp, _vp, _i32p] + [_c.c_int] * 12 + [_vp]),
+    "pydtnn_hip_max_pool_2d_bwd_f64": (_c.c_int, [_c.c_int, _vp, _i32p, _vp] + [_c.c_int] * 12 + [_vp]),
+    "pydtnn_hip_average_pool_2d_fwd_f64": (_c.c_int, [_c.c_int, _vp, _vp] + [_c.c_int] * 12 + [_vp]),
+    "pydtnn_hip_average_pool_2d_bwd_f64": (_c.c_int, [_c.c_int, _vp, _vp] + [_c.c_int] * 12 + [_vp]),
+    "pydtnn_hip_softmax_fwd_f64": (_c.c_int, [_vp, _vp, _c.c_int, _c.c_int, _vp]),
+    "pydtnn_hip_softmax_bwd_f64": (_c.c_int, [_vp, _vp, _vp, _c.c_int, _c.c_int, _vp]),
+    "pydtnn_hip_categorical_cross_entropy_f64": (_c.c_int, [_vp, _vp, _vp, _vp, _c.c_int, _c.c_int, _c.c_double,
+                                                            _c.c_int, _vp, _c.c_size_t, _vp]),
+    "pydtnn_hip_sgd_momentum_f64": (_c.c_int, [_vp, _vp, _vp, _c.c_long, _c.c_double, _c.c_double, _c.c_double,
+                                               _c.c_int, _vp]),
+    "pydtnn_hip_bn_training_fwd_f64": (_c.c_int, [_vp] * 8 + [_c.c_double, _c.c_double, _c.c_long, _c.c_int, _c.c_long,
+                                                            _vp]),
+    "pydtnn_hip_bn_training_bwd_f64": (_c.c_int, [_vp] * 7 + [_c.c_long, _c.c_int, _c.c_long, _vp]),
 }
 
 # Host-pointer flavour exported by libconvGemm.so with the reference's own names

@@ -214,31 +214,44 @@ def bias_grad(dy, channels, inner):
 
 def average_pool_2d_fwd(x, nhwc, kh, kw, vpadding, hpadding, vstride, hstride, vdilation=1, hdilation=1):
     """pydtnn/cython_modules/average_pool_2d_nchw_cython.pyx:25-52 / average_pool_2d_nhwc_cython.pyx:25-52"""
-    _need_f32(x)
+    fn = lib().pydtnn_hip_average_pool_2d_fwd_f64 if _is_f64(x) else lib().pydtnn_hip_average_pool_2d_fwd
     n, c, h, w = (x.shape[0], x.shape[3], x.shape[1], x.shape[2]) if nhwc else x.shape
     hh, ww = _out_hw(h, w, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
     y = torch.empty((n, hh, ww, c) if nhwc else (n, c, hh, ww), dtype=x.dtype, device=x.device)
-    check(lib().pydtnn_hip_average_pool_2d_fwd(int(nhwc), f32(x), f32(y), n, c, h, w, kh, kw, vpadding, hpadding,
+    check(fn(int(nhwc), ptr(x), ptr(y), n, c, h, w, kh, kw, vpadding, hpadding,
                                                vstride, hstride, vdilation, hdilation, stream_ptr()), "avg_pool_fwd")
     return y
 
 
 def average_pool_2d_bwd(dy, nhwc, n, c, h, w, kh, kw, vpadding, hpadding, vstride, hstride, vdilation=1, hdilation=1):
     """pydtnn/cython_modules/average_pool_2d_nchw_cython.pyx:135-160 / average_pool_2d_nhwc_cython.pyx:135-160"""
-    _need_f32(dy)
+    fn = lib().pydtnn_hip_average_pool_2d_bwd_f64 if _is_f64(dy) else lib().pydtnn_hip_average_pool_2d_bwd
     dx = torch.empty((n, h, w, c) if nhwc else (n, c, h, w), dtype=dy.dtype, device=dy.device)
-    check(lib().pydtnn_hip_average_pool_2d_bwd(int(nhwc), f32(dy), f32(dx), n, c, h, w, kh, kw, vpadding, hpadding,
+    check(fn(int(nhwc), ptr(dy), ptr(dx), n, c, h, w, kh, kw, vpadding, hpadding,
                                                vstride, hstride, vdilation, hdilation, stream_ptr()), "avg_pool_bwd")
+    return dx
+
+
+def _max_pool_bwd_f64(nhwc, dy, idx_max, dx, gate, n, c, h, w, *geom):
+    check(lib().pydtnn_hip_max_pool_2d_bwd_f64(nhwc, ptr(dy), ptr(idx_max), ptr(dx), n, c, h, w, *geom, stream_ptr()),
+          "max_pool_bwd_f64")
+    if gate is not None:   # the ReLU layer below, as a pass of its own
+        _need_gate(gate, dx)
+        check(lib().pydtnn_hip_relu_bwd_f64(ptr(dx), ptr(gate), ptr(dx), dx.numel(), stream_ptr()), "relu_bwd_f64")
     return dx
 
 
 def max_pool_2d_fwd_nchw(x, kh, kw, vpadding, hpadding, vstride, hstride, vdilation=1, hdilation=1):
     """pydtnn/cython_modules/max_pool_2d_nchw_cython.pyx:25-52 -> (y, idx_max int32)"""
-    _need_f32(x)
     n, c, h, w = x.shape
     hh, ww = _out_hw(h, w, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
     y = torch.empty((n, c, hh, ww), dtype=x.dtype, device=x.device)
     idx = torch.empty((n, c, hh, ww), dtype=torch.int32, device=x.device)
+    if _is_f64(x):
+        check(lib().pydtnn_hip_max_pool_2d_fwd_f64(0, ptr(x), ptr(y), ptr(idx), n, c, h, w, kh, kw, vpadding, hpadding,
+                                                   vstride, hstride, vdilation, hdilation, stream_ptr()),
+              "max_pool_fwd_f64")
+        return y, idx
     check(lib().pydtnn_hip_max_pool_2d_fwd_nchw(f32(x), f32(y), ptr(idx), n, c, h, w, kh, kw, vpadding, hpadding,
                                                 vstride, hstride, vdilation, hdilation, stream_ptr()), "max_pool_fwd")
     return y, idx
@@ -248,8 +261,10 @@ def max_pool_2d_bwd_nchw(dy, idx_max, n, c, h, w, kh, kw, vpadding, hpadding, vs
                          vdilation=1, hdilation=1, gate=None):
     """pydtnn/cython_modules/max_pool_2d_nchw_cython.pyx:140-166.  ``gate``: int8 mask of a ReLU layer below
     the pooling layer; dx is stored multiplied by it (that layer's backward, relu_cpu.py:38-40)."""
-    _need_f32(dy)
     dx = torch.empty((n, c, h, w), dtype=dy.dtype, device=dy.device)
+    if _is_f64(dy):
+        return _max_pool_bwd_f64(0, dy, idx_max, dx, gate, n, c, h, w, kh, kw, vpadding, hpadding, vstride, hstride,
+                                 vdilation, hdilation)
     if gate is not None:
         _need_gate(gate, dx)
         check(lib().pydtnn_hip_max_pool_2d_bwd_gated(0, f32(dy), ptr(idx_max), f32(dx), ptr(gate), n, c, h, w, kh, kw,
@@ -264,11 +279,15 @@ def max_pool_2d_bwd_nchw(dy, idx_max, n, c, h, w, kh, kw, vpadding, hpadding, vs
 
 def max_pool_2d_fwd_nhwc(x, kh, kw, vpadding, hpadding, vstride, hstride, vdilation=1, hdilation=1):
     """pydtnn/cython_modules/max_pool_2d_nhwc_cython.pyx:25-52 -> (y, idx_max int32)"""
-    _need_f32(x)
     n, h, w, c = x.shape
     hh, ww = _out_hw(h, w, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
     y = torch.empty((n, hh, ww, c), dtype=x.dtype, device=x.device)
     idx = torch.empty((n, hh, ww, c), dtype=torch.int32, device=x.device)
+    if _is_f64(x):
+        check(lib().pydtnn_hip_max_pool_2d_fwd_f64(1, ptr(x), ptr(y), ptr(idx), n, c, h, w, kh, kw, vpadding, hpadding,
+                                                   vstride, hstride, vdilation, hdilation, stream_ptr()),
+              "max_pool_fwd_f64")
+        return y, idx
     check(lib().pydtnn_hip_max_pool_2d_fwd_nhwc(f32(x), f32(y), ptr(idx), n, h, w, c, kh, kw, vpadding, hpadding,
                                                 vstride, hstride, vdilation, hdilation, stream_ptr()), "max_pool_fwd")
     return y, idx
@@ -277,8 +296,10 @@ def max_pool_2d_fwd_nhwc(x, kh, kw, vpadding, hpadding, vstride, hstride, vdilat
 def max_pool_2d_bwd_nhwc(dy, idx_max, n, h, w, c, kh, kw, vpadding, hpadding, vstride, hstride,
                          vdilation=1, hdilation=1, gate=None):
     """pydtnn/cython_modules/max_pool_2d_nhwc_cython.pyx:140-166; ``gate`` as in the NCHW twin."""
-    _need_f32(dy)
     dx = torch.empty((n, h, w, c), dtype=dy.dtype, device=dy.device)
+    if _is_f64(dy):
+        return _max_pool_bwd_f64(1, dy, idx_max, dx, gate, n, c, h, w, kh, kw, vpadding, hpadding, vstride, hstride,
+                                 vdilation, hdilation)
     if gate is not None:
         _need_gate(gate, dx)
         check(lib().pydtnn_hip_max_pool_2d_bwd_gated(1, f32(dy), ptr(idx_max), f32(dx), ptr(gate), n, c, h, w, kh, kw,
@@ -294,11 +315,16 @@ def max_pool_2d_bwd_nhwc(dy, idx_max, n, h, w, c, kh, kw, vpadding, hpadding, vs
 def bn_training_forward(x, gamma, beta, running_mean, running_var, momentum, eps, channels, inner):
     """pydtnn/backends/cpu/layers/batch_normalization_cpu.py:59-82 on x viewed as (outer, channels, inner).
     Updates running_mean / running_var in place; returns (y, xn, std)."""
-    _need_f32(x, gamma, beta, running_mean, running_var)
+    f64 = _is_f64(x, gamma, beta, running_mean, running_var)
     x = x.contiguous()
     outer = x.numel() // (channels * inner)
     y, xn = torch.empty_like(x), torch.empty_like(x)
     std = torch.empty((channels,), dtype=x.dtype, device=x.device)
+    if f64:
+        check(lib().pydtnn_hip_bn_training_fwd_f64(ptr(x), ptr(y), ptr(xn), ptr(std), ptr(gamma), ptr(beta),
+                                                   ptr(running_mean), ptr(running_var), float(momentum), float(eps),
+                                                   outer, channels, inner, stream_ptr()), "bn_training_fwd_f64")
+        return y, xn, std
     ws, ws_bytes = native.workspace(lib().pydtnn_hip_bn_training_workspace_bytes(channels))
     check(lib().pydtnn_hip_bn_training_fwd(f32(x), f32(y), f32(xn), f32(std), f32(gamma), f32(beta), f32(running_mean),
                                            f32(running_var), float(momentum), float(eps), outer, channels, inner, ws,
@@ -308,12 +334,16 @@ def bn_training_forward(x, gamma, beta, running_mean, running_var, momentum, eps
 
 def bn_training_backward(dy, xn, std, gamma, channels, inner, need_dx=True):
     """batch_normalization_cpu.py:108-129 -> (dgamma, dbeta, dx or None)"""
-    _need_f32(dy, xn, std, gamma)
+    f64 = _is_f64(dy, xn, std, gamma)
     dy = dy.contiguous()
     outer = dy.numel() // (channels * inner)
     dgamma = torch.empty((channels,), dtype=dy.dtype, device=dy.device)
     dbeta = torch.empty_like(dgamma)
     dx = torch.empty_like(dy) if need_dx else None
+    if f64:
+        check(lib().pydtnn_hip_bn_training_bwd_f64(ptr(dy), ptr(xn), ptr(std), ptr(gamma), ptr(dgamma), ptr(dbeta),
+                                                   ptr(dx), outer, channels, inner, stream_ptr()), "bn_training_bwd_f64")
+        return dgamma, dbeta, dx
     ws, ws_bytes = native.workspace(lib().pydtnn_hip_bn_training_workspace_bytes(channels))
     check(lib().pydtnn_hip_bn_training_bwd(f32(dy), f32(xn), f32(std), f32(gamma), f32(dgamma), f32(dbeta), f32(dx),
                                            outer, channels, inner, ws, ws_bytes, stream_ptr()), "bn_training_bwd")
@@ -322,20 +352,27 @@ def bn_training_backward(dy, xn, std, gamma, channels, inner, need_dx=True):
 
 def softmax(x):
     """pydtnn/backends/cpu/activations/softmax_cpu.py:32-35 on a (batch, classes) matrix."""
-    _need_f32(x)
+    f64 = _is_f64(x)
     if x.dim() != 2:
         raise ValueError("softmax expects a (batch, classes) matrix")
     x = x.contiguous()
     y = torch.empty_like(x)
+    if f64:
+        check(lib().pydtnn_hip_softmax_fwd_f64(ptr(x), ptr(y), x.shape[0], x.shape[1], stream_ptr()), "softmax_fwd_f64")
+        return y
     check(lib().pydtnn_hip_softmax_fwd(f32(x), f32(y), x.shape[0], x.shape[1], stream_ptr()), "softmax_fwd")
     return y
 
 
 def softmax_backward(dy, y):
     """pydtnn/backends/cpu/activations/softmax_cpu.py:37-39"""
-    _need_f32(dy, y)
+    f64 = _is_f64(dy, y)
     dy, y = dy.contiguous(), y.contiguous()
     dx = torch.empty_like(y)
+    if f64:
+        check(lib().pydtnn_hip_softmax_bwd_f64(ptr(dy), ptr(y), ptr(dx), y.shape[0], y.shape[1], stream_ptr()),
+              "softmax_bwd_f64")
+        return dx
     check(lib().pydtnn_hip_softmax_bwd(f32(dy), f32(y), f32(dx), y.shape[0], y.shape[1], stream_ptr()),
           "softmax_bwd")
     return dx
@@ -343,10 +380,17 @@ def softmax_backward(dy, y):
 
 def categorical_cross_entropy(y_pred, y_targ, global_batch_size, eps=1e-8):
     """pydtnn/backends/cpu/losses/categorical_cross_entropy_cpu.py:28-35.  Returns (loss as a 0-d tensor, dx)."""
-    _need_f32(y_pred, y_targ)
+    f64 = _is_f64(y_pred, y_targ)
     y_pred, y_targ = y_pred.contiguous(), y_targ.contiguous()
     rows, cols = y_pred.shape
     dx = torch.empty_like(y_targ)
+    if f64:
+        loss = torch.empty(1, dtype=torch.float64, device=y_pred.device)
+        ws, ws_bytes = native.workspace(rows * 8)
+        check(lib().pydtnn_hip_categorical_cross_entropy_f64(ptr(y_pred), ptr(y_targ), ptr(dx), ptr(loss), rows, cols,
+                                                             float(eps), int(global_batch_size), ws, ws_bytes,
+                                                             stream_ptr()), "categorical_cross_entropy_f64")
+        return loss[0], dx
     loss = torch.empty(1, dtype=torch.float32, device=y_pred.device)
     ws, ws_bytes = native.workspace(rows * 4)
     check(lib().pydtnn_hip_categorical_cross_entropy(f32(y_pred), f32(y_targ), f32(dx), f32(loss), rows, cols,
@@ -357,7 +401,10 @@ def categorical_cross_entropy(y_pred, y_targ, global_batch_size, eps=1e-8):
 
 def sgd_momentum(w, dw, velocity, lr, momentum, decay=0.0, nesterov=False):
     """In place SGD step (pydtnn/backends/cpu/optimizers/sgd_cpu.py:28-41)."""
-    _need_f32(w, dw, velocity)
+    if _is_f64(w, dw, velocity):
+        check(lib().pydtnn_hip_sgd_momentum_f64(ptr(w), ptr(dw), ptr(velocity), w.numel(), lr, momentum, decay,
+                                                int(nesterov), stream_ptr()), "sgd_momentum_f64")
+        return
     check(lib().pydtnn_hip_sgd_momentum(f32(w), f32(dw), f32(velocity), w.numel(), lr, momentum, decay,
                                         int(nesterov), stream_ptr()), "sgd_momentum")
 

@@ -474,23 +474,35 @@ POOL_GEOMS = [  # (n, c, h, w, kh, kw, pv, ph, sv, sh, dv, dh)
 ]
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
 @pytest.mark.parametrize("geom", POOL_GEOMS, ids=str)
-def test_maxpool_padded_strided_dilated_against_torch(oracle, geom):
+def test_maxpool_padded_strided_dilated_against_torch(oracle, geom, dtype):
     """torch.nn.functional.max_pool2d pads with -inf, i.e. ignores padding taps like the reference's bound
     tests; distinct random values leave no ties, so values and gradients must agree exactly.  Square windows
-    only go through backward: the reference decodes the stored index with kh where kw belongs."""
+    only go through backward: the reference decodes the stored index with kh where kw belongs.  In float64
+    (pydtnn/cython_modules/max_pool_2d_nchw_cython.pyx:46-49) the values are not representable in float32, so
+    a pool that computed in float32 on the way would not reproduce them; the NHWC pair is checked against the
+    NCHW one in the same dtype."""
     n, c, h, w, kh, kw, pv, ph, sv, sh, dv, dh = geom
     rng = np.random.default_rng(21)
-    x = rng.permutation(n * c * h * w).astype(np.float32).reshape(n, c, h, w) / 7.0
+    x = rng.permutation(n * c * h * w).astype(dtype).reshape(n, c, h, w) / dtype(7.0)
     y, idx = oracle.max_pool_2d_fwd_nchw(x, kh, kw, pv, ph, sv, sh, dv, dh)
+    assert y.dtype == dtype
     xt = torch.from_numpy(x).requires_grad_(True)
     yt = F.max_pool2d(xt, (kh, kw), (sv, sh), (pv, ph), (dv, dh))
     assert np.array_equal(y, yt.detach().numpy())
+    yh, idxh = oracle.max_pool_2d_fwd_nhwc(np.ascontiguousarray(x.transpose(0, 2, 3, 1)), kh, kw, pv, ph, sv, sh, dv, dh)
+    assert yh.dtype == dtype and np.array_equal(yh, y.transpose(0, 2, 3, 1))
+    assert np.array_equal(idxh, idx.transpose(0, 2, 3, 1))
     if kh == kw:
-        dy = rng.standard_normal(y.shape).astype(np.float32)
+        dy = rng.standard_normal(y.shape).astype(dtype)
         yt.backward(torch.from_numpy(dy))
         dx = oracle.max_pool_2d_bwd_nchw(dy, idx, n, c, h, w, kh, kw, pv, ph, sv, sh, dv, dh)
-        np.testing.assert_allclose(dx, xt.grad.numpy(), rtol=1e-6, atol=1e-6)
+        tol = 1e-6 if dtype == np.float32 else 1e-14
+        np.testing.assert_allclose(dx, xt.grad.numpy(), rtol=tol, atol=tol)
+        dxh = oracle.max_pool_2d_bwd_nhwc(np.ascontiguousarray(dy.transpose(0, 2, 3, 1)), idxh, n, h, w, c, kh, kw, pv,
+                                          ph, sv, sh, dv, dh)
+        assert dxh.dtype == dtype and np.array_equal(dxh, dx.transpose(0, 2, 3, 1))
 
 
 @pytest.mark.parametrize("fmt", ["NCHW", "NHWC"])
@@ -511,6 +523,12 @@ def test_average_pool_against_torch(oracle, fmt, geom):
     dx = oracle.average_pool_2d_bwd(to_fmt(dy.astype(np.float32)), fmt, n, c, h, w, kh, kw, pv, ph, sv, sh)
     np.testing.assert_allclose(y, to_fmt(yt.detach().numpy()), rtol=1e-5, atol=1e-6)
     np.testing.assert_allclose(dx, to_fmt(xt.grad.numpy()), rtol=1e-5, atol=1e-6)
+    # the float64 pair (the reference's modules dispatch on the dtype) against the same float64 torch result
+    y64 = oracle.average_pool_2d_fwd(to_fmt(x), fmt, kh, kw, pv, ph, sv, sh)
+    dx64 = oracle.average_pool_2d_bwd(to_fmt(dy), fmt, n, c, h, w, kh, kw, pv, ph, sv, sh)
+    assert y64.dtype == np.float64 and dx64.dtype == np.float64
+    np.testing.assert_allclose(y64, to_fmt(yt.detach().numpy()), rtol=1e-13, atol=1e-14)
+    np.testing.assert_allclose(dx64, to_fmt(xt.grad.numpy()), rtol=1e-13, atol=1e-14)
 
 
 def test_average_pool_closed_forms(oracle):
