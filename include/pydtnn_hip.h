@@ -386,9 +386,16 @@ int pydtnn_hip_bn_training_bwd_f64(const double *dy, const double *xn, const dou
  * PyDTNN's ctypes shim calls (pydtnn/backends/cpu/libs/conv_gemm.py:91-92, :191-205, :234-248,
  * :299-307, :321-328).  ac_pack / bc_pack are accepted and ignored; alloc_pack_buffs hands out two
  * small malloc() blocks because the reference free()s them with libc (:109-115, :332-349).
- * Errors cannot be returned through this ABI (the reference has no error channel): a failure is
- * reported on stderr and aborts the process rather than returning wrong numbers.
+ * The operands are pageable host arrays: a call moves them in groups of whole images through pinned bounce
+ * buffers (worker threads copy, the DMA engines transfer, the kernels of the group between run, all at once).
+ * Errors cannot be returned through this ABI (the reference has no error channel): a failure is reported on
+ * stderr, the call returns, and pydtnn_convgemm_last_status() gives the PYDTNN_HIP_* status of the most recent of
+ * the four compute calls in this process (PYDTNN_HIP_OK after a good one).  Arguments are checked before anything
+ * is copied, so a call rejected as invalid or unsupported leaves its output array untouched; after a run-time
+ * failure (status PYDTNN_HIP_ERR_LAUNCH) the output holds the groups that had already come back.  This status
+ * function has no counterpart in the reference's libconvGemm: a shim that never calls it behaves as before.
  * ---------------------------------------------------------------------------------------- */
+int pydtnn_convgemm_last_status(void);
 int alloc_pack_buffs(float **ac_pack, float **bc_pack);
 void sconvGemmNCHW(char trans, unsigned b, unsigned c, unsigned h, unsigned w, unsigned kn, unsigned kh, unsigned kw,
                    unsigned vpadding, unsigned hpadding, unsigned vstride, unsigned hstride, unsigned vdilation,

@@ -15,6 +15,8 @@ LIB_PATH = os.path.join(LIB_DIR, "libpydtnn_hip.so")
 COMPAT_LIB_PATH = os.path.join(LIB_DIR, "libconvGemm.so")
 
 OP_FWD, OP_DW, OP_DX, OP_DX_I2C, OP_DB = range(5)
+# status codes of include/pydtnn_hip.h
+PYDTNN_HIP_OK, PYDTNN_HIP_ERR_INVALID, PYDTNN_HIP_ERR_WORKSPACE, PYDTNN_HIP_ERR_LAUNCH, PYDTNN_HIP_ERR_UNSUPPORTED = range(5)
 
 _c = ctypes
 _f32p, _i8p, _i32p, _vp = _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p
@@ -100,7 +102,8 @@ SIGNATURES = {
 }
 
 # Host-pointer flavour exported by libconvGemm.so with the reference's own names
-COMPAT_SYMBOLS = ["alloc_pack_buffs", "sconvGemmNCHW", "sconvGemmNHWC", "sconvGemmNCHW_back", "sconvGemmNHWC_back"]
+COMPAT_SYMBOLS = ["alloc_pack_buffs", "sconvGemmNCHW", "sconvGemmNHWC", "sconvGemmNCHW_back", "sconvGemmNHWC_back",
+                  "pydtnn_convgemm_last_status"]
 
 _LIB = None
 

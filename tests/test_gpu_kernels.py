@@ -1019,6 +1019,26 @@ def test_libconvgemm_compat_abi_runs_like_the_reference_shim(oracle):
                       ctypes.c_void_p(b.ctypes.data), none, none, none, none, ctypes.c_bool(True), ac, bc)
     ref = np.maximum(_fwd_ref(oracle, x, w, b, d), 0)
     assert_close(y, ref, what="compat fwd")
+    lib.pydtnn_convgemm_last_status.restype = ctypes.c_int
+    assert lib.pydtnn_convgemm_last_status() == 0
+    # calls the library must refuse return, report through the status function and leave the output alone:
+    # a filter that does not fit the image, a zero stride, a missing BN vector, an image beyond the addressing limit
+    y[:] = 7.0
+    bad_calls = [dict(kh=d.h + 5), dict(vstride=0), dict(bn=(ctypes.c_void_p(b.ctypes.data), none, none, none)),
+                 dict(b=1, c=1, h=1 << 15, w=1 << 15, kn=1, kh=1, kw=1)]
+    for bad in bad_calls:
+        a = dict(b=d.b, c=d.c, h=d.h, w=d.w, kn=d.kn, kh=d.kh, kw=d.kw, vpadding=d.vpadding, hpadding=d.hpadding,
+                 vstride=d.vstride, hstride=d.hstride, vdilation=d.vdilation, hdilation=d.hdilation)
+        bn_args = bad.pop("bn", (none, none, none, none))
+        a.update(bad)
+        announce("compat abi, refused call", bad or "bn vectors")
+        lib.sconvGemmNCHW(ctypes.c_char(b'N'), *[u(a[k]) for k in ("b", "c", "h", "w", "kn", "kh", "kw", "vpadding",
+                                                                    "hpadding", "vstride", "hstride", "vdilation",
+                                                                    "hdilation")],
+                          ctypes.c_void_p(w.ctypes.data), ctypes.c_void_p(x.ctypes.data), ctypes.c_void_p(y.ctypes.data),
+                          ctypes.c_void_p(b.ctypes.data), *bn_args, ctypes.c_bool(True), ac, bc)
+        assert lib.pydtnn_convgemm_last_status() in (native.PYDTNN_HIP_ERR_INVALID, native.PYDTNN_HIP_ERR_UNSUPPORTED)
+        assert np.all(y == 7.0), "a refused call must not touch its output"
     dw = np.empty(w.shape, np.float32)
     lib.sconvGemmNCHW(ctypes.c_char(b'Y'), u(d.b), u(d.c), u(d.h), u(d.w), u(d.kn), u(d.kh), u(d.kw),
                       u(d.vpadding), u(d.hpadding), u(d.vstride), u(d.hstride), u(d.vdilation), u(d.hdilation),
@@ -1034,6 +1054,30 @@ def test_libconvgemm_compat_abi_runs_like_the_reference_shim(oracle):
                            ctypes.c_void_p(w.ctypes.data), ctypes.c_void_p(dy.ctypes.data),
                            ctypes.c_void_p(dx.ctypes.data), ac, bc)
     assert_close(dx, dx_ref, what="compat dx")
+    assert lib.pydtnn_convgemm_last_status() == 0       # a good call clears the status of the refused ones
+    # a batch that travels as several groups of images, the last one smaller (16 MiB of the larger tensor per group)
+    d3 = D(11, 32, 160, 160, 64, 3, 3, 1, 1, 1, 1, 1, 1)
+    announce("compat abi, several groups", d3)
+    x3, w3, b3, dy3 = case(d3)
+    y3 = np.full((d3.b, d3.kn, d3.ho, d3.wo), np.nan, np.float32)
+    g3 = [u(v) for v in (d3.b, d3.c, d3.h, d3.w, d3.kn, d3.kh, d3.kw)]
+    lib.sconvGemmNCHW(ctypes.c_char(b'N'), *g3, u(1), u(1), u(1), u(1), u(1), u(1), ctypes.c_void_p(w3.ctypes.data),
+                      ctypes.c_void_p(x3.ctypes.data), ctypes.c_void_p(y3.ctypes.data), ctypes.c_void_p(b3.ctypes.data),
+                      none, none, none, none, ctypes.c_bool(False), ac, bc)
+    assert lib.pydtnn_convgemm_last_status() == 0
+    assert_close(y3, _fwd_ref(oracle, x3, w3, b3, d3), what="compat fwd in groups")
+    dx3 = np.full(x3.shape, np.nan, np.float32)
+    lib.sconvGemmNCHW_back(*g3, u(1), u(1), u(1), u(1), u(1), u(1), ctypes.c_void_p(w3.ctypes.data),
+                           ctypes.c_void_p(dy3.ctypes.data), ctypes.c_void_p(dx3.ctypes.data), ac, bc)
+    dw3 = np.full(w3.shape, np.nan, np.float32)
+    lib.sconvGemmNCHW(ctypes.c_char(b'Y'), *g3, u(1), u(1), u(1), u(1), u(1), u(1), ctypes.c_void_p(dy3.ctypes.data),
+                      ctypes.c_void_p(x3.ctypes.data), ctypes.c_void_p(dw3.ctypes.data), none, none, none, none, none,
+                      ctypes.c_bool(False), ac, bc)
+    p3 = oracle.ConvParams(*d3.geom())
+    _, cols3 = oracle.conv2d_forward_nchw_i2c(x3, w3, None, p3)
+    dw_ref3, _, dx_ref3 = oracle.conv2d_backward_nchw_i2c(dy3, cols3, w3, x3.shape, p3)
+    assert_close(dx3, dx_ref3, what="compat dx in groups")
+    assert_close(dw3, dw_ref3, what="compat dw, inputs streamed")
     # the NHWC entry points and the batch-normalisation arguments (pydtnn/backends/cpu/libs/conv_gemm.py:234-248,
     # :321-328), on a larger and then a smaller problem so that the library's cached device buffers are reused
     # at a different size
