@@ -230,23 +230,60 @@ def cpu_baseline_vgg16(sample_images=16, budget_s=14.0):
 
 
 def run_cfg1(torch, pd, timed_steps, steps, warmup):
+    """The Conv2D layer's forward in EVALUATE_MODE: the layer prepares its call once (geometry, filter and bias bound
+    in the library's plan) and, with Model(enable_memory_cache=True), keeps its output tensor between steps, as the
+    reference's GPU layers do.  Beside it: the same convolution through the ConvGemm shim with every argument passed
+    and a fresh output per call, and the kernel alone (HIP events around 200 launches in a row)."""
+    import time
     from pydtnn_amd.conv_gemm import ConvGemm
     cg = ConvGemm()
     x, w, b = make_cfg1()
     xd, wd, bd = (torch.from_numpy(a).cuda() for a in (x, w, b))
+    model = pd.Model(tensor_format="NHWC", batch_size=64, enable_memory_cache=True)
+    model.mode = pd.EVALUATE_MODE
+    conv = pd.Conv2D(nfilters=32, filter_shape=(3, 3), padding=1)
+    conv.set_model(model)
+    conv.initialize(prev_shape=(28, 28, 1))
+    conv.weights, conv.biases = wd, bd
+    assert conv.forward.__name__ == "_forward_nhwc_cg"
+    forward = conv.forward
 
     def step(timers):
-        cg.conv_gemm_nhwc(wd, xd, biases_vector=bd, vpadding=1, hpadding=1)
+        forward(xd)
 
     ms, _ = timed_steps(torch, step, steps, warmup)
+
+    def shim_step(timers):
+        cg.conv_gemm_nhwc(wd, xd, biases_vector=bd, vpadding=1, hpadding=1)
+
+    shim_ms, _ = timed_steps(torch, shim_step, steps, warmup)
+    assert torch.equal(forward(xd), cg.conv_gemm_nhwc(wd, xd, biases_vector=bd, vpadding=1, hpadding=1))
+    # the kernel alone: launches back to back between two events, so that the queue never runs dry
+    reps = 200
+    for _ in range(20):
+        forward(xd)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(reps):
+        forward(xd)
+    host_us = (time.perf_counter() - t0) * 1e6 / reps     # what the launching thread spends per call
+    e1.record()
+    torch.cuda.synchronize()
+    device_us = e0.elapsed_time(e1) * 1e3 / reps
     flop = 2.0 * 32 * 9 * 64 * 28 * 28
     nbytes = x.nbytes + w.nbytes + 64 * 28 * 28 * 32 * 4
     gbs = nbytes / (ms * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": "conv_stream_nchw_kernel<1, 1, 0, 12, true, true>",
                 "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
                 "traffic": None}
-    workload = "cfg1: Conv2D forward, fp32 NHWC, N=64, 28x28x1 -> 32, 3x3, stride 1, pad 1 (launch-latency bound)"
-    return ms, flop / (ms * 1e-3) / 1e9, "GFLOP/s", workload, roofline, {"bytes": nbytes, "gbs": round(gbs, 1)}
+    workload = ("cfg1: Conv2D layer forward (EVALUATE_MODE, call prepared at initialisation, output tensor kept: "
+                "Model(enable_memory_cache=True)), fp32 NHWC, N=64, 28x28x1 -> 32, 3x3, stride 1, pad 1 "
+                "(launch-latency bound)")
+    extra = {"bytes": nbytes, "gbs": round(gbs, 1), "shim_ms": round(shim_ms, 4),
+             "host_us_per_call": round(host_us, 2), "device_us_per_call_back_to_back": round(device_us, 2)}
+    return ms, flop / (ms * 1e-3) / 1e9, "GFLOP/s", workload, roofline, extra
 
 
 def run_cfg3(torch, pd, timed_steps, steps, warmup):
@@ -351,6 +388,10 @@ def other_configs_extra(torch, pd, timed_steps, cpu=True, steps=50, warmup=5):
         out[f"{name}_ms"] = round(ms, 4)
         out[f"{name}_gflops"] = round(value, 1)
         out[f"{name}_roofline"] = {k: roofline[k] for k in ("bound", "achieved", "peak", "unit", "frac")}
+        if name == "cfg1":
+            out["cfg1_shim_ms"] = extra["shim_ms"]
+            out["cfg1_host_us_per_call"] = extra["host_us_per_call"]
+            out["cfg1_device_us_per_call_back_to_back"] = extra["device_us_per_call_back_to_back"]
         if name == "cfg4":
             out["cfg4_unfused_ms"] = extra["unfused_ms"]
             out["cfg4_gbs_of_min_traffic"] = extra["block_gbs_vs_8TBs"]

@@ -251,6 +251,25 @@ int pydtnn_hip_max_pool_2d_bwd_gated(int nhwc, const float *dy, const int32_t *i
                                      int b, int c, int h, int w, int kh, int kw, int vpadding, int hpadding,
                                      int vstride, int hstride, int vdilation, int hdilation, void *stream);
 
+/* A forward convolution with everything but the activations bound once: a layer that calls with the same
+ * geometry, filter and per-channel vectors at every step (an inference loop) builds the plan when it is
+ * initialised, as the reference's layers build their ConvGemm object and its kernel arguments in initialize()
+ * (pydtnn/backends/cpu/layers/conv_2d_cpu.py:89-143; the GPU layers also keep their output tensor,
+ * pydtnn/backends/gpu/layers/conv_2d_gpu.py:89-96), and then passes four pointers per call.
+ * pydtnn_hip_conv_plan_forward(plan, x, y, ...) computes exactly what pydtnn_hip_sconvGemmNCHW / NHWC
+ * (nhwc = 0 / 1; b, c, h, w name the input's extents in either format) computes with trans = 'N' and the plan's
+ * arguments; the plan keeps the pointers it was given, not copies, so the filter and the vectors may change in
+ * place but must stay where they are.  Creating and destroying a plan touches host memory only. */
+typedef struct pydtnn_hip_conv_plan pydtnn_hip_conv_plan;
+int pydtnn_hip_conv_plan_create(pydtnn_hip_conv_plan **plan, int nhwc, int b, int c, int h, int w, int kn, int kh,
+                                int kw, int vpadding, int hpadding, int vstride, int hstride, int vdilation,
+                                int hdilation, const float *weights, const float *bias_vector,
+                                const float *bn_running_mean, const float *bn_inv_std, const float *bn_gamma,
+                                const float *bn_beta, bool relu);
+int pydtnn_hip_conv_plan_forward(const pydtnn_hip_conv_plan *plan, const float *x, float *y, void *workspace,
+                                 size_t workspace_bytes, void *stream);
+void pydtnn_hip_conv_plan_destroy(pydtnn_hip_conv_plan *plan);
+
 /* The sum of an addition block done by the store of the convolution that ends one of its two paths
  * (inference).  The forward of pydtnn_hip_sconvGemmNCHW / NHWC (nhwc = 0 / 1; b, c, h, w name the input's
  * batch, channels, height, width in either format) followed by

@@ -10,6 +10,8 @@ import torch
 from . import native
 from .native import check, f32, lib, ptr, stream_ptr
 
+import ctypes
+
 is_conv_gemm_available = True  # pydtnn/backends/cpu/libs/conv_gemm.py:32-36: probe result of load_library
 
 
@@ -206,3 +208,79 @@ class ConvGemm:
             b, h, w, c, kn, kh, kw, vstride, hstride, vpadding, hpadding, vdilation, hdilation,
             f32(weights), f32(dy), f32(dx), ws, ws_bytes, stream_ptr()), "sconvGemmNHWC_back")
         return dx
+
+
+class PreparedForward:
+    """A forward convolution whose geometry, filter and per-channel vectors are bound once (the library's
+    ``pydtnn_hip_conv_plan``): what a layer's ``initialize`` prepares so that each inference step passes only the
+    activations.  The reference's layers fix the same things in ``initialize``
+    (pydtnn/backends/cpu/layers/conv_2d_cpu.py:89-143) and its GPU layers also keep their output tensor between
+    steps (pydtnn/backends/gpu/layers/conv_2d_gpu.py:89-96): with ``keep_output`` every call returns the same
+    tensor, overwritten; without it a fresh one.
+
+    The tensors are referenced, not copied: they may be updated in place; ``binds(...)`` tells whether a layer's
+    current tensors are still the ones bound here."""
+
+    def __init__(self, nhwc, x_shape, weights, geom8, biases_vector=None, bn=None, relu=False, keep_output=False):
+        if weights.dtype != torch.float32:
+            raise ValueError("Type {} not supported by this version of libconvGemm!".format(weights.dtype))
+        kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation = geom8
+        if nhwc:
+            b, h, w, c = x_shape
+            ck, kh_, kw_, kn = weights.shape
+        else:
+            b, c, h, w = x_shape
+            kn, ck, kh_, kw_ = weights.shape
+        assert ck == c, "Number of channels in weights and x should be the same!"
+        assert (kh_, kw_) == (kh, kw)
+        ho = (h + 2 * vpadding - vdilation * (kh - 1) - 1) // vstride + 1
+        wo = (w + 2 * hpadding - hdilation * (kw - 1) - 1) // hstride + 1
+        self.nhwc = int(bool(nhwc))
+        self.x_shape = tuple(x_shape)
+        self.out_shape = (b, ho, wo, kn) if nhwc else (b, kn, ho, wo)
+        self.geom13 = (b, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation)
+        self.bound = (weights, biases_vector) + (tuple(bn) if bn is not None else (None,) * 4)
+        self.relu = bool(relu)
+        self.device = weights.device
+        self.keep_output = keep_output
+        self._y = None
+        self._ws = {}      # raw stream handle -> (pointer, bytes, key and tensor of the stream's scratch buffer)
+        self._run = lib().pydtnn_hip_conv_plan_forward
+        self._plan = ctypes.c_void_p()
+        check(lib().pydtnn_hip_conv_plan_create(ctypes.byref(self._plan), self.nhwc, *self.geom13,
+                                                *[f32(t) for t in self.bound], self.relu), "conv_plan_create")
+
+    def binds(self, weights, biases_vector, bn, relu):
+        t = self.bound
+        return t[0] is weights and t[1] is biases_vector and self.relu == bool(relu) and \
+            ((bn is None and t[2] is None) or
+             (bn is not None and t[2] is bn[0] and t[3] is bn[1] and t[4] is bn[2] and t[5] is bn[3]))
+
+    def __call__(self, x):
+        if x.shape != self.x_shape or x.dtype != torch.float32 or not x.is_contiguous() or x.device != self.device:
+            raise ValueError(f"expected a contiguous float32 tensor of shape {self.x_shape} on {self.device}")
+        stream = torch._C._cuda_getCurrentRawStream(self.device.index)
+        ws = self._ws.get(stream)
+        if ws is None or native.workspace_buffer(ws[2]) is not ws[3]:
+            # first call on this stream, or the stream's scratch buffer has been replaced by a larger one
+            ptr_, size = native.conv_workspace(native.OP_FWD, self.nhwc, self.geom13, stream)
+            key = (self.device.index, stream)
+            ws = self._ws[stream] = (ptr_, size, key, native.workspace_buffer(key))
+        if self.keep_output:
+            y = self._y
+            if y is None:
+                y = self._y = torch.empty(self.out_shape, dtype=torch.float32, device=self.device)
+        else:
+            y = torch.empty(self.out_shape, dtype=torch.float32, device=self.device)
+        rc = self._run(self._plan, x.data_ptr(), y.data_ptr(), ws[0], ws[1], stream)
+        if rc:
+            check(rc, "conv_plan_forward")
+        return y
+
+    def __del__(self):
+        plan, self._plan = getattr(self, "_plan", None), None
+        if plan:
+            try:
+                lib().pydtnn_hip_conv_plan_destroy(plan)
+            except Exception:     # interpreter shutdown
+                pass

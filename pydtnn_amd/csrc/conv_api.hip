@@ -3,6 +3,7 @@
 #include "conv_internal.h"
 #include "../../include/pydtnn_hip_test.h"
 #include <mutex>
+#include <new>
 
 namespace {
 
@@ -407,6 +408,52 @@ int pydtnn_hip_sconvGemmNHWC_back(unsigned b, unsigned h, unsigned w, unsigned c
 {
     return conv_dx_batched(1, GEOM_ARGS, weights, dy, dx, (float*)workspace, workspace_bytes, as_stream(stream));
 }
+
+// ---------------------------------------------------------------- a forward call with its arguments bound
+struct pydtnn_hip_conv_plan {
+    int nhwc;
+    long geom[13];
+    const float *weights, *bias, *mean, *inv_std, *gamma, *beta;
+    bool relu;
+};
+
+int pydtnn_hip_conv_plan_create(pydtnn_hip_conv_plan** plan, int nhwc, int b, int c, int h, int w, int kn, int kh,
+                                int kw, int vpadding, int hpadding, int vstride, int hstride, int vdilation,
+                                int hdilation, const float* weights, const float* bias_vector,
+                                const float* bn_running_mean, const float* bn_inv_std, const float* bn_gamma,
+                                const float* bn_beta, bool relu)
+{
+    if (!plan) return PYDTNN_HIP_ERR_INVALID;
+    *plan = nullptr;
+    if (!weights || !bn_args_consistent(bn_running_mean, bn_inv_std, bn_gamma, bn_beta)) return PYDTNN_HIP_ERR_INVALID;
+    ImageGroups ig;
+    int rc = plan_image_groups(&ig, GEOM_ARGS);
+    if (rc != PYDTNN_HIP_OK) return rc;
+    ConvGeom g;   // refuses here what the call would refuse: extents the index arithmetic does not cover
+    rc = geom_from_args(&g, ig.images, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation);
+    if (rc != PYDTNN_HIP_OK) return rc;
+    pydtnn_hip_conv_plan* p = new (std::nothrow) pydtnn_hip_conv_plan;
+    if (!p) return PYDTNN_HIP_ERR_INVALID;
+    p->nhwc = nhwc ? 1 : 0;
+    const long geom[13] = {GEOM_ARGS};
+    for (int i = 0; i < 13; ++i) p->geom[i] = geom[i];
+    p->weights = weights; p->bias = bias_vector; p->mean = bn_running_mean; p->inv_std = bn_inv_std;
+    p->gamma = bn_gamma; p->beta = bn_beta; p->relu = relu;
+    *plan = p;
+    return PYDTNN_HIP_OK;
+}
+
+int pydtnn_hip_conv_plan_forward(const pydtnn_hip_conv_plan* plan, const float* x, float* y, void* workspace,
+                                 size_t workspace_bytes, void* stream)
+{
+    if (!plan) return PYDTNN_HIP_ERR_INVALID;
+    const long* q = plan->geom;
+    return sconv_gemm_batched(plan->nhwc, 'N', q[0], q[1], q[2], q[3], q[4], q[5], q[6], q[7], q[8], q[9], q[10], q[11],
+                              q[12], plan->weights, x, y, plan->bias, plan->mean, plan->inv_std, plan->gamma, plan->beta,
+                              plan->relu, workspace, workspace_bytes, as_stream(stream));
+}
+
+void pydtnn_hip_conv_plan_destroy(pydtnn_hip_conv_plan* plan) { delete plan; }
 
 // ---------------------------------------------------------------- explicit (i2c) GEMM steps
 int pydtnn_hip_conv_i2c_forward(int nhwc, int b, int c, int h, int w, int kn, int kh, int kw, int vpadding,

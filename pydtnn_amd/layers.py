@@ -16,7 +16,7 @@ import torch
 from . import ops
 from .best_of import BestOf
 from . import tracers as ev
-from .conv_gemm import ConvGemm
+from .conv_gemm import ConvGemm, PreparedForward
 from .utils import PYDTNN_TENSOR_FORMAT_NCHW, decode_tensor, encode_tensor
 
 EVALUATE_MODE, TRAIN_MODE, UNSPECIFIED_MODE = (0, 1, 2)  # pydtnn/model.py:56
@@ -281,6 +281,7 @@ class Conv2D(Layer):
         self.cg = None
         self.x_cols = self.x_rows = self.cg_x = None
         self.dw = self.db = None
+        self._prepared = None
 
     def initialize(self, prev_shape, need_dx=True):
         super().initialize(prev_shape, need_dx)
@@ -440,6 +441,19 @@ class Conv2D(Layer):
             self._end()
             return dx
 
+    def _evaluate_forward(self, x, nhwc, bn=None, relu=False):
+        """EVALUATE_MODE forward through a call prepared once per (input shape, bound tensors): the geometry, the
+        filter and the per-channel vectors are fixed when the layer is initialised, so a step passes only x
+        (conv_2d_cpu.py:89-143 fixes them in ``initialize`` too).  With ``Model(enable_memory_cache=True)`` the
+        layer also keeps its output tensor between steps, as the reference's GPU layers do
+        (pydtnn/backends/gpu/layers/conv_2d_gpu.py:89-96): each call then returns the same tensor, overwritten."""
+        biases_vector = self.biases if self.use_bias else None
+        p = self._prepared
+        if p is None or p.x_shape != x.shape or not p.binds(self.weights, biases_vector, bn, relu):
+            p = self._prepared = PreparedForward(nhwc, x.shape, self.weights, self._geom(), biases_vector, bn, relu,
+                                                 keep_output=bool(self.model.enable_memory_cache))
+        return p(x)
+
     # ---------------------------------------------------------------- cg, NHWC (conv_2d_cpu.py:211-227, :399-427)
     def _folded_forward(self, conv_gemm, x, out_shape, biases_vector):
         """TRAIN_MODE forward that also does the Relu layer above: y = relu(conv(x) + b) and that layer's mask."""
@@ -458,6 +472,8 @@ class Conv2D(Layer):
         if self._folds_relu_above():
             y = self._folded_forward(self.cg.conv_gemm_nhwc, x, (x.shape[0], self.ho, self.wo, self.co),
                                      biases_vector)
+        elif self.model.mode == EVALUATE_MODE:
+            y = self._evaluate_forward(x, True)
         else:
             y = self.cg.conv_gemm_nhwc(self.weights, x, biases_vector=biases_vector, **self._cg_kwargs())
         self._end()
@@ -496,6 +512,8 @@ class Conv2D(Layer):
         if self._folds_relu_above():
             y = self._folded_forward(self.cg.conv_gemm_nchw, x, (x.shape[0], self.co, self.ho, self.wo),
                                      biases_vector)
+        elif self.model.mode == EVALUATE_MODE:
+            y = self._evaluate_forward(x, False)
         else:
             y = self.cg.conv_gemm_nchw(self.weights, x, biases=None, biases_vector=biases_vector,
                                        **self._cg_kwargs())
@@ -809,15 +827,27 @@ class _FusedConv(Conv2D, _FromParents):
                       bn_beta=self.beta)
         return kw
 
+    def _bound_bn(self):
+        if not self._with_bn:
+            return None
+        if self.updated_running_var:
+            self.updated_running_var = False
+            self.inv_std = 1.0 / torch.sqrt(self.running_var + self.epsilon)
+        return (self.running_mean, self.inv_std, self.gamma, self.beta)
+
     def _forward_nchw_cg(self, x, residual=None, relu_after_residual=False):
         if self.model.mode == TRAIN_MODE:
             raise RuntimeError("Fused layers cannot be used in training mode!")
+        if residual is None and self.model.mode == EVALUATE_MODE:
+            return self._evaluate_forward(x, False, self._bound_bn(), self._with_relu)
         return self.cg.conv_gemm_nchw(self.weights, x, biases=None, residual=residual,
                                       relu_after_residual=relu_after_residual, **self._epilogue_kwargs())
 
     def _forward_nhwc_cg(self, x, residual=None, relu_after_residual=False):
         if self.model.mode == TRAIN_MODE:
             raise RuntimeError("Fused layers cannot be used in training mode!")
+        if residual is None and self.model.mode == EVALUATE_MODE:
+            return self._evaluate_forward(x, True, self._bound_bn(), self._with_relu)
         return self.cg.conv_gemm_nhwc(self.weights, x, biases=None, residual=residual,
                                       relu_after_residual=relu_after_residual, **self._epilogue_kwargs())
 

@@ -43,6 +43,10 @@ SIGNATURES = {
     "pydtnn_hip_sconvGemmNHWC": (_c.c_int, [_c.c_char] + _geom13_u + [_f32p] * 8 + [_c.c_bool, _vp, _c.c_size_t, _vp]),
     "pydtnn_hip_sconvGemmNCHW_back": (_c.c_int, _geom13_u + [_f32p] * 3 + [_vp, _c.c_size_t, _vp]),
     "pydtnn_hip_sconvGemmNHWC_back": (_c.c_int, _geom13_u + [_f32p] * 3 + [_vp, _c.c_size_t, _vp]),
+    "pydtnn_hip_conv_plan_create": (_c.c_int, [_c.POINTER(_c.c_void_p), _c.c_int] + _geom13_i + [_f32p] * 6 + [_c.c_bool]),
+    "pydtnn_hip_conv_plan_forward": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_size_t,
+                                                _c.c_void_p]),
+    "pydtnn_hip_conv_plan_destroy": (None, [_c.c_void_p]),
     "pydtnn_hip_sconvGemm_relu_mask": (_c.c_int, [_c.c_int] + _geom13_u + [_f32p] * 4 + [_i8p, _vp, _c.c_size_t, _vp]),
     "pydtnn_hip_sconvGemm_residual": (_c.c_int, [_c.c_int] + _geom13_u + [_f32p] * 8 + [_c.c_bool, _f32p, _c.c_bool, _vp,
                                                  _c.c_size_t, _vp]),
@@ -167,12 +171,14 @@ def f32(t, name="tensor"):
 _WORKSPACE = {}
 
 
-def workspace(nbytes):
-    """Returns (void* or None, size) for a scratch buffer of at least ``nbytes`` bytes."""
+def workspace(nbytes, dev=None, raw_stream=None):
+    """Returns (void* or None, size) for a scratch buffer of at least ``nbytes`` bytes on the current device and
+    stream (or the given ones: a device index and a raw stream handle)."""
     if nbytes == 0:
         return None, 0
-    dev = torch.cuda.current_device()
-    key = (dev, torch.cuda.current_stream().cuda_stream)
+    if dev is None:
+        dev = torch.cuda.current_device()
+    key = (dev, torch.cuda.current_stream().cuda_stream if raw_stream is None else raw_stream)
     buf = _WORKSPACE.get(key)
     if buf is None or buf.numel() < nbytes:
         if buf is not None:
@@ -183,10 +189,15 @@ def workspace(nbytes):
     return ctypes.c_void_p(buf.data_ptr()), buf.numel()
 
 
+def workspace_buffer(key):
+    """The tensor that currently backs the scratch buffer of ``key`` = (device index, raw stream handle), or None."""
+    return _WORKSPACE.get(key)
+
+
 _WORKSPACE_BYTES = {}
 
 
-def conv_workspace(op, nhwc, geom13):
+def conv_workspace(op, nhwc, geom13, raw_stream=None):
     """Scratch buffer for one convolution call; the size query is remembered per (device, operation, geometry),
     since it depends on nothing else and a layer asks with the same geometry at every step."""
     key = (torch.cuda.current_device(), op, int(nhwc), tuple(geom13))
@@ -195,4 +206,4 @@ def conv_workspace(op, nhwc, geom13):
         nbytes = lib().pydtnn_hip_conv_workspace_bytes(op, int(nhwc), *geom13)
         if len(_WORKSPACE_BYTES) < 4096:
             _WORKSPACE_BYTES[key] = nbytes
-    return workspace(nbytes)
+    return workspace(nbytes, raw_stream=raw_stream)

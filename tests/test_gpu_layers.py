@@ -679,3 +679,76 @@ def test_tracers_see_layers_and_operations_of_a_training_step(pd, tmp_path):
     model.set_tracer(t.RoctxTracer(True))
     model.train_batch(x, y, pd.CategoricalCrossEntropy(), pd.SGD(0.01, 0.9))
     assert not model.tracer._open
+
+
+# ------------------------------------------------------------------ the call a layer prepares for inference
+@pytest.mark.parametrize("fmt", ["NCHW", "NHWC"])
+@pytest.mark.parametrize("d", [D(64, 1, 28, 28, 32, 3, 3, 1, 1, 1, 1), D(4, 16, 20, 20, 40, 3, 3, 1, 1, 1, 1),
+                               D(3, 8, 17, 17, 12, 3, 3, 1, 1, 2, 2), D(16, 64, 56, 56, 64, 1, 1, 0, 0, 1, 1)], ids=repr)
+def test_evaluate_mode_forward_uses_a_prepared_call_with_the_same_bits(pd, oracle, fmt, d):
+    """In EVALUATE_MODE a cg convolution goes through a call prepared once (geometry, filter, bias, BN vectors bound in
+    the library's plan).  It must give the bits of the ConvGemm shim's call with all arguments, agree with the
+    oracle, notice tensors that were replaced or a new batch size, follow in-place updates, and keep its output
+    tensor between steps only under Model(enable_memory_cache=True)
+    (pydtnn/backends/gpu/layers/conv_2d_gpu.py:89-96 keeps it always)."""
+    announce("prepared forward", fmt, d)
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal((d.b, d.c, d.h, d.w)).astype(np.float32)
+    w = (rng.standard_normal((d.kn, d.c, d.kh, d.kw)) * 0.2).astype(np.float32)
+    b = rng.standard_normal(d.kn).astype(np.float32)
+    p = oracle.ConvParams(*d.geom())
+    if fmt == "NCHW":
+        xs, ws = dev(x), dev(w)
+        ref = lambda w_, b_: oracle.conv2d_forward_nchw_i2c(x, w_, b_, p)[0]
+    else:
+        xs, ws = dev(nhwc(x)), dev(np.ascontiguousarray(w.transpose(1, 2, 3, 0)))
+        ref = lambda w_, b_: nhwc(oracle.conv2d_forward_nchw_i2c(x, w_, b_, p)[0])
+    for keep in (False, True):
+        model = pd.Model(tensor_format=fmt, batch_size=d.b, enable_memory_cache=keep)
+        model.mode = pd.EVALUATE_MODE
+        conv = pd.Conv2D(nfilters=d.kn, filter_shape=(d.kh, d.kw), padding=(d.vpadding, d.hpadding),
+                         stride=(d.vstride, d.hstride), dilation=(d.vdilation, d.hdilation))
+        conv.set_model(model)
+        conv.initialize(prev_shape=(d.c, d.h, d.w) if fmt == "NCHW" else (d.h, d.w, d.c))
+        conv.weights, conv.biases = ws.clone(), dev(b)
+        shim = conv.cg.conv_gemm_nchw if fmt == "NCHW" else conv.cg.conv_gemm_nhwc
+        y1 = conv.forward(xs)
+        plan = conv._prepared
+        assert plan is not None
+        assert torch.equal(y1, shim(conv.weights, xs, biases_vector=conv.biases, **conv._cg_kwargs()))
+        assert_close(host(y1), ref(w, b), what="prepared forward")
+        y2 = conv.forward(xs)
+        assert conv._prepared is plan and (y2 is y1) == keep and torch.equal(y2, y1)
+        # an update in place is seen by the same plan ...
+        conv.weights.mul_(0.5)
+        assert_close(host(conv.forward(xs)), ref(w * np.float32(0.5), b), what="after an in-place update")
+        assert conv._prepared is plan
+        # ... replaced tensors and another batch size make a new one
+        conv.biases = dev(b + 1)
+        assert_close(host(conv.forward(xs)), ref(w * np.float32(0.5), b + 1), what="after replacing the bias")
+        assert conv._prepared is not plan
+        half = conv.forward(xs[: max(1, d.b // 2)].contiguous())
+        assert half.shape[0] == max(1, d.b // 2)
+        # (another batch size may take another launch form: same values, not necessarily the same bits)
+        assert_close(host(half), host(conv.forward(xs)[: max(1, d.b // 2)]), what="half the batch")
+        with pytest.raises(ValueError):
+            conv._prepared(xs.double())
+    # the fused inference layers bind their BN vectors and the ReLU as well
+    model = pd.Model(tensor_format=fmt, batch_size=d.b, enable_fused_conv_bn_relu=True)
+    model.add(pd.Input(shape=(d.h, d.w, d.c)))
+    model.add(pd.Conv2D(nfilters=d.kn, filter_shape=(d.kh, d.kw), padding=(d.vpadding, d.hpadding),
+                        stride=(d.vstride, d.hstride), dilation=(d.vdilation, d.hdilation)))
+    model.add(pd.BatchNormalization())
+    model.add(pd.Relu())
+    conv, bn = model.layers[1], model.layers[2]
+    conv.weights, conv.biases = ws.clone(), dev(b)
+    stats = [rng.uniform(0.5, 1.5, d.kn).astype(np.float32) for _ in range(4)]
+    bn.running_mean, bn.running_var, bn.gamma, bn.beta = (dev(v) for v in stats)
+    bn.updated_running_var = True
+    y = model.evaluate_dataset_batch(xs)
+    fused = model.layers[1]
+    assert type(fused).__name__ == "Conv2DBatchNormalizationRelu" and fused._prepared is not None
+    inv_std = (1.0 / np.sqrt(stats[1] + np.float32(bn.epsilon))).astype(np.float32)
+    plain = oracle.conv2d_forward_nchw_i2c(x, w, b, p)[0]
+    want = oracle.fused_epilogue(plain, "NCHW", bn=[stats[0], inv_std, stats[2], stats[3]], relu_flag=True)
+    assert_close(host(y), want if fmt == "NCHW" else nhwc(want), what="fused layer through its prepared call")
