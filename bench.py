@@ -210,14 +210,17 @@ def run_cfg2(torch, pd, args):
     # the explicit route on the same layer (Conv2D with enable_conv_gemm=False): the three GEMMs over the
     # materialised column matrix, (co,K)@(K,P) forward, (co,P)@(P,K) for dw and (K,co)@(co,P) + col2im for dx,
     # each 236.76 GFLOP, with the buffers of the gather timings above
-    kxp = torch.empty(256 * 9 * n * 56 * 56, device="cuda")   # the (K x P) product of the explicit dx
+    # the (K x P) product of the explicit dx and, behind it, the scratch of the balanced launch
+    kxp_bytes = lib().pydtnn_hip_conv_workspace_bytes(native.OP_DX_I2C, 0, n, 256, 56, 56, 256, 3, 3, 1, 1, 1, 1, 1, 1)
+    kxp = torch.empty(kxp_bytes // 4, device="cuda")
     g13 = (n, 256, 56, 56, 256, 3, 3, 1, 1, 1, 1, 1, 1)
     calls["im2col"]()
     y_i2c, dw_i2c = torch.empty_like(xd), torch.empty_like(conv.weights)
     dw_ws, dw_ws_bytes = native.conv_workspace(native.OP_DW, False, g13)
     i2c = {
         "i2c_fwd": lambda: check(lib().pydtnn_hip_conv_i2c_forward(0, *g13, f32(conv.weights), f32(mat), f32(y_i2c),
-                                                                   f32(conv.biases), stream_ptr()), "i2c forward"),
+                                                                   f32(conv.biases), dw_ws, dw_ws_bytes, stream_ptr()),
+                                 "i2c forward"),
         "i2c_dw": lambda: check(lib().pydtnn_hip_conv_i2c_dw(0, *g13, f32(dyd), f32(mat), f32(dw_i2c), dw_ws,
                                                              dw_ws_bytes, stream_ptr()), "i2c dw"),
         "i2c_dx": lambda: check(lib().pydtnn_hip_conv_i2c_dx(0, *g13, f32(conv.weights), f32(dyd), f32(back), f32(kxp),

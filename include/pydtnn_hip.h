@@ -117,6 +117,7 @@ int pydtnn_hip_sgemm_static(int transa, int transb, long m, long n, long k, cons
 #define PYDTNN_HIP_OP_DX 2
 #define PYDTNN_HIP_OP_DX_I2C 3 /* explicit GEMM + col2im/row2im variant of dX */
 #define PYDTNN_HIP_OP_DB 4     /* bias gradient */
+#define PYDTNN_HIP_OP_FWD_I2C 5 /* forward GEMM over a materialised column / row matrix (optional workspace) */
 
 size_t pydtnn_hip_conv_workspace_bytes(int op, int nhwc, int b, int c, int h, int w, int kn, int kh, int kw,
                                        int vpadding, int hpadding, int vstride, int hstride, int vdilation,
@@ -157,15 +158,17 @@ int pydtnn_hip_sconvGemmNHWC_back(unsigned b, unsigned h, unsigned w, unsigned c
  *   Conv2DCPU._forward_nhwc_i2c / _backward_nhwc_i2c   pydtnn/backends/cpu/layers/conv_2d_cpu.py:183-209, :363-397
  * `mat` is x_cols (NCHW: c*kh*kw x b*ho*wo) or x_rows (NHWC: b*ho*wo x c*kh*kw).
  *   forward : y = W * x_cols (+ bias), written straight in the tensor format (the reference's
- *             separate bias pass and 1023 transpose are folded into the store).
+ *             separate bias pass and 1023 transpose are folded into the store).  Workspace: optional,
+ *             OP_FWD_I2C bytes; with it the launch is balanced over the chip like the implicit forward.
  *   dw      : dw = dy_cols * x_cols^T   (NHWC: x_rows^T * dy_rows).  Workspace: OP_DW bytes.
  *   dx      : dx = col2im(W^T * dy_cols) (NHWC: row2im(dy_rows * W^T)); the (K x P) product goes
- *             through the workspace: OP_DX_I2C bytes.
+ *             through the workspace: OP_DX_I2C bytes (the product, then the partial tiles of the balanced
+ *             launch; with no more than the product's K*P*4 bytes the GEMM runs as a plain grid).
  * ---------------------------------------------------------------------------------------- */
 int pydtnn_hip_conv_i2c_forward(int nhwc, int b, int c, int h, int w, int kn, int kh, int kw, int vpadding,
                                 int hpadding, int vstride, int hstride, int vdilation, int hdilation,
                                 const float *weights, const float *mat, float *y, const float *bias_vector,
-                                void *stream);
+                                void *workspace, size_t workspace_bytes, void *stream);
 int pydtnn_hip_conv_i2c_dw(int nhwc, int b, int c, int h, int w, int kn, int kh, int kw, int vpadding, int hpadding,
                            int vstride, int hstride, int vdilation, int hdilation, const float *dy, const float *mat,
                            float *dw, void *workspace, size_t workspace_bytes, void *stream);

@@ -351,7 +351,7 @@ size_t pydtnn_hip_conv_workspace_bytes(int op, int nhwc, int b, int c, int h, in
     ConvGeom g;
     ImageGroups ig;
     long nb = b;
-    if (op != PYDTNN_HIP_OP_DX_I2C && plan_image_groups(&ig, GEOM_ARGS) == PYDTNN_HIP_OK) nb = ig.images;
+    if (op != PYDTNN_HIP_OP_DX_I2C && op != PYDTNN_HIP_OP_FWD_I2C && plan_image_groups(&ig, GEOM_ARGS) == PYDTNN_HIP_OK) nb = ig.images;
     if (geom_from_args(&g, nb, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation) !=
         PYDTNN_HIP_OK)
         return 0;
@@ -364,8 +364,9 @@ size_t pydtnn_hip_conv_workspace_bytes(int op, int nhwc, int b, int c, int h, in
         case PYDTNN_HIP_OP_FWD: return kBalanceBytes;  // optional: a smaller or absent workspace only costs speed
         case PYDTNN_HIP_OP_DX:
             return dx_as_forward(g) ? (((size_t)g.kn * g.k * 4 + 255) & ~(size_t)255) + kBalanceBytes
-                                    : (size_t)g.k * g.p * 4;
-        case PYDTNN_HIP_OP_DX_I2C: return (size_t)g.k * g.p * 4;
+                                    : i2c_product_bytes(g) + kBalanceBytes;
+        case PYDTNN_HIP_OP_DX_I2C: return i2c_product_bytes(g) + kBalanceBytes;  // the (K x P) product, then partial tiles
+        case PYDTNN_HIP_OP_FWD_I2C: return kBalanceBytes;                       // optional, as for the implicit forward
         case PYDTNN_HIP_OP_DB: return bias_grad_workspace_floats(g.n, g.kn) * 4;
         default: return 0;
     }
@@ -459,7 +460,7 @@ void pydtnn_hip_conv_plan_destroy(pydtnn_hip_conv_plan* plan) { delete plan; }
 int pydtnn_hip_conv_i2c_forward(int nhwc, int b, int c, int h, int w, int kn, int kh, int kw, int vpadding,
                                 int hpadding, int vstride, int hstride, int vdilation, int hdilation,
                                 const float* weights, const float* mat, float* y, const float* bias_vector,
-                                void* stream)
+                                void* workspace, size_t workspace_bytes, void* stream)
 {
     if (!weights || !mat || !y) return PYDTNN_HIP_ERR_INVALID;
     ConvGeom g;
@@ -467,20 +468,38 @@ int pydtnn_hip_conv_i2c_forward(int nhwc, int b, int c, int h, int w, int kn, in
     if (rc != PYDTNN_HIP_OK) return rc;
     const ChanEpilogue chan = make_chan(bias_vector, nullptr, nullptr, nullptr, nullptr, 0);
     const hipStream_t st = as_stream(stream);
+    float* ws = (float*)workspace;   // optional: without it the launch is a plain grid of tiles
+    // rows of k floats read with 128-bit loads when k is a multiple of 4 and the matrix is aligned
     if (!nhwc) {
-        const TileSel sel = pick_tile(g.kn, g.p, g.k);
+        // y (kn x P, stored as N,kn,ho,wo) = weights (kn x K) * x_cols (K x P)
+        if (!span_ok_mn(g.p)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+        const bool quads = g.k % 4 == 0 && aligned16(weights);
+        const TileSel sel = quads ? pick_tile_fwd(g.kn, g.p, g.k) : pick_tile(g.kn, g.p, g.k);
+        if (sel == SEL_256x128) {
+            typedef T256x128 T;
+            return launch_balanced<T>(plain_k4<T::BM>(weights, (long)g.kn * g.k, g.k, g.kn),
+                                      plain_mn<T::BN>(mat, (long)g.k * g.p, g.p, 0, g.p),
+                                      epi_nchw(y, g.kn, g.howo, g.p, chan), g.kn, g.p, g.k, ws, workspace_bytes, st);
+        }
         WITH_TILE(sel, {
-            if (!span_ok_mn(g.p)) return PYDTNN_HIP_ERR_UNSUPPORTED;
-            rc = launch<T>(plain_k<T::BM, false>(weights, (long)g.kn * g.k, g.k, 0, g.kn, 0),
-                           plain_mn<T::BN>(mat, (long)g.k * g.p, g.p, 0, g.p),
-                           epi_nchw(y, g.kn, g.howo, g.p, chan), g.kn, g.p, no_split(g.k), 1, st);
+            rc = launch_balanced<T>(plain_k<T::BM, false>(weights, (long)g.kn * g.k, g.k, 0, g.kn, 0),
+                                    plain_mn<T::BN>(mat, (long)g.k * g.p, g.p, 0, g.p),
+                                    epi_nchw(y, g.kn, g.howo, g.p, chan), g.kn, g.p, g.k, ws, workspace_bytes, st);
         })
     } else {
+        // y (P x kn) = x_rows (P x K) * weights (K x kn)
         const TileSel sel = pick_tile(g.p, g.kn, g.k);
+        const bool quads = g.k % 4 == 0 && aligned16(mat);
         WITH_TILE(sel, {
-            rc = launch<T>(plain_k<T::BM, false>(mat, g.p * g.k, g.k, 0, g.p, 0),
-                           plain_mn<T::BN>(weights, (long)g.k * g.kn, g.kn, 0, g.kn),
-                           epi_plain(y, g.kn, 0, g.p, g.kn, chan), g.p, g.kn, no_split(g.k), 1, st);
+            if (!span_ok_k(T::BM, g.k, 0, 0) || !span_ok_mn(g.kn)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+            auto bl = plain_mn<T::BN>(weights, (long)g.k * g.kn, g.kn, 0, g.kn);
+            const EpiPlain ep = epi_plain(y, g.kn, 0, g.p, g.kn, chan);
+            if (quads)
+                rc = launch_balanced<T>(plain_k4<T::BM>(mat, g.p * g.k, g.k, g.p), bl, ep, g.p, g.kn, g.k, ws,
+                                        workspace_bytes, st);
+            else
+                rc = launch_balanced<T>(plain_k<T::BM, false>(mat, g.p * g.k, g.k, 0, g.p, 0), bl, ep, g.p, g.kn, g.k, ws,
+                                        workspace_bytes, st);
         })
     }
     return rc;

@@ -181,20 +181,33 @@ int conv_dx_i2c(const ConvGeom& g, int nhwc, const float* w, const float* dy, fl
     const size_t need = (size_t)g.k * g.p * 4;
     if (!ws || ws_bytes < need) return PYDTNN_HIP_ERR_WORKSPACE;
     if ((long)g.k * g.p >= (1l << 33)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+    // what lies behind the product balances the GEMM's launch
+    const size_t product = i2c_product_bytes(g);
+    float* balance = ws_bytes >= product + kBalanceBytes ? ws + product / 4 : nullptr;
+    const size_t balance_bytes = balance ? ws_bytes - product : 0;
     int rc = PYDTNN_HIP_OK;
     if (!nhwc) {
         // res(K x P) = W^T (A(m = k, kk = filter) = w[kk*K + m]) * dy_cols (dy seen as a 1x1 im2col)
         ConvGeom g1;
         rc = make_conv_geom(&g1, g.n, g.kn, g.ho, g.wo, 1, 1, 1, 0, 0, 1, 1, 1, 1);
         if (rc != PYDTNN_HIP_OK) return rc;
-        const TileSel sel = pick_tile(g.k, g.p);
-        WITH_TILE(sel, {
-            auto al = plain_mn<T::BM>(w, (long)g.kn * g.k, g.k, 0, g.k);
+        const TileSel sel = pick_tile_fwd(g.k, g.p, g.kn);
+        if (sel == SEL_256x128) {
+            typedef T256x128 T;
             Im2colNchwMN<T::BN> bl;
             bl.x = dy; bl.g = g1;
-            rc = launch<T>(al, bl, epi_plain(ws, g.p, 0, g.k, g.p, no_epilogue()), g.k, g.p, no_split(g.kn), 1,
-                           stream);
-        })
+            rc = launch_balanced<T>(plain_mn<T::BM>(w, (long)g.kn * g.k, g.k, 0, g.k), bl,
+                                    epi_plain(ws, g.p, 0, g.k, g.p, no_epilogue()), g.k, g.p, g.kn, balance,
+                                    balance_bytes, stream);
+        } else {
+            WITH_TILE(sel, {
+                auto al = plain_mn<T::BM>(w, (long)g.kn * g.k, g.k, 0, g.k);
+                Im2colNchwMN<T::BN> bl;
+                bl.x = dy; bl.g = g1;
+                rc = launch_balanced<T>(al, bl, epi_plain(ws, g.p, 0, g.k, g.p, no_epilogue()), g.k, g.p, g.kn, balance,
+                                        balance_bytes, stream);
+            })
+        }
         if (rc != PYDTNN_HIP_OK) return rc;
         rc = launch_col2im_nchw(ws, dx, g, stream);
         if (rc != PYDTNN_HIP_OK || !gate) return rc;
@@ -205,7 +218,8 @@ int conv_dx_i2c(const ConvGeom& g, int nhwc, const float* w, const float* dy, fl
     WITH_TILE(sel, {
         auto al = plain_k<T::BM, false>(dy, g.p * g.kn, g.kn, 0, g.p, 0);
         auto bl = plain_k<T::BN, false>(w, (long)g.k * g.kn, g.kn, 0, g.k, 0);
-        rc = launch<T>(al, bl, epi_plain(ws, g.k, 0, g.p, g.k, no_epilogue()), g.p, g.k, no_split(g.kn), 1, stream);
+        rc = launch_balanced<T>(al, bl, epi_plain(ws, g.k, 0, g.p, g.k, no_epilogue()), g.p, g.k, g.kn, balance,
+                                balance_bytes, stream);
     })
     if (rc != PYDTNN_HIP_OK) return rc;
     rc = launch_row2im_nhwc(ws, dx, g, stream);

@@ -284,6 +284,9 @@ inline bool pointwise_nhwc(const ConvGeom& g)
     return g.khw == 1 && g.vstride == 1 && g.hstride == 1 && g.vpadding == 0 && g.hpadding == 0;
 }
 
+// bytes of the (K x P) product of the explicit input gradient, rounded so that what follows it stays aligned
+inline size_t i2c_product_bytes(const ConvGeom& g) { return ((size_t)g.k * g.p * 4 + 255) & ~(size_t)255; }
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 // Row-major forward launch (y is P x kn) with the epilogue variant the masks ask for.

@@ -14,7 +14,7 @@ LIB_DIR = os.path.join(_HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libpydtnn_hip.so")
 COMPAT_LIB_PATH = os.path.join(LIB_DIR, "libconvGemm.so")
 
-OP_FWD, OP_DW, OP_DX, OP_DX_I2C, OP_DB = range(5)
+OP_FWD, OP_DW, OP_DX, OP_DX_I2C, OP_DB, OP_FWD_I2C = range(6)
 # status codes of include/pydtnn_hip.h
 PYDTNN_HIP_OK, PYDTNN_HIP_ERR_INVALID, PYDTNN_HIP_ERR_WORKSPACE, PYDTNN_HIP_ERR_LAUNCH, PYDTNN_HIP_ERR_UNSUPPORTED = range(5)
 
@@ -52,7 +52,7 @@ SIGNATURES = {
                                                  _c.c_size_t, _vp]),
     "pydtnn_hip_sconvGemm_back_gated": (_c.c_int, [_c.c_int] + _geom13_u + [_f32p] * 3 + [_i8p, _vp, _c.c_size_t, _vp]),
     "pydtnn_hip_max_pool_2d_bwd_gated": (_c.c_int, [_c.c_int, _f32p, _i32p, _f32p, _i8p] + [_c.c_int] * 12 + [_vp]),
-    "pydtnn_hip_conv_i2c_forward": (_c.c_int, [_c.c_int] + _geom13_i + [_f32p] * 4 + [_vp]),
+    "pydtnn_hip_conv_i2c_forward": (_c.c_int, [_c.c_int] + _geom13_i + [_f32p] * 4 + [_vp, _c.c_size_t, _vp]),
     "pydtnn_hip_conv_i2c_dw": (_c.c_int, [_c.c_int] + _geom13_i + [_f32p] * 3 + [_vp, _c.c_size_t, _vp]),
     "pydtnn_hip_conv_i2c_dx": (_c.c_int, [_c.c_int] + _geom13_i + [_f32p] * 3 + [_vp, _c.c_size_t, _vp]),
     "pydtnn_hip_chan_eltwise": (_c.c_int, [_f32p, _f32p, _f32p, _c.c_long, _c.c_int, _c.c_int] + [_f32p] * 5 +

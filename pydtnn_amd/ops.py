@@ -469,8 +469,9 @@ def _i2c_dx_f64(nhwc, geom13, weights, dy, dx):
 def conv_i2c_forward(nhwc, geom13, weights, mat, y, biases):
     if _is_f64(weights, mat, y, biases):
         return _i2c_forward_f64(nhwc, geom13, weights, mat, y, biases)
-    check(lib().pydtnn_hip_conv_i2c_forward(int(nhwc), *geom13, f32(weights), f32(mat), f32(y), f32(biases),
-                                            stream_ptr()), "conv_i2c_forward")
+    ws, ws_bytes = native.conv_workspace(native.OP_FWD_I2C, nhwc, geom13)
+    check(lib().pydtnn_hip_conv_i2c_forward(int(nhwc), *geom13, f32(weights), f32(mat), f32(y), f32(biases), ws,
+                                            ws_bytes, stream_ptr()), "conv_i2c_forward")
     return y
 
 

@@ -66,8 +66,10 @@ def test_workspace_queries_are_pure_host_code(native):
     # explicit route
     assert lib.pydtnn_hip_conv_workspace_bytes(native.OP_DX, 0, *cfg2) == kn_k + balance
     strided = (8, 3, 32, 32, 16, 3, 3, 1, 1, 2, 2, 1, 1)
-    assert lib.pydtnn_hip_conv_workspace_bytes(native.OP_DX, 0, *strided) == 27 * 8 * 16 * 16 * 4
-    assert lib.pydtnn_hip_conv_workspace_bytes(native.OP_DX_I2C, 1, *cfg2) == 2304 * 64 * 56 * 56 * 4
+    assert lib.pydtnn_hip_conv_workspace_bytes(native.OP_DX, 0, *strided) == 27 * 8 * 16 * 16 * 4 + balance
+    # the explicit route: the (K x P) product and behind it the scratch of the balanced launch; forward only the latter
+    assert lib.pydtnn_hip_conv_workspace_bytes(native.OP_DX_I2C, 1, *cfg2) == 2304 * 64 * 56 * 56 * 4 + balance
+    assert lib.pydtnn_hip_conv_workspace_bytes(native.OP_FWD_I2C, 0, *cfg2) == balance
     # invalid geometry (kernel larger than the padded image) yields 0, not a crash
     assert lib.pydtnn_hip_conv_workspace_bytes(native.OP_DW, 0, 1, 1, 2, 2, 1, 5, 5, 0, 0, 1, 1, 1, 1) == 0
     assert lib.pydtnn_hip_sgemm_workspace_bytes(4096, 4096, 4096) == 0
