@@ -328,6 +328,12 @@ int pydtnn_hip_categorical_cross_entropy(const float *y_pred, const float *y_tar
 /* SGD with momentum, in place (pydtnn/backends/cpu/optimizers/sgd_cpu.py:28-41). */
 int pydtnn_hip_sgd_momentum(float *w, const float *dw, float *velocity, long total, float lr, float momentum,
                             float decay, int nesterov, void *stream);
+/* The same step for `count` tensors in one pass (a layer's weights and biases: SGDCPU.update walks
+ * layer.grad_vars, pydtnn/backends/cpu/optimizers/sgd_cpu.py:30-41).  w, dw, velocity and total are host arrays of
+ * `count` device pointers / element counts; every element gets what pydtnn_hip_sgd_momentum gives it. */
+int pydtnn_hip_sgd_momentum_multi(int count, float *const *w, const float *const *dw, float *const *velocity,
+                                  const long *total, float lr, float momentum, float decay, int nesterov,
+                                  void *stream);
 
 /* ------------------------------------------------------------------------------------------
  * The float64 route.  The reference computes in float64 through its explicit path only: the im2col / im2row /

@@ -729,4 +729,10 @@ int pydtnn_hip_sgd_momentum(float* w, const float* dw, float* velocity, long tot
     return launch_sgd_momentum(w, dw, velocity, total, lr, momentum, decay, nesterov, as_stream(stream));
 }
 
+int pydtnn_hip_sgd_momentum_multi(int count, float* const* w, const float* const* dw, float* const* velocity,
+                                  const long* total, float lr, float momentum, float decay, int nesterov, void* stream)
+{
+    return launch_sgd_momentum_multi(count, w, dw, velocity, total, lr, momentum, decay, nesterov, as_stream(stream));
+}
+
 }  // extern "C"

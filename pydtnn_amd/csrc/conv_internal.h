@@ -31,6 +31,8 @@ int launch_max_pool_bwd_nhwc(const float*, const int32_t*, float*, const ConvGeo
 int launch_avg_pool_fwd(int nhwc, const float*, float*, const ConvGeom&, hipStream_t);
 int launch_avg_pool_bwd(int nhwc, const float*, float*, const ConvGeom&, hipStream_t);
 int launch_sgd_momentum(float*, const float*, float*, long, float, float, float, int, hipStream_t);
+int launch_sgd_momentum_multi(int, float* const*, const float* const*, float* const*, const long*, float, float, float,
+                              int, hipStream_t);
 
 namespace convint {
 

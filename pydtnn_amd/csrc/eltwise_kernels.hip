@@ -947,19 +947,61 @@ __global__ void __launch_bounds__(kThreads) max_pool_bwd_windows_nhwc_kernel(con
 }
 
 // ---------------------------------------------------------------- SGD with momentum
-// pydtnn/backends/cpu/optimizers/sgd_cpu.py:28-41
-__global__ void __launch_bounds__(kThreads) sgd_momentum_kernel(float* __restrict__ w, const float* __restrict__ dw,
-                                                               float* __restrict__ velocity, long total, float lr,
-                                                               float momentum, float decay, int nesterov)
+// pydtnn/backends/cpu/optimizers/sgd_cpu.py:28-41: velocity = momentum * velocity + dw;
+// w -= lr * (decay * w + velocity)   (Nesterov: w -= lr * (decay * w + dw + momentum * velocity)).
+// One launch updates up to kSgdTensors tensors (a layer's weights and biases, or more): every workgroup of
+// kSgdBlock elements belongs to one tensor (first_block[] is the running sum of the tensors' workgroup counts)
+// and a thread moves four consecutive elements with 128-bit accesses where the tensor allows it.
+constexpr int kSgdTensors = 8;
+constexpr int kSgdBlock = kThreads * 4;
+struct SgdBatch {
+    float* w[kSgdTensors];
+    const float* dw[kSgdTensors];
+    float* velocity[kSgdTensors];
+    long total[kSgdTensors];
+    unsigned first_block[kSgdTensors + 1];
+    int count;
+};
+
+__device__ __forceinline__ float sgd_step(float wv, float g, float* v, float lr, float momentum, float decay, int nesterov)
 {
-    const long idx = (long)blockIdx.x * kThreads + threadIdx.x;
+    *v = momentum * *v + g;
+    const float upd = nesterov ? (decay * wv + g + momentum * *v) : (decay * wv + *v);
+    return wv - lr * upd;
+}
+
+__global__ void __launch_bounds__(kThreads) sgd_momentum_kernel(SgdBatch b, float lr, float momentum, float decay,
+                                                               int nesterov)
+{
+    int t = 0;
+#pragma unroll
+    for (int i = 1; i < kSgdTensors; ++i)
+        if (i < b.count && blockIdx.x >= b.first_block[i]) t = i;
+    float* __restrict__ w = b.w[t];
+    const float* __restrict__ dw = b.dw[t];
+    float* __restrict__ velocity = b.velocity[t];
+    const long total = b.total[t];
+    const long idx = ((long)(blockIdx.x - b.first_block[t]) * kThreads + threadIdx.x) * 4;
     if (idx >= total) return;
-    const float g = dw[idx];
-    const float v = momentum * velocity[idx] + g;
-    const float wv = w[idx];
-    const float upd = nesterov ? (decay * wv + g + momentum * v) : (decay * wv + v);
-    w[idx] = wv - lr * upd;
-    velocity[idx] = v;
+    const bool vec = idx + 4 <= total &&
+                     (((uintptr_t)w | (uintptr_t)dw | (uintptr_t)velocity) & 15) == 0;   // wave-uniform but for the tail
+    if (vec) {
+        const float4 g = *reinterpret_cast<const float4*>(dw + idx);
+        float4 v = *reinterpret_cast<const float4*>(velocity + idx);
+        float4 wv = *reinterpret_cast<const float4*>(w + idx);
+        wv.x = sgd_step(wv.x, g.x, &v.x, lr, momentum, decay, nesterov);
+        wv.y = sgd_step(wv.y, g.y, &v.y, lr, momentum, decay, nesterov);
+        wv.z = sgd_step(wv.z, g.z, &v.z, lr, momentum, decay, nesterov);
+        wv.w = sgd_step(wv.w, g.w, &v.w, lr, momentum, decay, nesterov);
+        *reinterpret_cast<float4*>(w + idx) = wv;
+        *reinterpret_cast<float4*>(velocity + idx) = v;
+        return;
+    }
+    for (long i = idx; i < total && i < idx + 4; ++i) {
+        float v = velocity[i];
+        w[i] = sgd_step(w[i], dw[i], &v, lr, momentum, decay, nesterov);
+        velocity[i] = v;
+    }
 }
 
 // ---------------------------------------------------------------- BatchNormalization, training
@@ -1600,14 +1642,34 @@ int launch_max_pool_bwd_nhwc(const float* dy, const int32_t* idx_max, float* dx,
     return PYDTNN_HIP_OK;
 }
 
+int launch_sgd_momentum_multi(int count, float* const* w, const float* const* dw, float* const* velocity,
+                              const long* total, float lr, float momentum, float decay, int nesterov, hipStream_t stream)
+{
+    if (count <= 0 || !w || !dw || !velocity || !total) return PYDTNN_HIP_ERR_INVALID;
+    for (int i0 = 0; i0 < count; i0 += kSgdTensors) {
+        SgdBatch b;
+        b.count = count - i0 < kSgdTensors ? count - i0 : kSgdTensors;
+        unsigned blocks = 0;
+        for (int i = 0; i < kSgdTensors; ++i) {
+            const int j = i < b.count ? i0 + i : i0;
+            if (!w[j] || !dw[j] || !velocity[j] || total[j] <= 0) return PYDTNN_HIP_ERR_INVALID;
+            const long nb = (total[j] + kSgdBlock - 1) / kSgdBlock;
+            if (nb + blocks >= (1l << 31)) return PYDTNN_HIP_ERR_UNSUPPORTED;
+            b.w[i] = w[j]; b.dw[i] = dw[j]; b.velocity[i] = velocity[j]; b.total[i] = total[j];
+            b.first_block[i] = blocks;
+            if (i < b.count) blocks += (unsigned)nb;
+        }
+        b.first_block[kSgdTensors] = blocks;
+        hipLaunchKernelGGL(sgd_momentum_kernel, dim3(blocks), dim3(kThreads), 0, stream, b, lr, momentum, decay, nesterov);
+        HIP_RETURN_IF_LAUNCH_FAILED();
+    }
+    return PYDTNN_HIP_OK;
+}
+
 int launch_sgd_momentum(float* w, const float* dw, float* velocity, long total, float lr, float momentum, float decay,
                         int nesterov, hipStream_t stream)
 {
-    if (total <= 0) return PYDTNN_HIP_ERR_INVALID;
-    hipLaunchKernelGGL(sgd_momentum_kernel, dim3(blocks_for(total)), dim3(kThreads), 0, stream, w, dw, velocity, total,
-                       lr, momentum, decay, nesterov);
-    HIP_RETURN_IF_LAUNCH_FAILED();
-    return PYDTNN_HIP_OK;
+    return launch_sgd_momentum_multi(1, &w, &dw, &velocity, &total, lr, momentum, decay, nesterov, stream);
 }
 
 int launch_softmax_fwd(const float* x, float* y, int rows, int cols, hipStream_t stream)

@@ -22,6 +22,18 @@ from .layers import EVALUATE_MODE, TRAIN_MODE, UNSPECIFIED_MODE
 from .utils import PYDTNN_TENSOR_FORMAT_NCHW, PYDTNN_TENSOR_FORMAT_NHWC
 
 
+# The second stream of enable_backward_overlap, one per device for the whole process: the scratch buffers of the
+# library binding are kept per (device, stream), so models that come and go must not each bring a stream of their own.
+_SIDE_STREAMS = {}
+
+
+def _side_stream(device):
+    side = _SIDE_STREAMS.get(device.index)
+    if side is None:
+        side = _SIDE_STREAMS[device.index] = torch.cuda.Stream(device=device)     # default priority
+    return side
+
+
 def _layer_id_generator():
     current_layer_id = 0
     while True:
@@ -88,9 +100,9 @@ class Model:
         self.batch_size = self.kwargs["batch_size"]
         self._fused = False
         self.stepping = False  # True while train_batch runs its own forward / backward loops
-        self._side_streams = {}  # device index -> second stream of enable_backward_overlap
         self._overlap_min_elements = 1 << 16
-        self._side_refs = []     # (stream, tensors it still reads): kept alive until the caller's stream has waited
+        self._side_used = set()  # second streams this step has put work on and not yet waited for
+        self._side_launches = 0  # bodies sent to a second stream so far
         # pydtnn/model.py:216-218: without the flag every BestOf just calls its first alternative
         BestOf.use_always_the_first_alternative(not self.kwargs["enable_best_of"])
 
@@ -236,8 +248,8 @@ class Model:
     def beside_backward(self, layer, *tensors):
         """Inside train_batch with ``enable_backward_overlap``: the body's work (the gradients of ``layer``'s
         variables) goes to the model's second stream, after everything enqueued so far on the caller's, and
-        ``layer.grads_ready`` is the event that marks its end; ``tensors`` (what the body reads) stay referenced until
-        the caller's stream has waited for that stream, so the allocator cannot hand their memory out in between.
+        ``layer.grads_ready`` is the event that marks its end; ``tensors`` (what the body reads) are marked as in
+        use by that stream, so the allocator cannot hand their memory out before it has read them.
         Otherwise, and for small problems (under 2^16 elements read: nothing to overlap but launches), the body
         runs in place."""
         if not (self.stepping and self.kwargs["enable_backward_overlap"] and tensors and tensors[0].is_cuda
@@ -245,20 +257,23 @@ class Model:
             yield
             return
         device = tensors[0].device
-        side = self._side_streams.get(device.index)
-        if side is None:
-            side = self._side_streams[device.index] = torch.cuda.Stream(device=device)     # default priority
+        side = _side_stream(device)
         side.wait_stream(torch.cuda.current_stream(device))
-        self._side_refs.append((side, tensors))
+        self._side_used.add(side)
+        self._side_launches += 1
+        for t in tensors:
+            # the allocator hands the tensor's memory out again only after the second stream has passed this point,
+            # so the tensor itself can be dropped as soon as the layers are done with it
+            t.record_stream(side)
         with torch.cuda.stream(side):
             yield
             layer.grads_ready = torch.cuda.Event()
             layer.grads_ready.record(side)
 
     def _join_side_stream(self):
-        for side in {s for s, _ in self._side_refs}:
+        for side in self._side_used:
             torch.cuda.current_stream(side.device).wait_stream(side)
-        self._side_refs.clear()
+        self._side_used.clear()
 
     def evaluate_batch(self, x):
         """Forward pass of pydtnn/model.py:623-644."""
@@ -389,11 +404,13 @@ class SGD:
         self.decay = decay
 
     def update(self, layer):
+        triples = []
         for w_, dw_ in layer.grad_vars.items():
             w, dw = getattr(layer, w_), getattr(layer, dw_)
             velocity = getattr(layer, "velocity_%s" % w_, None)
             if velocity is None:
                 velocity = torch.zeros_like(w)
                 setattr(layer, "velocity_%s" % w_, velocity)
-            ops.sgd_momentum(w, dw.reshape(w.shape).contiguous(), velocity, self.learning_rate, self.momentum,
-                             self.decay, self.nesterov)
+            triples.append((w, dw.reshape(w.shape).contiguous(), velocity))
+        if triples:   # the layer's variables in one launch
+            ops.sgd_momentum_multi(triples, self.learning_rate, self.momentum, self.decay, self.nesterov)

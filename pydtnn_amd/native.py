@@ -76,6 +76,8 @@ SIGNATURES = {
                                                         _c.c_int, _vp, _c.c_size_t, _vp]),
     "pydtnn_hip_sgd_momentum": (_c.c_int, [_f32p, _f32p, _f32p, _c.c_long, _c.c_float, _c.c_float, _c.c_float,
                                            _c.c_int, _vp]),
+    "pydtnn_hip_sgd_momentum_multi": (_c.c_int, [_c.c_int, _vp, _vp, _vp, _vp, _c.c_float, _c.c_float, _c.c_float,
+                                                 _c.c_int, _vp]),
     # float64 route
     "pydtnn_hip_dgemm_workspace_bytes": (_c.c_size_t, [_c.c_long] * 3),
     "pydtnn_hip_dgemm": (_c.c_int, [_c.c_int, _c.c_int, _c.c_long, _c.c_long, _c.c_long, _vp, _c.c_long, _vp, _c.c_long,

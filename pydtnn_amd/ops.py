@@ -409,6 +409,24 @@ def sgd_momentum(w, dw, velocity, lr, momentum, decay=0.0, nesterov=False):
                                         int(nesterov), stream_ptr()), "sgd_momentum")
 
 
+def sgd_momentum_multi(tensors, lr, momentum, decay=0.0, nesterov=False):
+    """The SGD step of ``sgd_momentum`` for several (w, dw, velocity) triples in one launch (a layer's variables)."""
+    import ctypes
+    if len(tensors) == 1 or any(_is_f64(*t) for t in tensors):
+        for w, dw, velocity in tensors:
+            sgd_momentum(w, dw, velocity, lr, momentum, decay, nesterov)
+        return
+    n = len(tensors)
+    ptrs = ctypes.c_void_p * n
+    for t in tensors:
+        for a in t:
+            f32(a)    # float32, contiguous, on the GPU
+    check(lib().pydtnn_hip_sgd_momentum_multi(
+        n, ptrs(*[t[0].data_ptr() for t in tensors]), ptrs(*[t[1].data_ptr() for t in tensors]),
+        ptrs(*[t[2].data_ptr() for t in tensors]), (ctypes.c_long * n)(*[t[0].numel() for t in tensors]), lr, momentum,
+        decay, int(nesterov), stream_ptr()), "sgd_momentum_multi")
+
+
 # --------------------------------------------------------------------------- explicit (i2c) conv GEMMs
 
 def _geom13(b, c, h, w, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation):

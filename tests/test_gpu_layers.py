@@ -428,14 +428,14 @@ def test_backward_overlap_changes_no_bit_of_a_training_run(pd, fmt, conv_gemm, n
         losses = []
         for _ in range(8):     # long enough for the caching allocator to hand freed blocks out again
             losses.append(model.train_batch(x, y_targ, loss_fn, opt))    # no synchronization between the steps
-            assert not model._side_refs
+            assert not model._side_used
         losses = [float(v) for v in losses]
         state = {}
         for l in model.get_all_layers():
             for var, grad in l.grad_vars.items():
                 state[f"{l.id}.{var}"] = getattr(l, var).clone()
                 state[f"{l.id}.{grad}"] = getattr(l, grad).clone()
-        return losses, state, bool(model._side_streams)
+        return losses, state, model._side_launches > 0
 
     losses_a, state_a, used_a = run(True)
     losses_b, state_b, used_b = run(False)
@@ -458,7 +458,7 @@ def test_backward_overlap_stays_inside_the_training_step(pd):
     model._overlap_min_elements = 0
     conv.forward(torch.randn(2, 3, 6, 6, device="cuda"))
     conv.backward(torch.randn(2, 3, 6, 6, device="cuda"))
-    assert not model._side_streams and not model._side_refs
+    assert model._side_launches == 0 and not model._side_used
 
 
 def test_relu_folding_stays_inside_the_training_step(pd):
