@@ -92,7 +92,9 @@ __global__ void __launch_bounds__(kThreads) im2col_nchw_lds_kernel(const float* 
                 v[e] = ok ? val : 0.0f;
             }
             if (VEC4) {
-                *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+                // the matrix is written once and read by a later kernel: a streaming store
+                const gemm::floatx4 quad = {v[0], v[1], v[2], v[3]};
+                __builtin_nontemporal_store(quad, reinterpret_cast<gemm::floatx4*>(dst));
             } else {
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
@@ -195,6 +197,8 @@ __global__ void __launch_bounds__(kThreads) col2im_nchw_kernel(const float* __re
                 int ox = 0;
                 const bool ok =
                     out_coord<UNIT>(ww + g.hpadding - g.hdilation * jj, g.hstride, g.fd_hs, g.wo, &ox) && row_ok;
+                // (a streaming load here measured 4.57 against 5.17 TB/s: neighbouring rows of dx share lines of the
+                // matrix through the caches)
                 const float val = src[(long)(ii * kw + jj) * g.p + (ok ? oy * g.wo + ox : 0)];
                 acc += ok ? val : 0.0f;
             }
@@ -298,11 +302,15 @@ __global__ void __launch_bounds__(kThreads) im2row_nhwc_quads_kernel(const float
     __syncthreads();
     const long left = g.p - p0;
     const long valid4 = (left < rows_per_block ? left : (long)rows_per_block) * c4n * KHW;  // float4s of this block
-    float4* dst = reinterpret_cast<float4*>(rows + p0 * g.k);
+    gemm::floatx4* dst = reinterpret_cast<gemm::floatx4*>(rows + p0 * g.k);
 #pragma unroll
     for (int t = 0; t < KHW; ++t) {
         const int f4 = t * kThreads + threadIdx.x;
-        if (f4 < valid4) dst[f4] = staged[f4];
+        if (f4 < valid4) {
+            const float4 q = staged[f4];
+            const gemm::floatx4 quad = {q.x, q.y, q.z, q.w};
+            __builtin_nontemporal_store(quad, dst + f4);   // written once, read by a later kernel
+        }
     }
 }
 
@@ -542,7 +550,9 @@ __global__ void __launch_bounds__(kThreads) row2im_nhwc_walk_kernel(const float*
         const bool row_ok = (unsigned)oy < (unsigned)g.ho;
         const uint32_t soff = row_ok ? (uint32_t)oy * g.wo * g.k * 4u : 0u;
 #pragma unroll
-        for (int j = 0; j < NLD; ++j) v[j] = gemm::buf_load4(src, row_ok ? off[j] : gemm::kOob, soff);
+        for (int j = 0; j < NLD; ++j)   // streaming loads (cache policy nt): each line of the matrix is read once
+            v[j] = __builtin_bit_cast(gemm::floatx4, __builtin_amdgcn_raw_buffer_load_b128(
+                src, (int)(row_ok ? off[j] : gemm::kOob), (int)soff, 2));
     };
 
     const int cc = threadIdx.x & (CB - 1), slot = threadIdx.x / CB;

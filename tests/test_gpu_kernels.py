@@ -253,6 +253,59 @@ def test_streaming_kernel_shapes_nhwc(cg, oracle, d):
     assert_close(host(dw), dw_ref, what="dw")
 
 
+# one shape per chunk count the streaming kernel is built for (1, 2 and 4 chunks of 64 channels at 1x1, 9 at 3x3)
+stream_chunk_grid = [D(16, 64, 56, 56, 64, 1, 1, 0, 0, 1, 1, 1, 1), D(16, 128, 56, 56, 64, 1, 1, 0, 0, 1, 1, 1, 1),
+                     D(16, 256, 56, 56, 64, 1, 1, 0, 0, 1, 1, 1, 1), D(16, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1, 1, 1)]
+
+
+@pytest.mark.parametrize("masks", ["none", "relu_mask", "residual", "gate"])
+@pytest.mark.parametrize("d", stream_chunk_grid, ids=repr)
+def test_streaming_kernel_walks_both_ways_with_every_store(ops, cg, oracle, d, masks):
+    """A launch of the streaming kernel walks the pixel blocks forwards or backwards, the opposite way of the launch
+    that last walked its input on the same stream.  Calling twice (three times) with the same tensors therefore
+    runs both directions of each built (chunk count, store) instance: plain, with the ReLU mask, with the residual
+    sum and ReLU, and (the input gradient as a forward launch) with the gate.  Every repetition must give the same
+    bits, and they must agree with the oracle."""
+    announce("stream kernel both directions", masks, d)
+    x, w, b, dy = case(d)
+    xr, wr, dyr = nhwc(x), w_nhwc(w), nhwc(dy)
+    p = oracle.ConvParams(*d.geom())
+    y_ref, rows = oracle.conv2d_forward_nhwc_i2c(xr, wr, b, p)
+    xd, wd, bd, dyd = dev(xr), dev(wr), dev(b), dev(dyr)
+    rng = np.random.default_rng(4)
+    if masks == "none":
+        out = torch.empty(y_ref.shape, device="cuda")
+        run = lambda: (cg.conv_gemm_nhwc(wd, xd, biases=out, biases_vector=bd, **_kw(d)).clone(),)
+        want = (y_ref,)
+    elif masks == "relu_mask":
+        out, mask = torch.empty(y_ref.shape, device="cuda"), torch.empty(y_ref.shape, dtype=torch.int8, device="cuda")
+        run = lambda: (cg.conv_gemm_nhwc(wd, xd, biases=out, biases_vector=bd, relu=True, relu_mask=mask,
+                                         **_kw(d)).clone(), mask.clone())
+        want = (np.maximum(y_ref, 0), (y_ref > 0).astype(np.int8))
+    elif masks == "residual":
+        res_np = rng.standard_normal(y_ref.shape).astype(np.float32)
+        out, res = torch.empty(y_ref.shape, device="cuda"), dev(res_np)
+        run = lambda: (cg.conv_gemm_nhwc(wd, xd, biases=out, biases_vector=bd, residual=res, relu_after_residual=True,
+                                         **_kw(d)).clone(),)
+        want = (np.maximum(y_ref + res_np, 0),)
+    else:
+        gate_np = (rng.random(xr.shape) < 0.6).astype(np.int8)
+        out, gate = torch.empty(xr.shape, device="cuda"), dev(gate_np)
+        run = lambda: (cg.deconv_gemm_nhwc(wd, dyd, out, gate=gate, **_kw(d)).clone(),)
+        _, _, dx_ref = oracle.conv2d_backward_nhwc_i2c(dyr, rows, wr, xr.shape, p)
+        want = (dx_ref * gate_np,)
+    first = run()
+    for rep in range(2):
+        for a, ref in zip(run(), first):
+            assert torch.equal(a, ref), f"repetition {rep + 1} differs from the first launch"
+    for a, ref in zip(first, want):
+        if ref.dtype == np.int8:
+            # a value within rounding of zero may fall on either side of the mask
+            assert np.mean(host(a) != ref) < 1e-4
+        else:
+            assert_close(host(a), ref, what=masks)
+
+
 # unpadded NCHW layers with wide filter rows (AlexNet-style first layers): rows of 5 .. 12 taps, strides 1 .. 4,
 # vertical dilation, filter counts on and off the 96-row tile
 quad_grid = [
