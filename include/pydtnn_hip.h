@@ -254,6 +254,27 @@ int pydtnn_hip_max_pool_2d_bwd_gated(int nhwc, const float *dy, const int32_t *i
                                      int b, int c, int h, int w, int kh, int kw, int vpadding, int hpadding,
                                      int vstride, int hstride, int vdilation, int hdilation, void *stream);
 
+/* Two consecutive convolutions of one path as a single launch, NHWC, inference: the forward of
+ * pydtnn_hip_sconvGemmNHWC with the first set of arguments (filter `weights`, its bias / BN vectors and ReLU flag),
+ * whose result is never stored but fed, as it leaves the matrix cores, to a 1 x 1 convolution at unit stride
+ * without padding with the second set (`weights2` of shape (kn, 1, 1, kn2), its vectors), which stores y
+ * (b, ho, wo, kn2) and, with `residual`, adds it and rectifies as pydtnn_hip_sconvGemm_residual does.  This is the
+ * tail of a ResNet bottleneck after the fusion pass (pydtnn/model.py:294-349): Conv2DBatchNormalizationRelu 3x3,
+ * Conv2DBatchNormalization 1x1, the AdditionBlock's sum (pydtnn/backends/cpu/layers/addition_block_cpu.py:41-45) and
+ * the Relu after it.  Results equal the two separate calls bit for bit.  Built for the shapes of the first
+ * bottlenecks only (3x3, pad 1, unit stride and dilation, 64 -> 64 filters, then at most 256, BN on the second
+ * layer, at least 32768 output pixels in multiples of 32, 16-byte aligned tensors): any other call returns
+ * PYDTNN_HIP_ERR_UNSUPPORTED before anything is launched, and the caller makes the two calls.  No workspace. */
+int pydtnn_hip_sconvGemm_pair_nhwc(unsigned b, unsigned h, unsigned w, unsigned c, unsigned kn, unsigned kh, unsigned kw,
+                                   unsigned vpadding, unsigned hpadding, unsigned vstride, unsigned hstride,
+                                   unsigned vdilation, unsigned hdilation, const float *weights, const float *x,
+                                   const float *bias_vector, const float *bn_running_mean, const float *bn_inv_std,
+                                   const float *bn_gamma, const float *bn_beta, bool relu, unsigned kn2,
+                                   const float *weights2, float *y, const float *bias_vector2,
+                                   const float *bn_running_mean2, const float *bn_inv_std2, const float *bn_gamma2,
+                                   const float *bn_beta2, bool relu2, const float *residual, bool relu_after_add,
+                                   void *stream);
+
 /* A forward convolution with everything but the activations bound once: a layer that calls with the same
  * geometry, filter and per-channel vectors at every step (an inference loop) builds the plan when it is
  * initialised, as the reference's layers build their ConvGemm object and its kernel arguments in initialize()

@@ -143,6 +143,35 @@ class ConvGemm:
             f32(bn_gamma), f32(bn_beta), bool(relu), ws, ws_bytes, stream_ptr()), "sconvGemmNHWC")
         return biases
 
+    def conv_gemm_pair_nhwc(self, weights, x, weights2, vpadding=0, hpadding=0, vstride=1, hstride=1, vdilation=1,
+                            hdilation=1, biases_vector=None, bn_running_mean=None, bn_inv_std=None, bn_gamma=None,
+                            bn_beta=None, relu=False, biases_vector2=None, bn_running_mean2=None, bn_inv_std2=None,
+                            bn_gamma2=None, bn_beta2=None, relu2=False, residual=None, relu_after_residual=False):
+        """Not in the reference: ``conv_gemm_nhwc`` with the first set of arguments followed by a 1 x 1 convolution
+        with ``weights2`` (kn, 1, 1, kn2) and the second set, as one launch that never stores the tensor between
+        them (the 3 x 3 and the last 1 x 1 layer of a ResNet bottleneck after the fusion pass, with the block's sum
+        and ReLU).  Returns the output, or None when the library is not built for the shapes: the caller then makes
+        the two calls, which give the same bits."""
+        b, h, w, c = x.shape
+        ck, kh, kw, kn = weights.shape
+        c2, kh2, kw2, kn2 = weights2.shape
+        if (ck, c2, kh2, kw2) != (c, kn, 1, 1) or x.dtype != torch.float32:
+            return None
+        ho = (h + 2 * vpadding - vdilation * (kh - 1) - 1) // vstride + 1
+        wo = (w + 2 * hpadding - hdilation * (kw - 1) - 1) // hstride + 1
+        y = torch.empty((b, ho, wo, kn2), dtype=x.dtype, device=x.device)
+        if residual is not None:
+            self._check_residual(residual, y, False, None)
+        rc = lib().pydtnn_hip_sconvGemm_pair_nhwc(
+            b, h, w, c, kn, kh, kw, vpadding, hpadding, vstride, hstride, vdilation, hdilation, f32(weights), f32(x),
+            f32(biases_vector), f32(bn_running_mean), f32(bn_inv_std), f32(bn_gamma), f32(bn_beta), bool(relu), kn2,
+            f32(weights2), f32(y), f32(biases_vector2), f32(bn_running_mean2), f32(bn_inv_std2), f32(bn_gamma2),
+            f32(bn_beta2), bool(relu2), f32(residual), bool(relu_after_residual), stream_ptr())
+        if rc == native.PYDTNN_HIP_ERR_UNSUPPORTED:
+            return None
+        check(rc, "sconvGemm_pair_nhwc")
+        return y
+
     @staticmethod
     def _check_relu_mask(relu_mask, out, trans, relu, bn_running_mean):
         assert not trans and relu and bn_running_mean is None, \

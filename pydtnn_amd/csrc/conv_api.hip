@@ -1,6 +1,7 @@
 // Device-pointer C ABI: argument checks, batching over image groups, and the launches that are not
 // convolutions (GEMM, explicit-path GEMMs, streaming kernels).
 #include "conv_internal.h"
+#include "conv_pair.h"
 #include "../../include/pydtnn_hip_test.h"
 #include <mutex>
 #include <new>
@@ -408,6 +409,31 @@ int pydtnn_hip_sconvGemmNHWC_back(unsigned b, unsigned h, unsigned w, unsigned c
                                   const float* dy, float* dx, void* workspace, size_t workspace_bytes, void* stream)
 {
     return conv_dx_batched(1, GEOM_ARGS, weights, dy, dx, (float*)workspace, workspace_bytes, as_stream(stream));
+}
+
+// ---------------------------------------------------------------- two convolutions of a bottleneck in one launch
+int pydtnn_hip_sconvGemm_pair_nhwc(unsigned b, unsigned h, unsigned w, unsigned c, unsigned kn, unsigned kh, unsigned kw,
+                                   unsigned vpadding, unsigned hpadding, unsigned vstride, unsigned hstride,
+                                   unsigned vdilation, unsigned hdilation, const float* weights, const float* x,
+                                   const float* bias_vector, const float* bn_running_mean, const float* bn_inv_std,
+                                   const float* bn_gamma, const float* bn_beta, bool relu, unsigned kn2,
+                                   const float* weights2, float* y, const float* bias_vector2,
+                                   const float* bn_running_mean2, const float* bn_inv_std2, const float* bn_gamma2,
+                                   const float* bn_beta2, bool relu2, const float* residual, bool relu_after_add,
+                                   void* stream)
+{
+    if (!weights || !x || !weights2 || !y) return PYDTNN_HIP_ERR_INVALID;
+    if (!bn_args_consistent(bn_running_mean, bn_inv_std, bn_gamma, bn_beta) ||
+        !bn_args_consistent(bn_running_mean2, bn_inv_std2, bn_gamma2, bn_beta2))
+        return PYDTNN_HIP_ERR_INVALID;
+    if (kn2 == 0 || kn2 >= (1u << 24)) return PYDTNN_HIP_ERR_INVALID;
+    ConvGeom g;
+    const int rc = geom_from_args(&g, GEOM_ARGS);
+    if (rc != PYDTNN_HIP_OK) return rc;
+    const ChanEpilogue chan1 = make_chan(bias_vector, bn_running_mean, bn_inv_std, bn_gamma, bn_beta, relu ? 1 : 0);
+    const ChanEpilogue chan2 = make_chan(bias_vector2, bn_running_mean2, bn_inv_std2, bn_gamma2, bn_beta2, relu2 ? 1 : 0);
+    const ElemMasks masks = {nullptr, nullptr, residual, relu_after_add ? 1 : 0};
+    return conv_stream_pair(g, (int)kn2, weights, weights2, x, y, chan1, chan2, masks, as_stream(stream));
 }
 
 // ---------------------------------------------------------------- a forward call with its arguments bound

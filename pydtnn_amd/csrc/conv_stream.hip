@@ -25,6 +25,7 @@
 //     bound by memory, and the end of what the previous kernel wrote (or read) is still in the memory-side cache.
 // The store applies bias -> BN -> ReLU and one of: gate, ReLU mask, residual (+ ReLU), like the tile engine's.
 #include "conv_internal.h"
+#include "conv_pair.h"
 #include <mutex>
 #include <type_traits>
 
@@ -372,7 +373,9 @@ std::mutex walks_mutex;
 StreamWalks stream_walks[8];
 int next_stream_slot = 0;
 
-int choose_direction(hipStream_t stream, const void* x, const void* residual, const void* y)
+}  // namespace
+
+int conv_stream_choose_direction(hipStream_t stream, const void* x, const void* residual, const void* y)
 {
     std::lock_guard<std::mutex> lock(walks_mutex);
     StreamWalks* sw = nullptr;
@@ -407,8 +410,6 @@ int choose_direction(hipStream_t stream, const void* x, const void* residual, co
     return reverse;
 }
 
-}  // namespace
-
 // Shapes the streaming kernel takes: the filter matrix fits LDS, channels come in chunks of 64 floats that
 // 128-bit loads can fetch, and there is enough work for every compute unit.
 bool conv_stream_nhwc_eligible(const ConvGeom& g, const float* w, const float* x)
@@ -429,7 +430,7 @@ int conv_stream_nhwc(const ConvGeom& g, const float* w, const float* x, float* y
     a.cchunks = g.c / 64;
     a.chunks = g.khw * a.cchunks;
     a.row_blocks = (int)(g.p / 32);
-    a.reverse = choose_direction(stream, x, masks.residual, y);
+    a.reverse = conv_stream_choose_direction(stream, x, masks.residual, y);
 #define STREAM_CASE(KN, CH) \
     if (g.kn == KN && a.chunks == CH) return launch_stream_masks<KN, CH>(a, stream)
     STREAM_CASE(64, 1); STREAM_CASE(64, 2); STREAM_CASE(64, 4); STREAM_CASE(64, 9);

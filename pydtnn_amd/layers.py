@@ -854,6 +854,22 @@ class _FusedConv(Conv2D, _FromParents):
     # the sum of an addition block (and the Relu after it) can ride in this layer's store
     accepts_residual = True
 
+    def forward_with_next(self, nxt, x, residual=None, relu_after_residual=False):
+        """This layer followed by the 1 x 1 fused layer ``nxt`` as one launch (NHWC, the shapes the library builds it
+        for), or None: the caller then runs the two layers one after the other, with the same bits."""
+        if self.model.mode != EVALUATE_MODE or self.model.tensor_format == PYDTNN_TENSOR_FORMAT_NCHW or \
+                getattr(self, "_no_pair", False) or not isinstance(nxt, _FusedConv) or \
+                (nxt.kh, nxt.kw, nxt.vstride, nxt.hstride, nxt.vpadding, nxt.hpadding) != (1, 1, 1, 1, 0, 0):
+            return None
+        e1, e2 = self._epilogue_kwargs(), nxt._epilogue_kwargs()
+        second = {k + "2": e2[k] for k in ("biases_vector", "relu", "bn_running_mean", "bn_inv_std", "bn_gamma", "bn_beta")
+                  if k in e2}
+        y = self.cg.conv_gemm_pair_nhwc(self.weights, x, nxt.weights, residual=residual,
+                                        relu_after_residual=relu_after_residual, **e1, **second)
+        if y is None:
+            self._no_pair = True      # not a shape the fused launch is built for: do not ask again
+        return y
+
     def backward(self, x):
         raise RuntimeError(f"Backward method of {self.__class__.__name__} should not be called")
 
@@ -913,10 +929,21 @@ class AdditionBlock(Layer):
             for layer in self.paths[1 - k]:
                 other = layer.forward(other)
             cur = x
-            for layer in self.paths[k][:-1]:
-                cur = layer.forward(cur)
+            path = self.paths[k]
             relu = self.relu_above is not None
-            y = self.paths[k][-1].forward(cur, residual=other, relu_after_residual=relu)
+            y = None
+            if len(path) >= 2 and getattr(path[-2], "accepts_residual", False):
+                # the path's last two convolutions in one launch where the library has one
+                for layer in path[:-2]:
+                    cur = layer.forward(cur)
+                y = path[-2].forward_with_next(path[-1], cur, residual=other, relu_after_residual=relu)
+                if y is None:
+                    cur = path[-2].forward(cur)
+            else:
+                for layer in path[:-1]:
+                    cur = layer.forward(cur)
+            if y is None:
+                y = path[-1].forward(cur, residual=other, relu_after_residual=relu)
             if relu:
                 self.relu_above.take_folded(y, None)
             return y

@@ -43,6 +43,8 @@ SIGNATURES = {
     "pydtnn_hip_sconvGemmNHWC": (_c.c_int, [_c.c_char] + _geom13_u + [_f32p] * 8 + [_c.c_bool, _vp, _c.c_size_t, _vp]),
     "pydtnn_hip_sconvGemmNCHW_back": (_c.c_int, _geom13_u + [_f32p] * 3 + [_vp, _c.c_size_t, _vp]),
     "pydtnn_hip_sconvGemmNHWC_back": (_c.c_int, _geom13_u + [_f32p] * 3 + [_vp, _c.c_size_t, _vp]),
+    "pydtnn_hip_sconvGemm_pair_nhwc": (_c.c_int, _geom13_u + [_f32p] * 7 + [_c.c_bool, _c.c_uint] + [_f32p] * 7 +
+                                       [_c.c_bool, _f32p, _c.c_bool, _vp]),
     "pydtnn_hip_conv_plan_create": (_c.c_int, [_c.POINTER(_c.c_void_p), _c.c_int] + _geom13_i + [_f32p] * 6 + [_c.c_bool]),
     "pydtnn_hip_conv_plan_forward": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_size_t,
                                                 _c.c_void_p]),

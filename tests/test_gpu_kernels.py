@@ -1162,3 +1162,53 @@ def test_libconvgemm_compat_abi_runs_like_the_reference_shim(oracle):
     libc = ctypes.CDLL("libc.so.6")
     libc.free(ac)
     libc.free(bc)
+
+
+# ------------------------------------------------------------------ two convolutions of a bottleneck in one launch
+@pytest.mark.parametrize("kn2,with_bias,residual,relu_after", [(256, True, True, True), (256, False, True, False),
+                                                               (128, True, False, False), (64, False, True, True)])
+@pytest.mark.parametrize("d", [D(16, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1, 1, 1), D(34, 64, 32, 31, 64, 3, 3, 1, 1, 1, 1, 1, 1)],
+                         ids=repr)
+def test_fused_pair_of_bottleneck_convolutions_equals_the_two_launches(ops, cg, oracle, d, kn2, with_bias, residual,
+                                                                        relu_after):
+    """3x3 (64 -> 64) + BN + ReLU followed by 1x1 (64 -> kn2) + BN (+ residual, + ReLU) as one launch: bit for bit
+    the result of the two launches it replaces, and within 1e-4 of the oracle's chain of separate passes
+    (pydtnn/backends/cpu/layers/conv_2d_batch_normalization_relu_cpu.py:79-94, addition_block_cpu.py:34-46).  The
+    second shape has an odd number of pixel blocks per compute unit and images whose rows do not align with them;
+    both directions of the walk are taken (the call is repeated on the same tensors)."""
+    announce("fused pair", d, kn2, with_bias, residual, relu_after)
+    assert (d.b * d.ho * d.wo) % 32 == 0 and d.b * d.ho * d.wo >= 32768
+    x, w, b, _ = case(d)
+    rng = np.random.default_rng(21)
+    w2 = (rng.standard_normal((64, 1, 1, kn2)) * np.sqrt(2.0 / 64)).astype(np.float32)
+    b2 = rng.standard_normal(kn2).astype(np.float32)
+    bn1 = [rng.uniform(0.5, 1.5, 64).astype(np.float32) for _ in range(4)]
+    bn2 = [rng.uniform(0.5, 1.5, kn2).astype(np.float32) for _ in range(4)]
+    xr, wr = nhwc(x), w_nhwc(w)
+    res_np = rng.standard_normal((d.b, d.ho, d.wo, kn2)).astype(np.float32)
+    xd, wd, w2d, res = dev(xr), dev(wr), dev(w2), dev(res_np) if residual else None
+    e1 = dict(biases_vector=dev(b) if with_bias else None, bn_running_mean=dev(bn1[0]), bn_inv_std=dev(bn1[1]),
+              bn_gamma=dev(bn1[2]), bn_beta=dev(bn1[3]), relu=True)
+    e2 = dict(biases_vector=dev(b2) if with_bias else None, bn_running_mean=dev(bn2[0]), bn_inv_std=dev(bn2[1]),
+              bn_gamma=dev(bn2[2]), bn_beta=dev(bn2[3]))
+    mid = cg.conv_gemm_nhwc(wd, xd, **e1, **_kw(d))
+    two = cg.conv_gemm_nhwc(w2d, mid, residual=res, relu_after_residual=relu_after, **e2)
+    for rep in range(3):
+        one = cg.conv_gemm_pair_nhwc(wd, xd, w2d, residual=res, relu_after_residual=relu_after, **e1, **_kw(d),
+                                     **{k + "2": v for k, v in e2.items()})
+        assert one is not None, "the library refused a shape it is built for"
+        assert torch.equal(one, two), f"fused launch differs from the two launches (repetition {rep})"
+    p = oracle.ConvParams(*d.geom())
+    y1, _ = oracle.conv2d_forward_nhwc_i2c(xr, wr, b if with_bias else None, p)
+    y1 = oracle.fused_epilogue(y1, "NHWC", bn=bn1, relu_flag=True)
+    y2, _ = oracle.conv2d_forward_nhwc_i2c(y1, w2, b2 if with_bias else None, oracle.ConvParams(1, 1))
+    y2 = oracle.fused_epilogue(y2, "NHWC", bn=bn2, relu_flag=False)
+    if residual:
+        y2 = oracle.eltw_sum(np.ascontiguousarray(y2), res_np)
+    if relu_after:
+        y2, _ = oracle.relu(y2)
+    assert_close(host(two), y2, what="fused pair vs oracle")
+    # shapes it is not built for are declined, not computed wrongly
+    assert cg.conv_gemm_pair_nhwc(wd, xd, dev(np.zeros((64, 1, 1, 320), np.float32)), **e1, **_kw(d),
+                                  bn_running_mean2=dev(np.zeros(320, np.float32)), bn_inv_std2=dev(np.ones(320, np.float32)),
+                                  bn_gamma2=dev(np.ones(320, np.float32)), bn_beta2=dev(np.zeros(320, np.float32))) is None
