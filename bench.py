@@ -27,11 +27,28 @@ HBM_PEAK_GBS = 8000.0
 
 # HBM-side bytes per launch of the forward kernel, from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE), each
 # scaled by what the same counter reads for a 256 MiB copy (factors 2.000 and 1.000):
-# main launch (166125.0 * 2.0 + 262144.0) KiB plus the fixup launch of its cut tiles (32822.9 * 2.0 + 4096.0) KiB.
-# The summary of those runs is profiles/cfg2_conv3x3_pmc_counters.md.
-TRAFFIC_SOURCE = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in profiles/cfg2_conv3x3_pmc_counters.md "
-                  "(a constant read off that profile, not measured by this run)")
-MEASURED_TRAFFIC_BYTES = {"cfg2": int((166061.8 * 2.0 + 262144.0 + 32825.6 * 2.0 + 4096.0) * 1024)}
+# main launch (166061.8 * 2.0 + 262144.0) KiB plus the fixup launch of its cut tiles (32825.6 * 2.0 + 4096.0) KiB.
+# The figure belongs to one launch form of one build: `launch` is what pydtnn_hip_debug_last_launch reported for
+# the forward call in the profiled runs and `commit` the source revision they were built from.  A run whose
+# forward call launches anything else reports traffic null instead of this constant.
+TRAFFIC_PROFILE = {
+    "file": "profiles/cfg2_conv3x3_pmc_counters.md",
+    "commit": "16e4579",
+    "launch": {"kind": "balanced", "tile": [256, 128], "workgroups": 512, "cut_tiles": 32, "splits": 1},
+    "bytes": int((166061.8 * 2.0 + 262144.0 + 32825.6 * 2.0 + 4096.0) * 1024),
+}
+
+
+def traffic_of_forward(launch):
+    """(traffic, traffic_source) of the roofline object: the profiled constant when this run's forward call took
+    the profiled launch form, else null with the reason."""
+    if launch == TRAFFIC_PROFILE["launch"]:
+        return TRAFFIC_PROFILE["bytes"], (
+            f"rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of commit {TRAFFIC_PROFILE['commit']} summarised in "
+            f"{TRAFFIC_PROFILE['file']} (a constant read off that profile, not measured by this run; this run's "
+            f"forward call took the profiled launch form {launch})")
+    return None, (f"none: this run's forward call launched {launch}, the counters in {TRAFFIC_PROFILE['file']} were "
+                  f"collected for {TRAFFIC_PROFILE['launch']}")
 
 
 def parse_args():
@@ -158,6 +175,9 @@ def run_cfg2(torch, pd, args):
         timers["dx"](conv.cg.deconv_gemm_nchw, conv.weights, dyd, dx, **kw)
 
     ms, timers = timed_steps(torch, step, args.steps, args.warmup)
+    from pydtnn_amd import native
+    conv.cg.conv_gemm_nchw(conv.weights, xd, biases=None, biases_vector=conv.biases, **conv._cg_kwargs())
+    fwd_launch = native.last_launch()
     gemm_flop = 2.0 * 256 * 2304 * n * 56 * 56
     step_flop = 3 * gemm_flop
     fwd_ms = timers["fwd"].mean_ms()
@@ -173,7 +193,6 @@ def run_cfg2(torch, pd, args):
     }
     # explicit-path streams: bytes(x) + bytes(cols) and bytes(cols) + bytes(dx).  The C ABI is called on buffers
     # allocated once, so that no allocation falls between a pair of timing events.
-    from pydtnn_amd import native
     from pydtnn_amd.native import check, f32, lib, stream_ptr
     geom = (3, 3, 1, 1, 1, 1, 1, 1)
     mat = torch.empty(256 * 9 * n * 56 * 56, device="cuda")   # x_cols (K x P) or x_rows (P x K)
@@ -251,10 +270,14 @@ def run_cfg2(torch, pd, args):
     extra.update(compat_route(x, w, b, gemm_flop))
     del xd, dyd
     extra.update(f64_route(torch, gemm_flop))
-    roofline = {"bound": "mfma", "kernel": "gemm_streamk_kernel_big_tile<256x128, PlainK4, Im2colNchwMN, EpiNchw> + streamk_fixup_kernel (forward)",
+    traffic, traffic_source = traffic_of_forward(fwd_launch)
+    profiled = fwd_launch == TRAFFIC_PROFILE["launch"]
+    roofline = {"bound": "mfma",
+                "kernel": ("gemm_streamk_kernel_big_tile<256x128, PlainK4, Im2colNchwMN, EpiNchw> + streamk_fixup_kernel "
+                           "(forward)") if profiled else f"the forward call's launch: {fwd_launch}",
                 "achieved": round(achieved, 3), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES["cfg2"],
-                "traffic_source": TRAFFIC_SOURCE}
+                "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": traffic,
+                "traffic_source": traffic_source, "launch": fwd_launch}
     workload = ("cfg2: VGG16-style 3x3 conv layer fwd+dW+db+dX, fp32 NCHW, N=64, 256->256, 56x56, stride 1, pad 1, "
                 "implicit GEMM")
     return ms, step_flop / (ms * 1e-3) / 1e9, workload, roofline, extra

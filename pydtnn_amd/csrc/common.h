@@ -130,6 +130,20 @@ __device__ __forceinline__ float elem_masks_apply(const ElemMasks& mk, long i, f
     return v;
 }
 
+// The form of the calling thread's most recent GEMM or streaming-convolution launch, kept for the test-only
+// query pydtnn_hip_debug_last_launch: a benchmark that quotes counters taken for one kernel form checks with it
+// that the library still picks that form.
+enum { kLaunchNone = 0, kLaunchTiles = 1, kLaunchBalanced = 2, kLaunchStreamNhwc = 3, kLaunchStreamNchw = 4,
+       kLaunchPair = 5 };
+struct LaunchNote {
+    int kind, tile_m, tile_n, workgroups, cut_tiles, splits;
+};
+inline thread_local LaunchNote g_last_launch = {};
+inline void note_launch(int kind, int tile_m, int tile_n, long workgroups, int cut_tiles, int splits)
+{
+    g_last_launch = LaunchNote{kind, tile_m, tile_n, (int)workgroups, cut_tiles, splits};
+}
+
 #define HIP_RETURN_IF_LAUNCH_FAILED()                         \
     do {                                                      \
         hipError_t e__ = hipGetLastError();                   \

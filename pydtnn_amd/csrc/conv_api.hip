@@ -256,6 +256,12 @@ long pydtnn_hip_debug_set_tensor_floats_limit(long floats)
     return before;
 }
 
+void pydtnn_hip_debug_last_launch(int out[6])
+{
+    const LaunchNote n = g_last_launch;
+    out[0] = n.kind; out[1] = n.tile_m; out[2] = n.tile_n; out[3] = n.workgroups; out[4] = n.cut_tiles; out[5] = n.splits;
+}
+
 int pydtnn_hip_version(void) { return 10000 * 0 + 100 * 1 + 0; }
 
 const char* pydtnn_hip_status_string(int status)

@@ -329,6 +329,7 @@ int launch_stream(const StreamArgs& a, hipStream_t stream)
     const int grid = a.row_blocks < cus ? a.row_blocks : cus;
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(64 * stream_waves(CHUNKS, MASKS)), lds_bytes, stream, a);
     HIP_RETURN_IF_LAUNCH_FAILED();
+    note_launch(kLaunchStreamNhwc, 32, N, grid, 0, 1);
     return PYDTNN_HIP_OK;
 }
 

@@ -333,6 +333,7 @@ int launch_stream_nchw_waves(const StreamNchwArgs& a, int grid, hipStream_t stre
     if (rc != PYDTNN_HIP_OK) return rc;
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(64 * WAVES), lds_bytes, stream, a);
     HIP_RETURN_IF_LAUNCH_FAILED();
+    note_launch(kLaunchStreamNchw, MB, 32, grid, 0, 1);
     return PYDTNN_HIP_OK;
 }
 

@@ -359,6 +359,7 @@ int launch_pair(const PairArgs& a, hipStream_t stream)
     const int grid = a.row_blocks < cus ? a.row_blocks : cus;
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kPairThreads), lds_bytes, stream, a);
     HIP_RETURN_IF_LAUNCH_FAILED();
+    note_launch(kLaunchPair, 32, kN1, grid, 0, 1);
     return PYDTNN_HIP_OK;
 }
 

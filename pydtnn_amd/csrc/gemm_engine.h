@@ -1496,6 +1496,7 @@ inline int launch(const AL& al, const BL& bl, const EP& ep, long m, long n, cons
         hipLaunchKernelGGL((gemm_kernel_large_state<T, AL, BL, EP>), grid, dim3(kThreads), 0, stream, al, bl, ep,
                            (int)tiles_m, si);
     HIP_RETURN_IF_LAUNCH_FAILED();
+    note_launch(kLaunchTiles, T::BM, T::BN, tiles_m * tiles_n * splits, 0, splits);
     return PYDTNN_HIP_OK;
 }
 
@@ -1752,6 +1753,7 @@ inline int launch_balanced(const AL& al, const BL& bl, const EP& ep, long m, lon
                            stream, ep, (int)tiles_m, sk);
         HIP_RETURN_IF_LAUNCH_FAILED();
     }
+    note_launch(kLaunchBalanced, T::BM, T::BN, resident, sk.sk_tiles, 1);
     return PYDTNN_HIP_OK;
 }
 

@@ -28,6 +28,7 @@ SIGNATURES = {
     "pydtnn_hip_version": (_c.c_int, []),
     "pydtnn_hip_status_string": (_c.c_char_p, [_c.c_int]),
     "pydtnn_hip_debug_set_tensor_floats_limit": (_c.c_long, [_c.c_long]),  # test-only (include/pydtnn_hip_test.h)
+    "pydtnn_hip_debug_last_launch": (None, [_c.POINTER(_c.c_int)]),  # test-only (include/pydtnn_hip_test.h)
     "pydtnn_hip_im2col_nchw": (_c.c_int, [_f32p, _f32p] + [_c.c_int] * 12 + [_vp]),
     "pydtnn_hip_col2im_nchw": (_c.c_int, [_f32p, _f32p] + [_c.c_int] * 12 + [_vp]),
     "pydtnn_hip_im2row_nhwc": (_c.c_int, [_f32p, _f32p] + [_c.c_int] * 12 + [_vp]),
@@ -196,6 +197,19 @@ def workspace(nbytes, dev=None, raw_stream=None):
 def workspace_buffer(key):
     """The tensor that currently backs the scratch buffer of ``key`` = (device index, raw stream handle), or None."""
     return _WORKSPACE.get(key)
+
+
+_LAUNCH_KINDS = ("none", "tiles", "balanced", "stream_nhwc", "stream_nchw", "pair")
+
+
+def last_launch():
+    """The form of this thread's most recent GEMM or streaming-convolution launch, as the library's test-only query
+    pydtnn_hip_debug_last_launch reports it (include/pydtnn_hip_test.h): benchmarks and tests that are about one
+    kernel form check with it that the library picked that form."""
+    out = (_c.c_int * 6)()
+    lib().pydtnn_hip_debug_last_launch(out)
+    return {"kind": _LAUNCH_KINDS[out[0]], "tile": [out[1], out[2]], "workgroups": out[3], "cut_tiles": out[4],
+            "splits": out[5]}
 
 
 _WORKSPACE_BYTES = {}

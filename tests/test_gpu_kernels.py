@@ -580,9 +580,11 @@ def test_dw_of_wide_filter_sets_takes_the_256x128_tiles(cg, oracle):
 
 
 def test_dw_with_many_tiles_takes_the_balanced_launch(cg, oracle):
-    """512 x 4608 filter matrix = 144 tiles: the reduction units of all tiles are dealt evenly over the chip and
-    pieces of a tile summed by the fixup kernel (NCHW); the result must not depend on that."""
-    for d in [D(4, 512, 8, 8, 512, 3, 3, 1, 1, 1, 1), D(6, 512, 14, 14, 512, 3, 3, 1, 1, 1, 1)]:
+    """448 x 4608 filter matrix = 126 tiles of 64 x 256 (a filter count that none of the longer tiles divides):
+    the reduction units of all tiles are dealt evenly over the chip and pieces of a tile summed by the fixup kernel
+    (NCHW); the library reports that form, and the result must not depend on it."""
+    from pydtnn_amd import native
+    for d in [D(4, 512, 8, 8, 448, 3, 3, 1, 1, 1, 1), D(6, 512, 14, 14, 448, 3, 3, 1, 1, 1, 1)]:
         announce("dw balanced", d)
         x, w, _, dy = case(d)
         p = oracle.ConvParams(*d.geom())
@@ -590,6 +592,8 @@ def test_dw_with_many_tiles_takes_the_balanced_launch(cg, oracle):
         dw_ref, _, _ = oracle.conv2d_backward_nchw_i2c(dy, x_cols, w, x.shape, p, need_dx=False)
         dw = torch.full(w.shape, float("nan"), device="cuda")
         cg.conv_gemm_nchw(dev(dy), dev(x), biases=dw, trans=True, **_kw(d))
+        form = native.last_launch()
+        assert form["kind"] == "balanced" and form["cut_tiles"] > 0, form
         assert_close(host(dw), dw_ref, what="dw nchw, balanced")
 
 
@@ -1176,6 +1180,7 @@ def test_fused_pair_of_bottleneck_convolutions_equals_the_two_launches(ops, cg, 
     (pydtnn/backends/cpu/layers/conv_2d_batch_normalization_relu_cpu.py:79-94, addition_block_cpu.py:34-46).  The
     second shape has an odd number of pixel blocks per compute unit and images whose rows do not align with them;
     both directions of the walk are taken (the call is repeated on the same tensors)."""
+    from pydtnn_amd.native import last_launch
     announce("fused pair", d, kn2, with_bias, residual, relu_after)
     assert (d.b * d.ho * d.wo) % 32 == 0 and d.b * d.ho * d.wo >= 32768
     x, w, b, _ = case(d)
@@ -1197,6 +1202,7 @@ def test_fused_pair_of_bottleneck_convolutions_equals_the_two_launches(ops, cg, 
         one = cg.conv_gemm_pair_nhwc(wd, xd, w2d, residual=res, relu_after_residual=relu_after, **e1, **_kw(d),
                                      **{k + "2": v for k, v in e2.items()})
         assert one is not None, "the library refused a shape it is built for"
+        assert last_launch()["kind"] == "pair"
         assert torch.equal(one, two), f"fused launch differs from the two launches (repetition {rep})"
     p = oracle.ConvParams(*d.geom())
     y1, _ = oracle.conv2d_forward_nhwc_i2c(xr, wr, b if with_bias else None, p)

@@ -6,6 +6,7 @@ equality, on two calls in a row with the second problem smaller than the first (
 first call's contents).
 """
 import ctypes
+import gc
 
 import numpy as np
 import pytest
@@ -42,6 +43,9 @@ def _call_pair(native, m, n, k, ta, tb, bias, relu, seed):
                                          stream)
         assert rc == 0, rc
         _call_pair.warmed = True
+    # tensors of earlier tests that only a collection of reference cycles frees must not be freed between the
+    # two readings
+    gc.collect()
     torch.cuda.synchronize()
     before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
     rc = lib.pydtnn_hip_sgemm_static(ta, tb, m, n, k, p(a_d), lda, p(b_d), ldb, p(c_st), n, p(bias_d), int(relu),
