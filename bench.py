@@ -27,15 +27,15 @@ HBM_PEAK_GBS = 8000.0
 
 # HBM-side bytes per launch of the forward kernel, from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE), each
 # scaled by what the same counter reads for a 256 MiB copy (factors 2.000 and 1.000):
-# main launch (166061.8 * 2.0 + 262144.0) KiB plus the fixup launch of its cut tiles (32825.6 * 2.0 + 4096.0) KiB.
+# main launch (166365.0 * 2.0 + 262144.0) KiB plus the fixup launch of its cut tiles (32825.7 * 2.0 + 4096.0) KiB.
 # The figure belongs to one launch form of one build: `launch` is what pydtnn_hip_debug_last_launch reported for
 # the forward call in the profiled runs and `commit` the source revision they were built from.  A run whose
 # forward call launches anything else reports traffic null instead of this constant.
 TRAFFIC_PROFILE = {
     "file": "profiles/cfg2_conv3x3_pmc_counters.md",
-    "commit": "16e4579",
+    "commit": "c763f5b",
     "launch": {"kind": "balanced", "tile": [256, 128], "workgroups": 512, "cut_tiles": 32, "splits": 1},
-    "bytes": int((166061.8 * 2.0 + 262144.0 + 32825.6 * 2.0 + 4096.0) * 1024),
+    "bytes": int((166365.0 * 2.0 + 262144.0 + 32825.7 * 2.0 + 4096.0) * 1024),
 }
 
 

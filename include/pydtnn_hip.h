@@ -363,8 +363,11 @@ int pydtnn_hip_sgd_momentum_multi(int count, float *const *w, const float *const
  * a @ b (pydtnn/utils/__init__.py:148-158); libconvGemm is float32 only (conv_gemm.py:101-107).  Same index
  * maps, summation orders and argument meaning as the float32 entry points of the same name.
  *   pydtnn_hip_dgemm: C = op(A) op(B) (+ bias[n], ReLU) on v_mfma_f64_16x16x4_f64, operands row-major or the
- *       transposed view of a row-major matrix; small C with a long reduction is split along k into
- *       `workspace` (pydtnn_hip_dgemm_workspace_bytes, 0 = not needed; then C must be dense, ldc == n).
+ *       transposed view of a row-major matrix.  `workspace` (pydtnn_hip_dgemm_workspace_bytes, 0 = not needed)
+ *       serves two cases: a small C with a long reduction is split along k into it (required then:
+ *       PYDTNN_HIP_ERR_WORKSPACE without it); a C of many tiles whose last round would leave most of the chip
+ *       idle gets those tiles from a second launch split along k (optional: without the workspace the call runs
+ *       the one grid of whole tiles).
  *   pydtnn_hip_transpose_1023_f64: dst[d1][d0][inner] = src[d0][d1][inner], the (co,N,ho,wo) <-> (N,co,ho,wo)
  *       copy of pydtnn/utils/best_transpose_1023.py:50-58.
  *   pydtnn_hip_bias_grad_f64: db[ch] = sum of dy over (outer, inner); needs no workspace.

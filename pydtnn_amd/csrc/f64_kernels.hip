@@ -33,6 +33,9 @@ struct Dgemm {
     int chunk;          // reduction elements per split (a multiple of 16)
     const double* bias; // per column, applied when splits == 1
     int relu;
+    int tiles_m;        // tiles along m; a workgroup's tile is blockIdx.x + tile0, m fastest
+    int tile0;
+    int compact;        // partial tiles go to c as [split][blockIdx.x][128][128] (the tail launch)
 };
 
 // element (row, kk) of op(A): A[row*lda + kk], or A[kk*lda + row] when transposed
@@ -55,8 +58,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     __shared__ double As[2][kBK64 * kPitch];
     __shared__ double Bs[2][kBK64 * kPitch];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int m0 = blockIdx.x * kBM, n0 = blockIdx.y * kBN;
-    const int split = blockIdx.z;
+    const int tile = (int)blockIdx.x + g.tile0;
+    const int m0 = (tile % g.tiles_m) * kBM, n0 = (tile / g.tiles_m) * kBN;
+    const int split = blockIdx.y;
     const int kbeg = split * g.chunk;
     const int kend = min(g.k, kbeg + g.chunk);
     const int wm0 = (wave & 1) * 64, wn0 = (wave >> 1) * 64;
@@ -115,6 +119,17 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
         buf ^= 1;
     }
 
+    if (g.compact) {
+        double* part = g.c + ((long)split * gridDim.x + blockIdx.x) * (kBM * kBN);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    part[(wm0 + i * 16 + 4 * v + fk) * kBN + wn0 + j * 16 + fi] = acc[i][j][v];
+        return;
+    }
     double* out = g.c + (long)split * g.m * g.ldc;  // split > 0 only with the workspace, whose ldc is n
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -150,9 +165,36 @@ __global__ void __launch_bounds__(256) dgemm_reduce_kernel(const double* ws, dou
     c[row * ldc + col] = s;
 }
 
+// The tiles of the tail launch: C[tile] = relu?(sum over splits of part[s][t] (+ bias[col])), ascending splits
+__global__ void __launch_bounds__(256) dgemm_tail_reduce_kernel(const double* ws, double* c, long ldc, int m, int n,
+                                                                int tiles_m, int tile0, int tail, int splits,
+                                                                const double* bias, int relu)
+{
+    const int t = blockIdx.x / (kBM * kBN / 256);
+    const int e = (blockIdx.x % (kBM * kBN / 256)) * 256 + threadIdx.x;
+    const int tile = tile0 + t;
+    const int row = (tile % tiles_m) * kBM + e / kBN, col = (tile / tiles_m) * kBN + e % kBN;
+    if (row >= m || col >= n) return;
+    double s = 0.0;
+    for (int z = 0; z < splits; ++z) s += ws[((long)z * tail + t) * (kBM * kBN) + e];
+    if (bias) s += bias[col];
+    if (relu) s = s > 0.0 ? s : 0.0;
+    c[(long)row * ldc + col] = s;
+}
+
+// What the chip holds at once: two workgroups on each of 256 compute units.
+constexpr long kDgemmResident = 512;
+
 struct DgemmPlan {
     int splits;
     int chunk;
+    // Many whole tiles: the grid runs as rounds of kDgemmResident tiles and a last, partly empty round costs as
+    // much as a full one (3136 tiles = 6.125 rounds take the time of 7).  The tiles of a last round that fills at
+    // most half the chip go to a second launch instead, split along k so that they fill it once, into a
+    // workspace of partial tiles that dgemm_tail_reduce_kernel sums.
+    int tail;          // tiles of the second launch (0: none)
+    int tail_splits;
+    int tail_chunk;
 };
 
 DgemmPlan plan_dgemm(long m, long n, long k)
@@ -166,7 +208,23 @@ DgemmPlan plan_dgemm(long m, long n, long k)
     DgemmPlan p;
     p.chunk = (int)chunk;
     p.splits = (int)((k + chunk - 1) / chunk);
+    p.tail = 0; p.tail_splits = 1; p.tail_chunk = p.chunk;
+    const long tail = tiles % kDgemmResident;
+    if (p.splits == 1 && tiles >= 2 * kDgemmResident && tail > 0 && 2 * tail <= kDgemmResident && k >= 512) {
+        long ts = kDgemmResident / tail;
+        if (ts > k / 256) ts = k / 256;
+        const long tc = ((k + ts - 1) / ts + 15) / 16 * 16;
+        p.tail = (int)tail;
+        p.tail_chunk = (int)tc;
+        p.tail_splits = (int)((k + tc - 1) / tc);
+    }
     return p;
+}
+
+size_t dgemm_plan_bytes(const DgemmPlan& p, long m, long n)
+{
+    if (p.splits > 1) return (size_t)p.splits * m * n * 8;
+    return (size_t)p.tail * p.tail_splits * kBM * kBN * 8;
 }
 
 // ---------------------------------------------------------------- streaming kernels
@@ -348,8 +406,7 @@ extern "C" {
 size_t pydtnn_hip_dgemm_workspace_bytes(long m, long n, long k)
 {
     if (m <= 0 || n <= 0 || k <= 0) return 0;
-    const DgemmPlan p = plan_dgemm(m, n, k);
-    return p.splits > 1 ? (size_t)p.splits * m * n * 8 : 0;
+    return dgemm_plan_bytes(plan_dgemm(m, n, k), m, n);
 }
 
 int pydtnn_hip_dgemm(int transa, int transb, long m, long n, long k, const double* a, long lda, const double* b,
@@ -360,12 +417,16 @@ int pydtnn_hip_dgemm(int transa, int transb, long m, long n, long k, const doubl
     const long lim = 1l << 31;
     if (m >= lim || n >= lim || k >= lim) return PYDTNN_HIP_ERR_UNSUPPORTED;
     if (lda < (transa ? m : k) || ldb < (transb ? k : n) || ldc < n) return PYDTNN_HIP_ERR_INVALID;
-    const DgemmPlan p = plan_dgemm(m, n, k);
+    DgemmPlan p = plan_dgemm(m, n, k);
     const long tiles_m = (m + kBM - 1) / kBM, tiles_n = (n + kBN - 1) / kBN;
-    if (tiles_n > 65535 || p.splits > 65535) return PYDTNN_HIP_ERR_UNSUPPORTED;
+    const long tiles = tiles_m * tiles_n;
+    if (tiles >= (1l << 31) || p.splits > 65535) return PYDTNN_HIP_ERR_UNSUPPORTED;
+    // the tail launch is an optimisation: without the workspace for it the one grid of whole tiles runs
+    if (p.tail > 0 && (!workspace || workspace_bytes < dgemm_plan_bytes(p, m, n))) p.tail = 0;
     Dgemm g;
     g.a = a; g.b = b; g.lda = lda; g.ldb = ldb; g.m = (int)m; g.n = (int)n; g.k = (int)k;
     g.transa = transa ? 1 : 0; g.transb = transb ? 1 : 0; g.chunk = p.chunk;
+    g.tiles_m = (int)tiles_m; g.tile0 = 0; g.compact = 0;
     if (p.splits > 1) {
         if (!workspace || workspace_bytes < (size_t)p.splits * m * n * 8) return PYDTNN_HIP_ERR_WORKSPACE;
         g.c = static_cast<double*>(workspace); g.ldc = n; g.bias = nullptr; g.relu = 0;
@@ -373,15 +434,29 @@ int pydtnn_hip_dgemm(int transa, int transb, long m, long n, long k, const doubl
         g.c = c; g.ldc = ldc; g.bias = bias; g.relu = relu ? 1 : 0;
     }
     const hipStream_t st = convint::as_stream(stream);
-    const dim3 grid((unsigned)tiles_m, (unsigned)tiles_n, (unsigned)p.splits);
-    if (g.transa && g.transb) hipLaunchKernelGGL((dgemm_kernel<true, true>), grid, dim3(256), 0, st, g);
-    else if (g.transa) hipLaunchKernelGGL((dgemm_kernel<true, false>), grid, dim3(256), 0, st, g);
-    else if (g.transb) hipLaunchKernelGGL((dgemm_kernel<false, true>), grid, dim3(256), 0, st, g);
-    else hipLaunchKernelGGL((dgemm_kernel<false, false>), grid, dim3(256), 0, st, g);
+    auto run = [&](const Dgemm& d, long count, int splits) {
+        const dim3 grid((unsigned)count, (unsigned)splits);
+        if (d.transa && d.transb) hipLaunchKernelGGL((dgemm_kernel<true, true>), grid, dim3(256), 0, st, d);
+        else if (d.transa) hipLaunchKernelGGL((dgemm_kernel<true, false>), grid, dim3(256), 0, st, d);
+        else if (d.transb) hipLaunchKernelGGL((dgemm_kernel<false, true>), grid, dim3(256), 0, st, d);
+        else hipLaunchKernelGGL((dgemm_kernel<false, false>), grid, dim3(256), 0, st, d);
+    };
+    run(g, tiles - p.tail, p.splits);
     HIP_RETURN_IF_LAUNCH_FAILED();
     if (p.splits > 1) {
         hipLaunchKernelGGL(dgemm_reduce_kernel, dim3(blocks_for(m * n)), dim3(256), 0, st,
                            static_cast<const double*>(workspace), c, ldc, m, (int)n, p.splits, bias, relu ? 1 : 0);
+        HIP_RETURN_IF_LAUNCH_FAILED();
+    }
+    if (p.tail > 0) {
+        Dgemm t = g;
+        t.c = static_cast<double*>(workspace); t.bias = nullptr; t.relu = 0;
+        t.tile0 = (int)(tiles - p.tail); t.compact = 1; t.chunk = p.tail_chunk;
+        run(t, p.tail, p.tail_splits);
+        HIP_RETURN_IF_LAUNCH_FAILED();
+        hipLaunchKernelGGL(dgemm_tail_reduce_kernel, dim3((unsigned)(p.tail * (kBM * kBN / 256))), dim3(256), 0, st,
+                           static_cast<const double*>(workspace), c, ldc, (int)m, (int)n, (int)tiles_m, t.tile0, p.tail,
+                           p.tail_splits, bias, relu ? 1 : 0);
         HIP_RETURN_IF_LAUNCH_FAILED();
     }
     return PYDTNN_HIP_OK;

@@ -56,7 +56,10 @@ def case64(d, seed=0):
 
 @pytest.mark.parametrize("m,n,k,ta,tb", [(130, 70, 96, 0, 0), (257, 129, 300, 1, 0), (64, 200, 1000, 0, 1),
                                           (5, 3, 17, 1, 1), (256, 2304, 9000, 0, 1), (64, 512, 4096, 0, 0),
-                                          (1000, 130, 64, 1, 0)])
+                                          (1000, 130, 64, 1, 0),
+                                          # 2 x 520 = 1040 tiles: two rounds of 512 and a tail of 16, which goes to
+                                          # the second launch (split in two along k); ragged last row and column tiles
+                                          (200, 66500, 520, 0, 0), (200, 66500, 520, 1, 1)])
 def test_dgemm_against_numpy(ops, m, n, k, ta, tb):
     announce("dgemm", m, n, k, ta, tb)
     rng = np.random.default_rng(m + n + k)
