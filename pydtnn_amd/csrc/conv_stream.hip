@@ -53,11 +53,14 @@ struct StreamArgs {
     int cchunks;         // c / 64
     int row_blocks;      // p / 32
     int reverse;         // workgroups and their units take the pixel blocks from the last to the first
+    int n_total;         // filters of the layer (SPLIT kernels: a workgroup computes N of them)
 };
 
 typedef float floatx4s __attribute__((ext_vector_type(4)));
 
-template <int N, int NB, int CHUNKS, int MASKS>
+// SPLIT: the layer has more filters than fit LDS beside each other (n_total = a multiple of N); workgroup b
+// computes filters (b % parts) * N .. + N - 1 of the pixel blocks of workgroup b / parts.
+template <int N, int NB, int CHUNKS, int MASKS, bool SPLIT = false>
 __global__ void __launch_bounds__(64 * stream_waves(CHUNKS, MASKS)) conv_stream_nhwc_kernel(StreamArgs a)
 {
     constexpr int kStreamWaves = stream_waves(CHUNKS, MASKS), kStreamThreads = 64 * kStreamWaves;
@@ -74,9 +77,13 @@ __global__ void __launch_bounds__(64 * stream_waves(CHUNKS, MASKS)) conv_stream_
     const int ln = lane & 31, lh = lane >> 5;
 
     // this workgroup's range of pixel blocks
-    const int wg = a.reverse ? (int)(gridDim.x - 1 - blockIdx.x) : (int)blockIdx.x;
-    const int rb0 = (int)((long)wg * a.row_blocks / gridDim.x);
-    const int rb1 = (int)((long)(wg + 1) * a.row_blocks / gridDim.x);
+    const int NT = SPLIT ? a.n_total : N;                  // row length of w, y and the side tensor
+    const int parts = SPLIT ? NT / N : 1;
+    const int wgs = (int)gridDim.x / parts, wgi = (int)blockIdx.x / parts;
+    const int nbase = SPLIT ? ((int)blockIdx.x - wgi * parts) * N : 0;
+    const int wg = a.reverse ? wgs - 1 - wgi : wgi;
+    const int rb0 = (int)((long)wg * a.row_blocks / wgs);
+    const int rb1 = (int)((long)(wg + 1) * a.row_blocks / wgs);
     const int units = (rb1 - rb0) * CG;
 
     // ---- set-up: filter matrix and per-channel parameters into LDS
@@ -94,7 +101,7 @@ __global__ void __launch_bounds__(64 * stream_waves(CHUNKS, MASKS)) conv_stream_
                 n4[u] = (qc - kk * (N / 4)) * 4;
                 const int t = kk / g.c, cc = kk - t * g.c;
                 kp[u] = q < quads ? kk : -1;
-                v[u] = w4[((size_t)(cc * g.khw + t) * N + n4[u]) / 4];  // the tensor's rows are (c, i, j)
+                v[u] = w4[((size_t)(cc * g.khw + t) * NT + nbase + n4[u]) / 4];  // the tensor's rows are (c, i, j)
             }
 #pragma unroll
             for (int u = 0; u < 6; ++u)
@@ -104,11 +111,11 @@ __global__ void __launch_bounds__(64 * stream_waves(CHUNKS, MASKS)) conv_stream_
                 }
         }
         for (int i = tid; i < N; i += kStreamThreads) {
-            params[i] = a.chan.bias ? a.chan.bias[i] : 0.0f;
-            params[N + i] = a.chan.mean ? a.chan.mean[i] : 0.0f;
-            params[2 * N + i] = a.chan.mean ? a.chan.inv_std[i] : 1.0f;
-            params[3 * N + i] = a.chan.mean ? a.chan.gamma[i] : 1.0f;
-            params[4 * N + i] = a.chan.mean ? a.chan.beta[i] : 0.0f;
+            params[i] = a.chan.bias ? a.chan.bias[nbase + i] : 0.0f;
+            params[N + i] = a.chan.mean ? a.chan.mean[nbase + i] : 0.0f;
+            params[2 * N + i] = a.chan.mean ? a.chan.inv_std[nbase + i] : 1.0f;
+            params[3 * N + i] = a.chan.mean ? a.chan.gamma[nbase + i] : 1.0f;
+            params[4 * N + i] = a.chan.mean ? a.chan.beta[nbase + i] : 0.0f;
         }
         if (tid == 0) *counter = kStreamWaves;  // the first unit of each wavefront is its own index
     }
@@ -117,7 +124,7 @@ __global__ void __launch_bounds__(64 * stream_waves(CHUNKS, MASKS)) conv_stream_
     const long x_floats = (long)g.n * g.c * g.h * g.w;
     const long lead = (long)(g.vpadding * g.w + g.hpadding) * g.c;  // keeps every lane's base offset >= 0
     const rsrc_t x_rsrc = make_rsrc(a.x - lead, x_floats + lead);
-    const long y_floats = g.p * N;
+    const long y_floats = g.p * NT;
     const rsrc_t y_rsrc = make_rsrc(a.y, y_floats);
     [[maybe_unused]] rsrc_t side_rsrc;  // gate bytes / mask bytes / residual floats, indexed like y
     if constexpr (MASKS == kGate) side_rsrc = make_rsrc_bytes(a.masks.gate, y_floats);
@@ -166,8 +173,8 @@ __global__ void __launch_bounds__(64 * stream_waves(CHUNKS, MASKS)) conv_stream_
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int row = 8 * (v / 4) + (v % 4);
-                const uint32_t e = (uint32_t)((4 * lh) * N + n0 + 32 * nb + ln);
-                const uint32_t soff = (uint32_t)(m0 + row) * N;
+                const uint32_t e = (uint32_t)((4 * lh) * NT + nbase + n0 + 32 * nb + ln);
+                const uint32_t soff = (uint32_t)(m0 + row) * NT;
                 if constexpr (MASKS == kResidual)
                     sd[nb][v] = buf_load(side_rsrc, live ? e * 4u : kOob, soff * 4u);
                 if constexpr (MASKS == kGate)
@@ -214,11 +221,11 @@ __global__ void __launch_bounds__(64 * stream_waves(CHUNKS, MASKS)) conv_stream_
                 mean = params[N + col]; inv_std = params[2 * N + col];
                 gamma = params[3 * N + col]; beta = params[4 * N + col];
             }
-            const uint32_t e = (uint32_t)((4 * lh) * N + col);
+            const uint32_t e = (uint32_t)((4 * lh) * NT + nbase + col);
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int row = 8 * (v / 4) + (v % 4);
-                const uint32_t soff = (uint32_t)(m0 + row) * N;
+                const uint32_t soff = (uint32_t)(m0 + row) * NT;
                 float val = ac[nb][v];
                 if constexpr ((F & kEpiBias) != 0) val += bias;
                 if constexpr ((F & kEpiBn) != 0) {
@@ -316,31 +323,36 @@ __global__ void __launch_bounds__(64 * stream_waves(CHUNKS, MASKS)) conv_stream_
     }
 }
 
-template <int N, int NB, int CHUNKS, int MASKS>
+template <int N, int NB, int CHUNKS, int MASKS, bool SPLIT = false>
 int launch_stream(const StreamArgs& a, hipStream_t stream)
 {
     static std::atomic<unsigned> raised{0};
     const size_t lds_bytes = ((size_t)a.g.k * N + 5 * N) * 4 + 16;
-    auto kernel = conv_stream_nhwc_kernel<N, NB, CHUNKS, MASKS>;
+    auto kernel = conv_stream_nhwc_kernel<N, NB, CHUNKS, MASKS, SPLIT>;
     int cus = 0;
     int rc = raise_lds_limit(reinterpret_cast<const void*>(kernel), raised, 160 * 1024);
     if (rc == PYDTNN_HIP_OK) rc = device_compute_units(&cus);
     if (rc != PYDTNN_HIP_OK) return rc;
-    const int grid = a.row_blocks < cus ? a.row_blocks : cus;
+    // one workgroup per compute unit; SPLIT: that many shared out between the parts of every pixel range
+    const int parts = SPLIT ? a.n_total / N : 1;
+    int ranges = cus / parts;
+    if (ranges > a.row_blocks) ranges = a.row_blocks;
+    if (ranges < 1) ranges = 1;
+    const int grid = ranges * parts;
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(64 * stream_waves(CHUNKS, MASKS)), lds_bytes, stream, a);
     HIP_RETURN_IF_LAUNCH_FAILED();
     note_launch(kLaunchStreamNhwc, 32, N, grid, 0, 1);
     return PYDTNN_HIP_OK;
 }
 
-template <int N, int CHUNKS>
+template <int N, int CHUNKS, bool SPLIT = false>
 int launch_stream_masks(const StreamArgs& a, hipStream_t stream)
 {
     switch (mask_kind(a.masks)) {
-    case kGate: return launch_stream<N, 2, CHUNKS, kGate>(a, stream);
-    case kReluMask: return launch_stream<N, 2, CHUNKS, kReluMask>(a, stream);
-    case kResidual: return launch_stream<N, 2, CHUNKS, kResidual>(a, stream);
-    default: return launch_stream<N, 2, CHUNKS, kNoMasks>(a, stream);
+    case kGate: return launch_stream<N, 2, CHUNKS, kGate, SPLIT>(a, stream);
+    case kReluMask: return launch_stream<N, 2, CHUNKS, kReluMask, SPLIT>(a, stream);
+    case kResidual: return launch_stream<N, 2, CHUNKS, kResidual, SPLIT>(a, stream);
+    default: return launch_stream<N, 2, CHUNKS, kNoMasks, SPLIT>(a, stream);
     }
 }
 
@@ -352,9 +364,12 @@ bool stream_shape_built(int kn, int chunks)
     case 64: return chunks == 1 || chunks == 2 || chunks == 4 || chunks == 9;
     case 128: return chunks == 1 || chunks == 2 || chunks == 4;
     case 256: return chunks == 1 || chunks == 2;
+    // more filters than fit LDS beside each other, in parts of 256 (a bottleneck's last 1x1 layer over 128 channels)
+    case 512: return chunks == 2;
     default: return false;
     }
 }
+constexpr int stream_part_filters(int kn) { return kn > 256 ? 256 : kn; }
 
 // The direction of a launch.  Per stream, the tensors the last few launches walked and the direction they walked
 // them in; a new launch goes the other way than the launch that last touched its residual (if it has one: that is
@@ -416,7 +431,7 @@ int conv_stream_choose_direction(hipStream_t stream, const void* x, const void* 
 bool conv_stream_nhwc_eligible(const ConvGeom& g, const float* w, const float* x)
 {
     if (g.c % 64 != 0 || !stream_shape_built(g.kn, g.khw * (g.c / 64))) return false;
-    if ((size_t)g.k * g.kn > kStreamMaxFilterFloats || g.khw > 31) return false;
+    if ((size_t)g.k * stream_part_filters(g.kn) > kStreamMaxFilterFloats || g.khw > 31) return false;
     if (!aligned16(w) || !aligned16(x)) return false;
     if (g.p < 32 * 1024 || g.p % 32 != 0) return false;
     return (long)g.n * g.c * g.h * g.w + (long)(g.vpadding * g.w + g.hpadding) * g.c < (1l << 29) &&
@@ -432,6 +447,8 @@ int conv_stream_nhwc(const ConvGeom& g, const float* w, const float* x, float* y
     a.chunks = g.khw * a.cchunks;
     a.row_blocks = (int)(g.p / 32);
     a.reverse = conv_stream_choose_direction(stream, x, masks.residual, y);
+    a.n_total = g.kn;
+    if (g.kn == 512 && a.chunks == 2) return launch_stream_masks<256, 2, true>(a, stream);
 #define STREAM_CASE(KN, CH) \
     if (g.kn == KN && a.chunks == CH) return launch_stream_masks<KN, CH>(a, stream)
     STREAM_CASE(64, 1); STREAM_CASE(64, 2); STREAM_CASE(64, 4); STREAM_CASE(64, 9);

@@ -38,6 +38,10 @@ stream_grid = [
     D(16, 64, 48, 48, 64, 3, 3, 2, 2, 1, 1, 2, 2),
     D(11, 128, 64, 64, 128, 1, 1, 0, 0, 1, 1, 1, 1),
     D(40, 64, 31, 33, 128, 2, 2, 1, 0, 1, 1, 1, 1),
+    # 512 filters over 128 channels: two workgroups per pixel range, 256 filters each (the second shape leaves the
+    # compute units pixel ranges of unequal length)
+    D(16, 128, 48, 48, 512, 1, 1, 0, 0, 1, 1, 1, 1),
+    D(13, 128, 56, 56, 512, 1, 1, 0, 0, 1, 1, 1, 1),
 ]
 
 
@@ -236,6 +240,8 @@ def test_streaming_kernel_shapes_nhwc(cg, oracle, d):
     y_ref, rows = oracle.conv2d_forward_nhwc_i2c(xr, wr, b, p)
     xd = dev(xr)
     y = cg.conv_gemm_nhwc(dev(wr), xd, biases_vector=dev(b), **_kw(d))
+    from pydtnn_amd.native import last_launch
+    assert last_launch()["kind"] == "stream_nhwc", last_launch()
     assert_close(host(y), y_ref, what="y")
     # the same input again: the kernel now walks the pixel blocks from the other end (it starts where the launch
     # that last touched its input ended), and once more the first way round; not a bit may change
@@ -255,7 +261,9 @@ def test_streaming_kernel_shapes_nhwc(cg, oracle, d):
 
 # one shape per chunk count the streaming kernel is built for (1, 2 and 4 chunks of 64 channels at 1x1, 9 at 3x3)
 stream_chunk_grid = [D(16, 64, 56, 56, 64, 1, 1, 0, 0, 1, 1, 1, 1), D(16, 128, 56, 56, 64, 1, 1, 0, 0, 1, 1, 1, 1),
-                     D(16, 256, 56, 56, 64, 1, 1, 0, 0, 1, 1, 1, 1), D(16, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1, 1, 1)]
+                     D(16, 256, 56, 56, 64, 1, 1, 0, 0, 1, 1, 1, 1), D(16, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1, 1, 1),
+                     # the form that splits 512 filters between two workgroups
+                     D(13, 128, 56, 56, 512, 1, 1, 0, 0, 1, 1, 1, 1)]
 
 
 @pytest.mark.parametrize("masks", ["none", "relu_mask", "residual", "gate"])
