@@ -367,7 +367,7 @@ int pydtnn_hip_sgd_momentum_multi(int count, float *const *w, const float *const
  *       serves two cases: a small C with a long reduction is split along k into it (required then:
  *       PYDTNN_HIP_ERR_WORKSPACE without it); a C of many tiles whose last round would leave most of the chip
  *       idle gets those tiles from a second launch split along k (optional: without the workspace the call runs
- *       the one grid of whole tiles).
+ *       the one grid of whole tiles).  lda, ldb < 2^22 (PYDTNN_HIP_ERR_UNSUPPORTED beyond).
  *   pydtnn_hip_transpose_1023_f64: dst[d1][d0][inner] = src[d0][d1][inner], the (co,N,ho,wo) <-> (N,co,ho,wo)
  *       copy of pydtnn/utils/best_transpose_1023.py:50-58.
  *   pydtnn_hip_bias_grad_f64: db[ch] = sum of dy over (outer, inner); needs no workspace.

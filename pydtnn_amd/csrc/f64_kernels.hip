@@ -38,18 +38,18 @@ struct Dgemm {
     int compact;        // partial tiles go to c as [split][blockIdx.x][128][128] (the tail launch)
 };
 
-// element (row, kk) of op(A): A[row*lda + kk], or A[kk*lda + row] when transposed
-template <bool TA>
-__device__ __forceinline__ double load_a(const Dgemm& g, int row, int kk, int kend)
+typedef unsigned int uintx2 __attribute__((ext_vector_type(2)));
+
+// A descriptor over "everything from p on": the loads below only use offsets of elements that exist (rows and
+// columns beyond the matrix are clamped, reduction indices beyond the chunk are not loaded), so no range check
+// is wanted from it.
+__device__ __forceinline__ gemm::rsrc_t open_rsrc(const double* p)
 {
-    if (row >= g.m || kk >= kend) return 0.0;
-    return TA ? g.a[(long)kk * g.lda + row] : g.a[(long)row * g.lda + kk];
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<double*>(p), 0, -1, 0x00020000);
 }
-template <bool TB>
-__device__ __forceinline__ double load_b(const Dgemm& g, int kk, int col, int kend)
+__device__ __forceinline__ double load64(gemm::rsrc_t r, uint32_t byte_offset)
 {
-    if (col >= g.n || kk >= kend) return 0.0;
-    return TB ? g.b[(long)col * g.ldb + kk] : g.b[(long)kk * g.ldb + col];
+    return __builtin_bit_cast(double, __builtin_amdgcn_raw_buffer_load_b64(r, (int)byte_offset, 0, 0));
 }
 
 template <bool TA, bool TB>
@@ -68,14 +68,41 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 
     // thread -> tile element maps for the global loads: lanes run along the operand's contiguous axis
     //   k contiguous: (kk = tid % 16, mn = tid / 16 + 16 e);  mn contiguous: (mn = tid % 128, kk = tid / 128 + 2 e)
+    // A step's elements are fetched with buffer loads from the step's corner of the operand (a scalar pointer
+    // that moves with k) at per-thread byte offsets that are computed once: no vector arithmetic per load.  Rows
+    // of A / columns of B beyond the matrix are clamped to the last one (they only feed rows / columns of C that
+    // are never stored); the one step that may reach beyond the chunk's end tests each element.
+    uint32_t offa[8], offb[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        if (TA) offa[e] = (uint32_t)(((long)((tid >> 7) + 2 * e) * g.lda + (min(m0 + (tid & 127), g.m - 1) - m0)) * 8);
+        else offa[e] = (uint32_t)(((long)(min(m0 + (tid >> 4) + 16 * e, g.m - 1) - m0) * g.lda + (tid & 15)) * 8);
+        if (TB) offb[e] = (uint32_t)(((long)(min(n0 + (tid >> 4) + 16 * e, g.n - 1) - n0) * g.ldb + (tid & 15)) * 8);
+        else offb[e] = (uint32_t)(((long)((tid >> 7) + 2 * e) * g.ldb + (min(n0 + (tid & 127), g.n - 1) - n0)) * 8);
+    }
     double ra[8], rb[8];
     auto fetch = [&](int k0) {
+        const gemm::rsrc_t wa = open_rsrc(TA ? g.a + (long)k0 * g.lda + m0 : g.a + (long)m0 * g.lda + k0);
+        const gemm::rsrc_t wb = open_rsrc(TB ? g.b + (long)n0 * g.ldb + k0 : g.b + (long)k0 * g.ldb + n0);
+        if (k0 + kBK64 <= kend) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            if (TA) ra[e] = load_a<TA>(g, m0 + (tid & 127), k0 + (tid >> 7) + 2 * e, kend);
-            else ra[e] = load_a<TA>(g, m0 + (tid >> 4) + 16 * e, k0 + (tid & 15), kend);
-            if (TB) rb[e] = load_b<TB>(g, k0 + (tid & 15), n0 + (tid >> 4) + 16 * e, kend);
-            else rb[e] = load_b<TB>(g, k0 + (tid >> 7) + 2 * e, n0 + (tid & 127), kend);
+            for (int e = 0; e < 8; ++e) {
+                ra[e] = load64(wa, offa[e]);
+                rb[e] = load64(wb, offb[e]);
+            }
+        } else {
+            // the reduction index of element e within the step, and the element's offset with that index set to 0
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int ka = TA ? (tid >> 7) + 2 * e : (tid & 15);
+                const int kb = TB ? (tid & 15) : (tid >> 7) + 2 * e;
+                const bool oka = k0 + ka < kend, okb = k0 + kb < kend;
+                const uint32_t za = offa[e] - (uint32_t)((TA ? (long)ka * g.lda : (long)ka) * 8);
+                const uint32_t zb = offb[e] - (uint32_t)((TB ? (long)kb : (long)kb * g.ldb) * 8);
+                const double va = load64(wa, oka ? offa[e] : za), vb = load64(wb, okb ? offb[e] : zb);
+                ra[e] = oka ? va : 0.0;
+                rb[e] = okb ? vb : 0.0;
+            }
         }
     };
     auto stash = [&](int buf) {
@@ -417,6 +444,8 @@ int pydtnn_hip_dgemm(int transa, int transb, long m, long n, long k, const doubl
     const long lim = 1l << 31;
     if (m >= lim || n >= lim || k >= lim) return PYDTNN_HIP_ERR_UNSUPPORTED;
     if (lda < (transa ? m : k) || ldb < (transb ? k : n) || ldc < n) return PYDTNN_HIP_ERR_INVALID;
+    // a thread's byte offsets inside a step's window of an operand (up to 128 rows) are 32-bit
+    if (lda >= (1l << 22) || ldb >= (1l << 22)) return PYDTNN_HIP_ERR_UNSUPPORTED;
     DgemmPlan p = plan_dgemm(m, n, k);
     const long tiles_m = (m + kBM - 1) / kBM, tiles_n = (n + kBN - 1) / kBN;
     const long tiles = tiles_m * tiles_n;
