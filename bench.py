@@ -511,7 +511,7 @@ def main():
         ms, value, workload, roofline, extra = run_cfg2(torch, pd, args)
         unit = "GFLOP/s"
         if not args.no_vgg16:
-            _, vgg = run_cfg5(torch, pd, args, steps=3, warmup=1)
+            _, vgg = run_cfg5(torch, pd, args, steps=6, warmup=2)
             extra.update(vgg)
         if not args.no_other_configs:
             from bench_configs import other_configs_extra
