@@ -416,9 +416,10 @@ int make_conv_geom(ConvGeom* g, int n, int c, int h, int w, int kn, int kh, int 
 int launch_im2col_nchw(const float* x, float* cols, const ConvGeom& g, hipStream_t stream)
 {
     const bool aligned = (reinterpret_cast<uintptr_t>(cols) & 15) == 0;
-    // Staged form: chunks of at most 1024 pixels, equal within an image and a multiple of 4 long.
+    // Staged form: chunks of at most 1024 pixels, about equal within an image and a multiple of 32 long, so that
+    // (with images that are a multiple of 32 pixels) every chunk's run of a matrix row starts on a 128-byte line.
     const int chunks = (g.howo + 1023) / 1024;
-    const int chunk_px = ((g.howo + chunks - 1) / chunks + 3) & ~3;
+    const int chunk_px = ((g.howo + chunks - 1) / chunks + 31) & ~31;
     const long rows_out = (chunk_px + g.wo - 2) / g.wo + 1;  // output rows a chunk can straddle
     const long rows_in = (long)g.vstride * (rows_out - 1) + (long)g.vdilation * (g.kh - 1) + 1;
     const long lds_bytes = (rows_in < g.h ? rows_in : g.h) * g.w * 4;
