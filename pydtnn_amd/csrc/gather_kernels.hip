@@ -208,8 +208,9 @@ __global__ void __launch_bounds__(kThreads) col2im_nchw_kernel(const float* __re
                 const bool ok =
                     out_coord<UNIT>(ww + g.hpadding - g.hdilation * jj, g.hstride, g.fd_hs, g.wo, &ox) && row_ok;
                 // (a streaming load here measured 4.57 against 5.17 TB/s: neighbouring rows of dx share lines of the
-                // matrix through the caches; four pixels per thread with unaligned 128-bit loads 5.09 against 5.24;
-                // planes taken with the image index fastest 5.13)
+                // matrix through the caches; four pixels per thread with unaligned 128-bit loads 5.09 against 5.24,
+                // with 36 scalar loads in flight over chunks of 800 pixels 4.80; planes taken with the image index
+                // fastest 5.13)
                 const float val = src[(long)(ii * kw + jj) * g.p + (ok ? oy * g.wo + ox : 0)];
                 acc += ok ? val : 0.0f;
             }
