@@ -1632,16 +1632,30 @@ __global__ void __launch_bounds__(kThreads) streamk_fixup_kernel(EP ep, int tile
     while (g + 1 < sk.sk_blocks && sk_first_unit(g + 1, total, sk.sk_blocks) <= a) ++g;
     if (sk_first_unit(g + 1, total, sk.sk_blocks) >= b) return;  // it held the whole tile and stored it
 
+    // The ranges of the workgroups are consecutive and none is empty, so the tile's pieces are those of the
+    // workgroups g .. g_last, one each; only the first can have begun before the tile did (it then lies in its
+    // workgroup's slot 1).  Eight pieces are requested at a time and added in ascending order.
+    int g_last = (int)((b * sk.sk_blocks - 1) / total);
+    while (g_last > g && sk_first_unit(g_last, total, sk.sk_blocks) >= b) --g_last;
+    while (g_last + 1 < sk.sk_blocks && sk_first_unit(g_last + 1, total, sk.sk_blocks) < b) ++g_last;
+    const int first_slot = sk_first_unit(g, total, sk.sk_blocks) < a ? 1 : 0;
+    const float* lane_base = sk.partial + quad * 4 * kThreads + tid;
     float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    for (; g < sk.sk_blocks; ++g) {
-        const long s0 = sk_first_unit(g, total, sk.sk_blocks), s1 = sk_first_unit(g + 1, total, sk.sk_blocks);
-        if (s0 >= b) break;
-        const long piece0 = s0 > a ? s0 : a, piece1 = s1 < b ? s1 : b;
-        if (piece1 <= piece0) continue;
-        const float* src =
-            sk.partial + (size_t)(2 * g + (piece0 == s0 ? 0 : 1)) * (T::BM * T::BN) + quad * 4 * kThreads + tid;
+    for (int g0 = g; g0 <= g_last; g0 += 8) {
+        float v[8][4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) acc[q] += src[q * kThreads];
+        for (int p = 0; p < 8; ++p) {
+            const int gg = g0 + p;
+            const float* src = lane_base + (size_t)(2 * gg + (gg == g ? first_slot : 0)) * (T::BM * T::BN);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) v[p][q] = gg <= g_last ? src[q * kThreads] : 0.0f;
+        }
+#pragma unroll
+        for (int p = 0; p < 8; ++p)
+            if (g0 + p <= g_last) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) acc[q] += v[p][q];
+            }
     }
     const int ij = quad >> 2, i = ij / T::TN, j = ij - i * T::TN, v0 = (quad & 3) * 4;
     const int wave = tid >> 6, lane = tid & 63;
