@@ -74,6 +74,22 @@ def test_workspace_queries_are_pure_host_code(native):
     assert lib.pydtnn_hip_conv_workspace_bytes(native.OP_DW, 0, 1, 1, 2, 2, 1, 5, 5, 0, 0, 1, 1, 1, 1) == 0
     assert lib.pydtnn_hip_sgemm_workspace_bytes(4096, 4096, 4096) == 0
     assert lib.pydtnn_hip_sgemm_workspace_bytes(64, 4096, 25088) > 0
+    # float64 GEMM: split along k for a small C with a long reduction; for a C of many tiles whose last round of
+    # the 512 resident workgroups is nearly empty (3136 tiles = 6.125 rounds) the partial tiles of the tail launch:
+    # 64 tiles x 8 chunks of k x 128 x 128 doubles; nothing for a C whose rounds come out even
+    assert lib.pydtnn_hip_dgemm_workspace_bytes(256, 2304, 200704) > 0
+    assert lib.pydtnn_hip_dgemm_workspace_bytes(256, 200704, 2304) == 64 * 8 * 128 * 128 * 8
+    assert lib.pydtnn_hip_dgemm_workspace_bytes(1024, 8192, 512) == 0
+
+
+def test_dgemm_refuses_leading_dimensions_its_offsets_cannot_hold(native):
+    """Argument checks only: the call returns before anything is launched."""
+    lib = native.lib()
+    one = ctypes.c_void_p(1)
+    args = lambda lda, ldb: (0, 0, 4, 4, 4, one, lda, one, ldb, one, 4, None, 0, None, 0, None)
+    assert lib.pydtnn_hip_dgemm(*args(1 << 22, 4)) == native.PYDTNN_HIP_ERR_UNSUPPORTED
+    assert lib.pydtnn_hip_dgemm(*args(4, 1 << 22)) == native.PYDTNN_HIP_ERR_UNSUPPORTED
+    assert lib.pydtnn_hip_dgemm(*args(3, 4)) == native.PYDTNN_HIP_ERR_INVALID      # lda < k
 
 
 def test_missing_library_is_an_import_error(native):

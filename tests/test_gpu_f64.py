@@ -59,7 +59,8 @@ def case64(d, seed=0):
                                           (1000, 130, 64, 1, 0),
                                           # 2 x 520 = 1040 tiles: two rounds of 512 and a tail of 16, which goes to
                                           # the second launch (split in two along k); ragged last row and column tiles
-                                          (200, 66500, 520, 0, 0), (200, 66500, 520, 1, 1)])
+                                          (200, 66500, 520, 0, 0), (200, 66500, 520, 1, 1),
+                                          (130, 66000, 530, 1, 0), (130, 66000, 530, 0, 1)])
 def test_dgemm_against_numpy(ops, m, n, k, ta, tb):
     announce("dgemm", m, n, k, ta, tb)
     rng = np.random.default_rng(m + n + k)
