@@ -858,7 +858,7 @@ class _FusedConv(Conv2D, _FromParents):
         """This layer followed by the 1 x 1 fused layer ``nxt`` as one launch (NHWC, the shapes the library builds it
         for), or None: the caller then runs the two layers one after the other, with the same bits."""
         if self.model.mode != EVALUATE_MODE or self.model.tensor_format == PYDTNN_TENSOR_FORMAT_NCHW or \
-                getattr(self, "_no_pair", False) or not isinstance(nxt, _FusedConv) or \
+                getattr(self, "_no_pair", None) == tuple(x.shape) or not isinstance(nxt, _FusedConv) or \
                 (nxt.kh, nxt.kw, nxt.vstride, nxt.hstride, nxt.vpadding, nxt.hpadding) != (1, 1, 1, 1, 0, 0):
             return None
         e1, e2 = self._epilogue_kwargs(), nxt._epilogue_kwargs()
@@ -867,7 +867,7 @@ class _FusedConv(Conv2D, _FromParents):
         y = self.cg.conv_gemm_pair_nhwc(self.weights, x, nxt.weights, residual=residual,
                                         relu_after_residual=relu_after_residual, **e1, **second)
         if y is None:
-            self._no_pair = True      # not a shape the fused launch is built for: do not ask again
+            self._no_pair = tuple(x.shape)      # not a shape the fused launch is built for: do not ask again
         return y
 
     def backward(self, x):
