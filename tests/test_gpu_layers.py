@@ -257,6 +257,52 @@ def test_residual_block_with_fusion(pd, oracle):
     assert_close(host(y_fused), ref, what="bottleneck vs oracle")
 
 
+@pytest.mark.parametrize("fmt", ["NCHW", "NHWC"])
+def test_block_of_one_convolution_adds_its_own_input(pd, oracle, fmt):
+    """An AdditionBlock whose one path is a single Conv2D + BN and whose other path is the identity: after the
+    fusion pass the convolution's store adds the residual, and the residual is the convolution's own input x
+    (the store reads a tile's residual before it writes the tile of y; x is only read).  Same bits as the separate
+    sum, x untouched, and the oracle's relu(x + bn(conv(x)))."""
+    announce("one-convolution block", fmt)
+    rng = np.random.default_rng(8)
+    c, hw, n = 12, 9, 4
+    shape = (c, hw, hw) if fmt == "NCHW" else (hw, hw, c)
+
+    model = pd.Model(tensor_format=fmt, enable_fused_conv_bn=True)
+    model.add(pd.Input(shape=(hw, hw, c)))                     # (h, w, c), encoded into the model's format
+    model.add(pd.AdditionBlock([pd.Conv2D(nfilters=c, filter_shape=(3, 3), padding=1), pd.BatchNormalization()], []))
+    model.add(pd.Relu())
+    conv, bn = [l for l in model.get_all_layers() if l.canonical_name in ("Conv2D", "BatchNormalization")]
+    conv.weights = dev((rng.standard_normal(tuple(conv.weights.shape)) * 0.3).astype(np.float32))
+    conv.biases = dev(rng.standard_normal(c).astype(np.float32))
+    bn.gamma, bn.beta = dev(rng.uniform(0.5, 1.5, c).astype(np.float32)), dev(rng.normal(0, 0.1, c).astype(np.float32))
+    bn.running_mean = dev(rng.normal(0, 0.1, c).astype(np.float32))
+    bn.running_var = dev(rng.uniform(0.5, 1.5, c).astype(np.float32))
+    bn.updated_running_var = True
+    w_h, b_h = host(conv.weights), host(conv.biases)
+    bn_h = (host(bn.running_mean), (1.0 / np.sqrt(host(bn.running_var) + np.float32(bn.epsilon))).astype(np.float32),
+            host(bn.gamma), host(bn.beta))
+    x = rng.standard_normal((n,) + shape).astype(np.float32)
+    xd = dev(x)
+    y = model.evaluate_dataset_batch(xd)
+    block = model.layers[1]
+    assert [l.canonical_name for l in block.paths[0]] == ["Conv2DBatchNormalization"]
+    assert block._folded_sum_path() == 0 and block.relu_above is model.layers[2]
+    assert np.array_equal(host(xd), x), "the block must not write into its input"
+    model._fused = False
+    try:
+        y_separate = model.evaluate_batch(xd)
+    finally:
+        model._fused = True
+    assert torch.equal(y, y_separate)
+    p = oracle.ConvParams(3, 3, 1, 1)
+    fwd = oracle.conv2d_forward_nchw_i2c if fmt == "NCHW" else oracle.conv2d_forward_nhwc_i2c
+    cur, _ = fwd(x, w_h, b_h, p)
+    cur = oracle.fused_epilogue(cur, fmt, bn=bn_h, relu_flag=False)
+    ref, _ = oracle.relu(oracle.eltw_sum(np.ascontiguousarray(cur), x))
+    assert_close(host(y), ref, what="one-convolution block vs oracle")
+
+
 # ------------------------------------------------------------------ a small VGG-style training step
 
 @pytest.mark.parametrize("folding", [False, True], ids=["plain", "relu_folding"])
